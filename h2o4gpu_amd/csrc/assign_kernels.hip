@@ -1,0 +1,637 @@
+// Fused distance + argmin ("assign") and full distance ("transform") kernels.
+//
+// Replaces, in one pass over the data and without an n x k buffer, the
+// reference sequence make_self_dots(C) -> all_dots -> matmul|cublas gemm ->
+// absolute_value -> make_new_labels
+// (src/gpu/kmeans/kmeans_labels.cu:183-244, kmeans_labels.h:187-244,360-392).
+// Kept from the reference: dist = |(xx + cc) - 2 x.c| with xx + cc rounded
+// first, strict '<' argmin, lowest index on ties, start value FLT_MAX, label -1
+// when nothing is below it.
+#include "kmeans_common.h"
+#include "mfma_traits.h"
+
+namespace kmhip {
+
+static constexpr int WG = 256;  // threads per workgroup (4 wavefronts)
+
+// ---------------------------------------------------------------------------
+// VALU variant: one thread per row, a chunk of centroids broadcast from LDS.
+// Arithmetic order is j ascending with separate multiply and add, so this
+// kernel reproduces a scalar CPU loop bit for bit. It carries the small shapes
+// (the reference's own k <= 16 && d <= 64 path) and is the any-shape fallback.
+// MODE 0: labels (+ optional mindist).  MODE 1: full distances D[c*ldn + i].
+// ---------------------------------------------------------------------------
+template <typename T, int DREG, int MODE>
+__global__ __launch_bounds__(WG) void assign_valu_kernel(
+    const T *__restrict__ X, const T *__restrict__ xnorm,
+    const T *__restrict__ C, const T *__restrict__ cnorm,
+    int *__restrict__ labels, T *__restrict__ mindist, T *__restrict__ D,
+    int64_t n, int64_t ldn, int d, int k, int kc) {
+#pragma clang fp contract(off)
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  T *Cs = reinterpret_cast<T *>(smem_raw);  // [kc][d]
+  T *ccs = Cs + (size_t)kc * d;             // [kc]
+  const int tid = threadIdx.x;
+  const int64_t row = (int64_t)blockIdx.x * WG + tid;
+  const bool valid = row < n;
+  const T *x = X + (valid ? row : 0) * (int64_t)d;
+  T xr[DREG > 0 ? DREG : 1];
+  if (DREG > 0) {
+#pragma unroll
+    for (int j = 0; j < DREG; j++) xr[j] = (valid && j < d) ? x[j] : (T)0;
+  }
+  const T xx = valid ? xnorm[row] : (T)0;
+  T best = argmin_start<T>();
+  int bidx = -1;
+  for (int c0 = 0; c0 < k; c0 += kc) {
+    const int nc = min(kc, k - c0);
+    __syncthreads();
+    for (int e = tid; e < nc * d; e += WG) Cs[e] = C[(size_t)c0 * d + e];
+    for (int c = tid; c < nc; c += WG) ccs[c] = cnorm[c0 + c];
+    __syncthreads();
+    if (!valid) continue;
+    for (int c = 0; c < nc; c++) {
+      const T *cp = Cs + (size_t)c * d;
+      T dot = 0;
+      if (DREG > 0) {
+#pragma unroll
+        for (int j = 0; j < DREG; j++)
+          if (j < d) dot = dot + xr[j] * cp[j];
+      } else {
+        for (int j = 0; j < d; j++) dot = dot + x[j] * cp[j];
+      }
+      T t = xx + ccs[c];
+      T dist = fabs(t - (T)2 * dot);
+      if (MODE == 1) {
+        D[(size_t)(c0 + c) * ldn + row] = dist;
+      } else if (dist < best) {
+        best = dist;
+        bidx = c0 + c;
+      }
+    }
+  }
+  if (MODE == 0 && valid) {
+    labels[row] = bidx;
+    if (mindist) mindist[row] = best;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// MFMA row-stationary variant (d <= DP, all centroids resident in LDS).
+//
+// A workgroup is persistent: it stages -2*C once into LDS, already permuted
+// into A-operand order so that every later read is one conflict-free 16-byte
+// load per lane, then walks over row tiles. Each wavefront keeps ROWT tiles of
+// MT data rows in registers (plain 16-byte global loads, never through LDS)
+// and sweeps all centroid tiles over them: accumulators start at xx + cc, the
+// matrix core adds -2 x.c, and the epilogue folds |acc| into a per-lane running
+// (min, index). Lane groups holding different centroid subsets of the same row
+// are merged with one (f32) or two (f64) cross-lane exchanges per row tile.
+// ---------------------------------------------------------------------------
+template <typename T, int DP, int ROWT, bool VECLOAD>
+__global__ __launch_bounds__(WG) void assign_rowstat_kernel(
+    const T *__restrict__ X, const T *__restrict__ xnorm,
+    const T *__restrict__ C, const T *__restrict__ cnorm,
+    int *__restrict__ labels, T *__restrict__ mindist, int64_t n, int d, int k,
+    int kp) {
+  typedef Mfma<T> M;
+  constexpr int MT = M::MT, KL = M::KL, NACC = M::NACC, VW = M::VW;
+  constexpr int DCH = DP / KL;  // features per lane group
+  constexpr int NV = DCH / VW;  // 16-byte vectors per lane per tile
+  static_assert(DCH % VW == 0, "DP must be a multiple of KL*VW");
+  typedef typename M::acc_t acc_t;
+  typedef typename M::vec_t vec_t;
+
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  T *Cs = reinterpret_cast<T *>(smem_raw);  // [KT][NV][64][VW]
+  T *ccs = Cs + (size_t)kp * DP;            // [kp]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int r = lane % MT;
+  const int g = lane / MT;
+  const int KT = kp / MT;
+
+  for (int e = tid; e < kp * DP; e += WG) {
+    const int c = e / DP, j = e - c * DP;
+    const T v = (c < k && j < d) ? (T)-2 * C[(size_t)c * d + j] : (T)0;
+    const int t = c / MT, i = c - t * MT, gg = j / DCH, s = j - gg * DCH;
+    Cs[((size_t)(t * NV + s / VW) * 64 + gg * MT + i) * VW + (s % VW)] = v;
+  }
+  for (int c = tid; c < kp; c += WG) ccs[c] = c < k ? cnorm[c] : pos_inf<T>();
+  __syncthreads();
+
+  constexpr int ROWS_PER_WAVE = ROWT * MT;
+  constexpr int ROWS_PER_WG = (WG / 64) * ROWS_PER_WAVE;
+  for (int64_t base = (int64_t)blockIdx.x * ROWS_PER_WG; base < n;
+       base += (int64_t)gridDim.x * ROWS_PER_WG) {
+    const int64_t wrow0 = base + (int64_t)wave * ROWS_PER_WAVE;
+    T x[ROWT][DCH];
+    T xx[ROWT];
+#pragma unroll
+    for (int rt = 0; rt < ROWT; rt++) {
+      const int64_t row = wrow0 + rt * MT + r;
+      const bool valid = row < n;
+      if (VECLOAD) {
+        const vec_t *src = reinterpret_cast<const vec_t *>(
+            X + (valid ? row : 0) * (int64_t)DP + g * DCH);
+#pragma unroll
+        for (int q = 0; q < NV; q++) {
+          vec_t v = src[q];
+#pragma unroll
+          for (int e = 0; e < VW; e++) x[rt][q * VW + e] = valid ? v[e] : (T)0;
+        }
+      } else {
+        const T *src = X + (valid ? row : 0) * (int64_t)d;
+#pragma unroll
+        for (int s = 0; s < DCH; s++) {
+          const int j = g * DCH + s;
+          x[rt][s] = (valid && j < d) ? src[j] : (T)0;
+        }
+      }
+      xx[rt] = valid ? xnorm[row] : (T)0;
+    }
+    T best[ROWT];
+    int bidx[ROWT];
+#pragma unroll
+    for (int rt = 0; rt < ROWT; rt++) {
+      best[rt] = argmin_start<T>();
+      bidx[rt] = -1;
+    }
+    for (int t = 0; t < KT; t++) {
+      acc_t acc[ROWT];
+#pragma unroll
+      for (int v = 0; v < NACC; v++) {
+        const T cc = ccs[t * MT + M::acc_row(v, g)];
+#pragma unroll
+        for (int rt = 0; rt < ROWT; rt++) acc[rt][v] = xx[rt] + cc;
+      }
+      const vec_t *ap = reinterpret_cast<const vec_t *>(Cs) + (size_t)t * NV * 64 + lane;
+#pragma unroll
+      for (int q = 0; q < NV; q++) {
+        const vec_t a = ap[q * 64];
+#pragma unroll
+        for (int e = 0; e < VW; e++) {
+#pragma unroll
+          for (int rt = 0; rt < ROWT; rt++)
+            acc[rt] = M::mma(a[e], x[rt][q * VW + e], acc[rt]);
+        }
+      }
+#pragma unroll
+      for (int v = 0; v < NACC; v++) {
+        const int cidx = t * MT + M::acc_row(v, g);
+#pragma unroll
+        for (int rt = 0; rt < ROWT; rt++) {
+          const T dist = fabs(acc[rt][v]);
+          if (dist < best[rt]) {
+            best[rt] = dist;
+            bidx[rt] = cidx;
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int rt = 0; rt < ROWT; rt++) {
+#pragma unroll
+      for (int off = MT; off < 64; off <<= 1) {
+        const T ob = __shfl_xor(best[rt], off, 64);
+        const int oi = __shfl_xor(bidx[rt], off, 64);
+        argmin_merge(best[rt], bidx[rt], ob, oi);
+      }
+      const int64_t row = wrow0 + rt * MT + r;
+      if (g == 0 && row < n) {
+        labels[row] = bidx[rt];
+        if (mindist) mindist[row] = best[rt];
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// MFMA tiled variant (any d, any k). A workgroup owns BR = 128 data rows and
+// walks over centroid blocks of BC = 128; for each block it runs the d-loop in
+// steps of BK features with both operand tiles staged through LDS in operand
+// order (double buffered). The four wavefronts split the block 2 x 2, each
+// holding (BC/2/MT) x (BR/2/MT) result tiles in accumulators.
+// MODE 0: running argmin kept in registers across centroid blocks, halves
+// merged through LDS at the end.  MODE 1: |acc| stored to D[c*ldn + i].
+// ---------------------------------------------------------------------------
+template <typename T>
+struct TiledCfg {
+  static constexpr int BC = 128;
+  static constexpr int BR = 128;
+  static constexpr int BK = sizeof(T) == 4 ? 32 : 16;
+};
+
+template <typename T, int MODE, bool VECLOAD>
+__global__ __launch_bounds__(WG) void assign_tiled_kernel(
+    const T *__restrict__ X, const T *__restrict__ xnorm,
+    const T *__restrict__ C, const T *__restrict__ cnorm,
+    int *__restrict__ labels, T *__restrict__ mindist, T *__restrict__ D,
+    int64_t n, int64_t ldn, int d, int k) {
+  typedef Mfma<T> M;
+  typedef TiledCfg<T> Cfg;
+  constexpr int MT = M::MT, KL = M::KL, NACC = M::NACC, VW = M::VW;
+  constexpr int BC = Cfg::BC, BR = Cfg::BR, BK = Cfg::BK;
+  constexpr int DCH = BK / KL;       // features per lane group per stage
+  constexpr int NV = DCH / VW;       // 16-byte vectors per lane per tile per stage
+  constexpr int CT = BC / 2 / MT;    // centroid tiles per wavefront
+  constexpr int RT = BR / 2 / MT;    // row tiles per wavefront
+  constexpr int TILE_ELEMS = MT * BK;               // one operand tile, one stage
+  constexpr int A_ELEMS = (BC / MT) * TILE_ELEMS;   // = BC*BK
+  constexpr int B_ELEMS = (BR / MT) * TILE_ELEMS;
+  constexpr int VEC_PER_ROW = BK / VW;              // 16-byte vectors per operand row per stage
+  constexpr int A_VECS = BC * VEC_PER_ROW / WG;     // vectors each thread stages for A
+  constexpr int B_VECS = BR * VEC_PER_ROW / WG;
+  typedef typename M::acc_t acc_t;
+  typedef typename M::vec_t vec_t;
+
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  T *As = reinterpret_cast<T *>(smem_raw);  // [2][A_ELEMS]
+  T *Bs = As + 2 * A_ELEMS;                 // [2][B_ELEMS]
+  // after the main loop the same memory is reused for the cross-wave merge
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wc = wave & 1;   // which half of the centroid block
+  const int wr = wave >> 1;  // which half of the row block
+  const int r = lane % MT;
+  const int g = lane / MT;
+  const int64_t row0 = (int64_t)blockIdx.x * BR;
+  const int nstage = (d + BK - 1) / BK;
+
+  // element (row rr of the operand block, features [j0, j0+VW)) goes to
+  // tile rr/MT, lane group (jj/DCH), slot s = jj%DCH as one 16-byte store.
+  auto lds_slot = [&](int rr, int jj) -> int {
+    const int t = rr / MT, i = rr - t * MT, gg = jj / DCH, s = jj - gg * DCH;
+    return ((t * NV + s / VW) * 64 + gg * MT + i) * VW;
+  };
+
+  T xx[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; rt++) {
+    const int64_t row = row0 + (wr * RT + rt) * MT + r;
+    xx[rt] = row < n ? xnorm[row] : (T)0;
+  }
+  T best[RT];
+  int bidx[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; rt++) {
+    best[rt] = argmin_start<T>();
+    bidx[rt] = -1;
+  }
+
+  vec_t areg[A_VECS], breg[B_VECS];
+  auto gload = [&](int c0, int st) {
+    const int j0 = st * BK;
+#pragma unroll
+    for (int q = 0; q < A_VECS; q++) {
+      const int vi = tid + q * WG;
+      const int rr = vi / VEC_PER_ROW, jj = (vi - rr * VEC_PER_ROW) * VW;
+      const int c = c0 + rr, j = j0 + jj;
+      vec_t v;
+      if (VECLOAD) {
+        if (c < k && j < d)
+          v = *reinterpret_cast<const vec_t *>(C + (size_t)c * d + j);
+        else
+#pragma unroll
+          for (int e = 0; e < VW; e++) v[e] = 0;
+      } else {
+#pragma unroll
+        for (int e = 0; e < VW; e++)
+          v[e] = (c < k && j + e < d) ? C[(size_t)c * d + j + e] : (T)0;
+      }
+      areg[q] = v * (T)-2;
+    }
+#pragma unroll
+    for (int q = 0; q < B_VECS; q++) {
+      const int vi = tid + q * WG;
+      const int rr = vi / VEC_PER_ROW, jj = (vi - rr * VEC_PER_ROW) * VW;
+      const int64_t row = row0 + rr;
+      const int j = j0 + jj;
+      vec_t v;
+      if (VECLOAD) {
+        if (row < n && j < d)
+          v = *reinterpret_cast<const vec_t *>(X + row * (int64_t)d + j);
+        else
+#pragma unroll
+          for (int e = 0; e < VW; e++) v[e] = 0;
+      } else {
+#pragma unroll
+        for (int e = 0; e < VW; e++)
+          v[e] = (row < n && j + e < d) ? X[row * (int64_t)d + j + e] : (T)0;
+      }
+      breg[q] = v;
+    }
+  };
+  auto lstore = [&](int buf) {
+#pragma unroll
+    for (int q = 0; q < A_VECS; q++) {
+      const int vi = tid + q * WG;
+      const int rr = vi / VEC_PER_ROW, jj = (vi - rr * VEC_PER_ROW) * VW;
+      *reinterpret_cast<vec_t *>(As + buf * A_ELEMS + lds_slot(rr, jj)) = areg[q];
+    }
+#pragma unroll
+    for (int q = 0; q < B_VECS; q++) {
+      const int vi = tid + q * WG;
+      const int rr = vi / VEC_PER_ROW, jj = (vi - rr * VEC_PER_ROW) * VW;
+      *reinterpret_cast<vec_t *>(Bs + buf * B_ELEMS + lds_slot(rr, jj)) = breg[q];
+    }
+  };
+
+  for (int c0 = 0; c0 < k; c0 += BC) {
+    acc_t acc[CT][RT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ct++) {
+#pragma unroll
+      for (int v = 0; v < NACC; v++) {
+        const int c = c0 + (wc * CT + ct) * MT + M::acc_row(v, g);
+        const T cc = c < k ? cnorm[c] : pos_inf<T>();
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) acc[ct][rt][v] = xx[rt] + cc;
+      }
+    }
+    gload(c0, 0);
+    __syncthreads();  // previous block's readers are done with buffer 0
+    lstore(0);
+    __syncthreads();
+    for (int st = 0; st < nstage; st++) {
+      const int buf = st & 1;
+      if (st + 1 < nstage) gload(c0, st + 1);
+      const vec_t *ap = reinterpret_cast<const vec_t *>(As + buf * A_ELEMS) + lane;
+      const vec_t *bp = reinterpret_cast<const vec_t *>(Bs + buf * B_ELEMS) + lane;
+#pragma unroll
+      for (int q = 0; q < NV; q++) {
+        vec_t a[CT], b[RT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ct++) a[ct] = ap[((wc * CT + ct) * NV + q) * 64];
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) b[rt] = bp[((wr * RT + rt) * NV + q) * 64];
+#pragma unroll
+        for (int e = 0; e < VW; e++) {
+#pragma unroll
+          for (int ct = 0; ct < CT; ct++) {
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++)
+              acc[ct][rt] = M::mma(a[ct][e], b[rt][e], acc[ct][rt]);
+          }
+        }
+      }
+      if (st + 1 < nstage) {
+        lstore(buf ^ 1);  // the other buffer was last read one stage ago
+        __syncthreads();
+      }
+    }
+    // epilogue for this centroid block
+#pragma unroll
+    for (int ct = 0; ct < CT; ct++) {
+#pragma unroll
+      for (int v = 0; v < NACC; v++) {
+        const int c = c0 + (wc * CT + ct) * MT + M::acc_row(v, g);
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) {
+          const T dist = fabs(acc[ct][rt][v]);
+          if (MODE == 1) {
+            const int64_t row = row0 + (wr * RT + rt) * MT + r;
+            if (c < k && row < n) D[(size_t)c * ldn + row] = dist;
+          } else if (dist < best[rt]) {
+            best[rt] = dist;
+            bidx[rt] = c;
+          }
+        }
+      }
+    }
+  }
+  if (MODE == 0) {
+    // lane groups of one wavefront, then the two wavefronts sharing the rows
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++) {
+#pragma unroll
+      for (int off = MT; off < 64; off <<= 1) {
+        const T ob = __shfl_xor(best[rt], off, 64);
+        const int oi = __shfl_xor(bidx[rt], off, 64);
+        argmin_merge(best[rt], bidx[rt], ob, oi);
+      }
+    }
+    __syncthreads();  // all waves are past their last LDS operand read
+    T *mb = reinterpret_cast<T *>(smem_raw);           // [BR]
+    int *mi = reinterpret_cast<int *>(mb + BR);        // [BR]
+    if (wc == 1 && g == 0) {
+#pragma unroll
+      for (int rt = 0; rt < RT; rt++) {
+        const int lr = (wr * RT + rt) * MT + r;
+        mb[lr] = best[rt];
+        mi[lr] = bidx[rt];
+      }
+    }
+    __syncthreads();
+    if (wc == 0 && g == 0) {
+#pragma unroll
+      for (int rt = 0; rt < RT; rt++) {
+        const int lr = (wr * RT + rt) * MT + r;
+        argmin_merge(best[rt], bidx[rt], mb[lr], mi[lr]);
+        const int64_t row = row0 + lr;
+        if (row < n) {
+          labels[row] = bidx[rt];
+          if (mindist) mindist[row] = best[rt];
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+const char *assign_variant_name(int variant) {
+  switch (variant) {
+    case ASSIGN_VALU: return "valu";
+    case ASSIGN_ROWSTAT: return "mfma_rowstat";
+    case ASSIGN_TILED: return "mfma_tiled";
+    default: return "auto";
+  }
+}
+
+static const size_t LDS_LIMIT = 160 * 1024;
+
+template <typename T>
+static int rowstat_dp(int d) {
+  const int maxdp = sizeof(T) == 4 ? 128 : 64;
+  for (int dp = 16; dp <= maxdp; dp *= 2)
+    if (d <= dp) return dp;
+  return 0;
+}
+template <typename T>
+static size_t rowstat_lds(int d, int k) {
+  const int MT = Mfma<T>::MT;
+  const int kp = (k + MT - 1) / MT * MT;
+  return ((size_t)kp * rowstat_dp<T>(d) + kp) * sizeof(T);
+}
+
+template <typename T>
+int pick_assign_variant(int requested, int64_t n, int d, int k) {
+  const bool rowstat_ok = rowstat_dp<T>(d) != 0 && rowstat_lds<T>(d, k) <= 96 * 1024;
+  if (requested == ASSIGN_ROWSTAT) return rowstat_ok ? ASSIGN_ROWSTAT : -1;
+  if (requested == ASSIGN_VALU || requested == ASSIGN_TILED) return requested;
+  // the reference switches to its hand-written small kernel at k<=16 && d<=64
+  // (kmeans_labels.cu:140,207); same boundary here
+  if (k <= 16 && d <= 64) return ASSIGN_VALU;
+  if (rowstat_ok) return ASSIGN_ROWSTAT;
+  return ASSIGN_TILED;
+}
+
+template <typename T, int MODE>
+static int launch_valu(hipStream_t s, const T *X, const T *xnorm, const T *C,
+                       const T *cnorm, int *labels, T *mindist, T *D, int64_t n,
+                       int64_t ldn, int d, int k) {
+  // centroid chunk: as many whole centroids as fit in 48 KB
+  int kc = (int)((48 * 1024) / ((size_t)(d + 1) * sizeof(T)));
+  if (kc < 1) return H2O4GPU_KMEANS_EARG;  // d beyond 12K features
+  if (kc > k) kc = k;
+  const size_t lds = (size_t)kc * (d + 1) * sizeof(T);
+  const dim3 grid((unsigned)((n + WG - 1) / WG));
+#define KM_VALU(DREG)                                                          \
+  hipLaunchKernelGGL((assign_valu_kernel<T, DREG, MODE>), grid, dim3(WG), lds, \
+                     s, X, xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k, kc)
+  if (d <= 16) KM_VALU(16);
+  else if (d <= 32) KM_VALU(32);
+  else if (d <= 64) KM_VALU(64);
+  else KM_VALU(0);
+#undef KM_VALU
+  KM_HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+template <typename T, int DP, int ROWT>
+static int launch_rowstat_dp(hipStream_t s, const T *X, const T *xnorm,
+                             const T *C, const T *cnorm, int *labels,
+                             T *mindist, int64_t n, int d, int k, int num_cu) {
+  const int MT = Mfma<T>::MT;
+  const int kp = (k + MT - 1) / MT * MT;
+  const size_t lds = ((size_t)kp * DP + kp) * sizeof(T);
+  const int rows_per_wg = (WG / 64) * ROWT * MT;
+  const int64_t tiles = (n + rows_per_wg - 1) / rows_per_wg;
+  const int wg_per_cu = lds <= 72 * 1024 ? 2 : 1;
+  int64_t grid = (int64_t)num_cu * wg_per_cu;
+  if (grid > tiles) grid = tiles;
+  if (grid < 1) grid = 1;
+  const bool vec = (d == DP) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0);
+  if (vec) {
+    auto kern = assign_rowstat_kernel<T, DP, ROWT, true>;
+    if (lds > 64 * 1024)
+      KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(WG), lds, s, X, xnorm, C,
+                       cnorm, labels, mindist, n, d, k, kp);
+  } else {
+    auto kern = assign_rowstat_kernel<T, DP, ROWT, false>;
+    if (lds > 64 * 1024)
+      KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(WG), lds, s, X, xnorm, C,
+                       cnorm, labels, mindist, n, d, k, kp);
+  }
+  KM_HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+template <typename T>
+struct RowstatDispatch;
+template <>
+struct RowstatDispatch<float> {
+  static int run(hipStream_t s, const float *X, const float *xnorm, const float *C,
+                 const float *cnorm, int *labels, float *mindist, int64_t n, int d,
+                 int k, int num_cu) {
+    switch (rowstat_dp<float>(d)) {
+      case 16: return launch_rowstat_dp<float, 16, 2>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu);
+      case 32: return launch_rowstat_dp<float, 32, 2>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu);
+      case 64: return launch_rowstat_dp<float, 64, 2>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu);
+      case 128: return launch_rowstat_dp<float, 128, 1>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu);
+    }
+    return H2O4GPU_KMEANS_EARG;
+  }
+};
+template <>
+struct RowstatDispatch<double> {
+  static int run(hipStream_t s, const double *X, const double *xnorm, const double *C,
+                 const double *cnorm, int *labels, double *mindist, int64_t n, int d,
+                 int k, int num_cu) {
+    switch (rowstat_dp<double>(d)) {
+      case 16: return launch_rowstat_dp<double, 16, 4>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu);
+      case 32: return launch_rowstat_dp<double, 32, 4>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu);
+      case 64: return launch_rowstat_dp<double, 64, 2>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu);
+    }
+    return H2O4GPU_KMEANS_EARG;
+  }
+};
+
+template <typename T, int MODE>
+static int launch_tiled(hipStream_t s, const T *X, const T *xnorm, const T *C,
+                        const T *cnorm, int *labels, T *mindist, T *D, int64_t n,
+                        int64_t ldn, int d, int k) {
+  typedef TiledCfg<T> Cfg;
+  const size_t lds = (size_t)2 * (Cfg::BC + Cfg::BR) * Cfg::BK * sizeof(T);
+  const dim3 grid((unsigned)((n + Cfg::BR - 1) / Cfg::BR));
+  const int vw = Mfma<T>::VW;
+  const bool vec = (d % vw == 0) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0) &&
+                   ((reinterpret_cast<uintptr_t>(C) & 15) == 0);
+  if (vec)
+    hipLaunchKernelGGL((assign_tiled_kernel<T, MODE, true>), grid, dim3(WG), lds, s,
+                       X, xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k);
+  else
+    hipLaunchKernelGGL((assign_tiled_kernel<T, MODE, false>), grid, dim3(WG), lds, s,
+                       X, xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k);
+  KM_HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+template <typename T>
+int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
+                  const T *C, const T *cnorm, int *labels, T *mindist, int64_t n,
+                  int d, int k, int num_cu, int *used) {
+  if (n <= 0) return 0;
+  if (d < 1 || k < 1) return H2O4GPU_KMEANS_EARG;
+  const int v = pick_assign_variant<T>(variant, n, d, k);
+  if (v < 0) return H2O4GPU_KMEANS_EARG;
+  if (used) *used = v;
+  switch (v) {
+    case ASSIGN_VALU:
+      return launch_valu<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k);
+    case ASSIGN_ROWSTAT:
+      return RowstatDispatch<T>::run(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu);
+    case ASSIGN_TILED:
+      return launch_tiled<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k);
+  }
+  return H2O4GPU_KMEANS_EARG;
+}
+
+template <typename T>
+int launch_transform(hipStream_t s, const T *X, const T *xnorm, const T *C,
+                     const T *cnorm, T *D, int64_t n, int64_t ldn, int d, int k,
+                     int num_cu) {
+  (void)num_cu;
+  if (n <= 0) return 0;
+  if (d < 1 || k < 1) return H2O4GPU_KMEANS_EARG;
+  if (k <= 16 && d <= 64)
+    return launch_valu<T, 1>(s, X, xnorm, C, cnorm, nullptr, nullptr, D, n, ldn, d, k);
+  return launch_tiled<T, 1>(s, X, xnorm, C, cnorm, nullptr, nullptr, D, n, ldn, d, k);
+}
+
+template int pick_assign_variant<float>(int, int64_t, int, int);
+template int pick_assign_variant<double>(int, int64_t, int, int);
+template int launch_assign<float>(hipStream_t, int, const float *, const float *,
+                                  const float *, const float *, int *, float *,
+                                  int64_t, int, int, int, int *);
+template int launch_assign<double>(hipStream_t, int, const double *, const double *,
+                                   const double *, const double *, int *, double *,
+                                   int64_t, int, int, int, int *);
+template int launch_transform<float>(hipStream_t, const float *, const float *,
+                                     const float *, const float *, float *, int64_t,
+                                     int64_t, int, int, int);
+template int launch_transform<double>(hipStream_t, const double *, const double *,
+                                      const double *, const double *, double *,
+                                      int64_t, int64_t, int, int, int);
+
+}  // namespace kmhip

@@ -1,0 +1,1012 @@
+// Host side of the gfx950 k-means engine: the resident-data handle, the Lloyd
+// loop, seeding, and the C entry points h2o4gpu's bindings call.
+//
+// Replaces src/gpu/kmeans/kmeans_h2o4gpu.cu (kmeans_fit :617-815,
+// kmeans_predict :817-889, kmeans_transform :891-975, kmeans_init :572-607, the
+// exported symbols :1060-1097) and the loop of src/gpu/kmeans/kmeans_impl.h
+// :109-232. One device, one stream, no global state: calls on different handles
+// are independent.
+#include <algorithm>
+#include <atomic>
+#include <csignal>
+#include <cstdarg>
+#include <cstdlib>
+#include <cstring>
+#include <ctime>
+#include <map>
+#include <numeric>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "kmeans_common.h"
+
+namespace kmhip {
+
+// ---------------------------------------------------------------------------
+// logging (format of src/common/logger.cpp:16-33)
+// ---------------------------------------------------------------------------
+void log_msg(int verbose, int level, const char *fmt, ...) {
+  if (!(verbose > LOG_NOTHING && level <= verbose)) return;
+  static const char *names[] = {"NOTHING", "FATAL", "ERROR", "INFO",
+                                "WARN",    "DEBUG", "VERBOSE"};
+  time_t now = time(nullptr);
+  struct tm tmv;
+  localtime_r(&now, &tmv);
+  char buf[16];
+  buf[strftime(buf, sizeof(buf), "%H:%M:%S", &tmv)] = '\0';
+  fprintf(stderr, "%s %-5s kmeans_hip: ", buf, names[(level / 100) % 7]);
+  va_list args;
+  va_start(args, fmt);
+  vfprintf(stderr, fmt, args);
+  va_end(args);
+  fprintf(stderr, "\n");
+}
+
+// Set by SIGINT/SIGTERM when the handlers are installed; the loop then finishes
+// the current iteration, relabels once and returns normally
+// (kmeans_h2o4gpu.cu:565-570, kmeans_impl.h:114,210-215). The reference
+// installs the handlers on every call and never restores them; here they are
+// installed only when H2O4GPU_KMEANS_SIGNALS=1 is set in the environment.
+static volatile std::sig_atomic_t g_stop_flag = 0;
+static void on_signal(int sig) {
+  (void)sig;
+  g_stop_flag = 1;
+}
+static void maybe_install_signal_handlers() {
+  const char *e = getenv("H2O4GPU_KMEANS_SIGNALS");
+  if (e && e[0] == '1') {
+    std::signal(SIGINT, on_signal);
+    std::signal(SIGTERM, on_signal);
+  }
+}
+
+static int visible_devices() {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return n;
+}
+
+}  // namespace kmhip
+
+using namespace kmhip;
+
+// ---------------------------------------------------------------------------
+// the handle
+// ---------------------------------------------------------------------------
+struct h2o4gpu_kmeans_handle {
+  int elem_size = 0;
+  int64_t n = 0;
+  int d = 0;
+  int k = 0;
+  int dev = 0;
+  int verbose = 0;
+  int num_cu = 0;
+  hipStream_t stream = nullptr;
+  int opt_assign = ASSIGN_AUTO;
+  int last_variant = ASSIGN_AUTO;
+
+  // profiling
+  bool prof_on = false;
+  struct Pending {
+    std::string name;
+    hipEvent_t a, b;
+  };
+  std::vector<Pending> pending;
+  std::vector<hipEvent_t> pool;
+  std::map<std::string, std::pair<int, double>> prof;
+  hipEvent_t t0 = nullptr, t1 = nullptr;
+
+  virtual ~h2o4gpu_kmeans_handle() {}
+  virtual int set_data_host(const void *X) = 0;
+  virtual int set_data_device(const void *dX) = 0;
+  virtual int set_centroids_host(const void *C) = 0;
+  virtual int init_random_rows(int seed) = 0;
+  virtual int init_plusplus(int seed) = 0;
+  virtual int fit(int max_iterations, double threshold, int *iters) = 0;
+  virtual int assign() = 0;
+  virtual int update(double *shift2) = 0;
+  virtual int set_labels_host(const int *labels) = 0;
+  virtual int get_centroids(void *C) = 0;
+  virtual int get_labels(int *labels) = 0;
+  virtual int get_counts(int *counts) = 0;
+  virtual int get_min_distances(void *m) = 0;
+  virtual int inertia(double *out) = 0;
+  virtual int predict_host(size_t rows, const void *X, int *labels) = 0;
+  virtual int transform_host(size_t rows, const void *X, void *dist) = 0;
+  virtual int transform_resident(void *d_dist) = 0;
+  virtual int release() = 0;
+
+  hipEvent_t get_event() {
+    if (!pool.empty()) {
+      hipEvent_t e = pool.back();
+      pool.pop_back();
+      return e;
+    }
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) return nullptr;
+    return e;
+  }
+  void prof_begin(const char *name) {
+    if (!prof_on) return;
+    Pending p;
+    p.name = name;
+    p.a = get_event();
+    p.b = get_event();
+    if (p.a) (void)hipEventRecord(p.a, stream);
+    pending.push_back(p);
+  }
+  void prof_end() {
+    if (!prof_on || pending.empty()) return;
+    if (pending.back().b) (void)hipEventRecord(pending.back().b, stream);
+  }
+  int prof_resolve() {
+    if (pending.empty()) return 0;
+    KM_HIP_TRY(hipStreamSynchronize(stream));
+    for (auto &p : pending) {
+      float ms = 0;
+      if (p.a && p.b && hipEventElapsedTime(&ms, p.a, p.b) == hipSuccess) {
+        auto &acc = prof[p.name];
+        acc.first += 1;
+        acc.second += ms;
+      }
+      if (p.a) pool.push_back(p.a);
+      if (p.b) pool.push_back(p.b);
+    }
+    pending.clear();
+    return 0;
+  }
+  void prof_free() {
+    for (auto &p : pending) {
+      if (p.a) (void)hipEventDestroy(p.a);
+      if (p.b) (void)hipEventDestroy(p.b);
+    }
+    pending.clear();
+    for (auto e : pool) (void)hipEventDestroy(e);
+    pool.clear();
+    if (t0) (void)hipEventDestroy(t0);
+    if (t1) (void)hipEventDestroy(t1);
+    t0 = t1 = nullptr;
+  }
+};
+
+namespace kmhip {
+
+#define PROFILED(name, call)   \
+  do {                         \
+    prof_begin(name);          \
+    int _prc = (call);         \
+    prof_end();                \
+    if (_prc != 0) return _prc; \
+  } while (0)
+
+template <typename T>
+struct Engine : h2o4gpu_kmeans_handle {
+  T *X = nullptr;
+  bool own_X = false;
+  T *xnorm = nullptr;
+  T *C[2] = {nullptr, nullptr};
+  int cur = 0;
+  T *cnorm = nullptr;
+  int *labels = nullptr;
+  T *mindist = nullptr;
+  int *counts = nullptr;
+  UpdatePlan plan;
+  T *psums = nullptr;
+  int *pcounts = nullptr;
+  T *shift_partials = nullptr;
+  T *shift2 = nullptr;
+  double *sum_partials = nullptr;  // [sum_partials_needed() + 1]
+  double *kpp_bsums = nullptr;
+  bool have_data = false, have_centroids = false, have_mindist = false;
+
+  template <typename U>
+  int dalloc(U **p, size_t count) {
+    *p = nullptr;
+    if (count == 0) count = 1;
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(p), count * sizeof(U));
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      log_msg(verbose ? verbose : LOG_ERROR, LOG_ERROR,
+              "device allocation of %zu bytes failed: %s", count * sizeof(U),
+              hipGetErrorString(e));
+      return H2O4GPU_KMEANS_EALLOC;
+    }
+    return 0;
+  }
+
+  int create() {
+    KM_HIP_TRY(hipSetDevice(dev));
+    hipDeviceProp_t prop;
+    KM_HIP_TRY(hipGetDeviceProperties(&prop, dev));
+    num_cu = prop.multiProcessorCount;
+    KM_HIP_TRY(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
+    plan = plan_update<T>(n, d, k, num_cu);
+    const size_t kd = (size_t)k * d;
+    KM_TRY(dalloc(&C[0], kd));
+    KM_TRY(dalloc(&C[1], kd));
+    KM_TRY(dalloc(&cnorm, k));
+    KM_TRY(dalloc(&counts, k));
+    KM_TRY(dalloc(&labels, n));
+    KM_TRY(dalloc(&xnorm, n));
+    KM_TRY(dalloc(&mindist, n));
+    KM_TRY(dalloc(&psums, (size_t)plan.row_blocks * kd));
+    KM_TRY(dalloc(&pcounts, (size_t)plan.row_blocks * k));
+    KM_TRY(dalloc(&shift_partials, (kd + 255) / 256 + 1));
+    KM_TRY(dalloc(&shift2, 1));
+    KM_TRY(dalloc(&sum_partials, sum_partials_needed() + 1));
+    KM_TRY(dalloc(&kpp_bsums, (n + KPP_BLOCK - 1) / KPP_BLOCK + 1));
+    // the reference's label vector starts zeroed (thrust::device_vector<int>)
+    KM_HIP_TRY(hipMemsetAsync(labels, 0, (size_t)n * sizeof(int), stream));
+    KM_HIP_TRY(hipMemsetAsync(counts, 0, (size_t)k * sizeof(int), stream));
+    KM_HIP_TRY(hipStreamSynchronize(stream));
+    log_msg(verbose, LOG_DEBUG,
+            "handle: rows=%lld cols=%d k=%d elem=%d device=%d CUs=%d update plan: "
+            "row_blocks=%d kc=%d k_chunks=%d vec=%d",
+            (long long)n, d, k, (int)sizeof(T), dev, num_cu, plan.row_blocks, plan.kc,
+            plan.k_chunks, plan.vec);
+    return 0;
+  }
+
+  int release() override {
+    (void)hipSetDevice(dev);
+    if (stream) (void)hipStreamSynchronize(stream);
+    prof_free();
+    if (own_X && X) (void)hipFree(X);
+    void *ptrs[] = {xnorm,  C[0],    C[1],           cnorm,  labels,       mindist,
+                    counts, psums,   pcounts,        shift_partials, shift2,
+                    sum_partials, kpp_bsums};
+    for (void *p : ptrs)
+      if (p) (void)hipFree(p);
+    if (stream) (void)hipStreamDestroy(stream);
+    stream = nullptr;
+    return 0;
+  }
+
+  int set_data_host(const void *hX) override {
+    KM_HIP_TRY(hipSetDevice(dev));
+    if (!hX) return H2O4GPU_KMEANS_EARG;
+    if (!own_X || !X) {
+      X = nullptr;
+      KM_TRY(dalloc(&X, (size_t)n * d));
+      own_X = true;
+    }
+    KM_HIP_TRY(hipMemcpyAsync(X, hX, (size_t)n * d * sizeof(T), hipMemcpyHostToDevice, stream));
+    PROFILED("row_norms", launch_row_norms<T>(stream, X, xnorm, n, d));
+    KM_HIP_TRY(hipStreamSynchronize(stream));
+    have_data = true;
+    return 0;
+  }
+
+  int set_data_device(const void *dX) override {
+    KM_HIP_TRY(hipSetDevice(dev));
+    if (!dX) return H2O4GPU_KMEANS_EARG;
+    if (own_X && X) (void)hipFree(X);
+    X = const_cast<T *>(static_cast<const T *>(dX));
+    own_X = false;
+    PROFILED("row_norms", launch_row_norms<T>(stream, X, xnorm, n, d));
+    KM_HIP_TRY(hipStreamSynchronize(stream));
+    have_data = true;
+    return 0;
+  }
+
+  int centroids_changed() {
+    PROFILED("row_norms", launch_row_norms<T>(stream, C[cur], cnorm, k, d));
+    have_centroids = true;
+    return 0;
+  }
+
+  int set_centroids_host(const void *hC) override {
+    KM_HIP_TRY(hipSetDevice(dev));
+    if (!hC) return H2O4GPU_KMEANS_EARG;
+    KM_HIP_TRY(hipMemcpyAsync(C[cur], hC, (size_t)k * d * sizeof(T), hipMemcpyHostToDevice, stream));
+    KM_TRY(centroids_changed());
+    KM_HIP_TRY(hipStreamSynchronize(stream));
+    return 0;
+  }
+
+  // Seeded random distinct rows: the same two standard-library calls as
+  // kmeans_h2o4gpu.cu:662-669; centroids are rows v[0..k-1] (:79-84, :692-693).
+  int init_random_rows(int seed) override {
+    KM_HIP_TRY(hipSetDevice(dev));
+    if (!have_data) return H2O4GPU_KMEANS_ESTATE;
+    std::vector<int> v((size_t)n);
+    std::iota(v.begin(), v.end(), 0);
+    if (seed >= 0) {
+      std::shuffle(v.begin(), v.end(), std::default_random_engine(seed));
+    } else {
+      std::random_device rd;
+      std::shuffle(v.begin(), v.end(), std::default_random_engine(rd()));
+    }
+    return init_from_rows(v.data());
+  }
+
+  int init_from_rows(const int *idx_host) {
+    int *didx = nullptr;
+    KM_TRY(dalloc(&didx, k));
+    hipError_t e = hipMemcpyAsync(didx, idx_host, (size_t)k * sizeof(int), hipMemcpyHostToDevice, stream);
+    int rc = e == hipSuccess ? launch_gather_rows<T>(stream, X, didx, C[cur], k, d)
+                             : H2O4GPU_KMEANS_EDEVICE;
+    if (rc == 0) rc = centroids_changed();
+    (void)hipStreamSynchronize(stream);
+    (void)hipFree(didx);
+    return rc;
+  }
+
+  // k-means++ (D^2 sampling). First centre: mt19937(seed) uniform over rows,
+  // as the reference draws its first k-means|| centre
+  // (kmeans_h2o4gpu.cu:343-347). Every further centre: u ~ U[0,1) from the same
+  // generator, target = u * total where total is the ordered double sum of the
+  // block sums; the block is found by an ordered scan of the block sums, the
+  // row by an ordered scan (in double) of that block's minima.
+  int init_plusplus(int seed) override {
+    KM_HIP_TRY(hipSetDevice(dev));
+    if (!have_data) return H2O4GPU_KMEANS_ESTATE;
+    std::mt19937 gen(seed >= 0 ? (unsigned)seed : std::random_device{}());
+    std::uniform_int_distribution<> first(0, (int)(n - 1));
+    std::uniform_real_distribution<double> uni(0.0, 1.0);
+    const int64_t nb = (n + KPP_BLOCK - 1) / KPP_BLOCK;
+    std::vector<int> idx(k);
+    std::vector<double> bs((size_t)nb);
+    std::vector<T> blk(KPP_BLOCK);
+    idx[0] = first(gen);
+    for (int c = 1; c <= k; c++) {
+      PROFILED("min_dist_update",
+               launch_min_dist_update<T>(stream, X, xnorm, idx[c - 1], mindist,
+                                         kpp_bsums, n, d, c == 1));
+      if (c == k) break;
+      KM_HIP_TRY(hipMemcpyAsync(bs.data(), kpp_bsums, (size_t)nb * sizeof(double),
+                                hipMemcpyDeviceToHost, stream));
+      KM_HIP_TRY(hipStreamSynchronize(stream));
+      double total = 0;
+      for (int64_t b = 0; b < nb; b++) total += bs[b];
+      const double u = uni(gen);
+      int64_t pick;
+      if (!(total > 0)) {
+        pick = (int64_t)(u * (double)n);
+        if (pick >= n) pick = n - 1;
+      } else {
+        const double target = u * total;
+        double run = 0;
+        int64_t b = 0;
+        for (; b < nb - 1; b++) {
+          if (run + bs[b] > target) break;
+          run += bs[b];
+        }
+        const int64_t lo = b * KPP_BLOCK;
+        const int cntb = (int)std::min<int64_t>(KPP_BLOCK, n - lo);
+        KM_HIP_TRY(hipMemcpyAsync(blk.data(), mindist + lo, (size_t)cntb * sizeof(T),
+                                  hipMemcpyDeviceToHost, stream));
+        KM_HIP_TRY(hipStreamSynchronize(stream));
+        int i = 0, last_pos = 0;
+        for (; i < cntb; i++) {
+          if ((double)blk[i] > 0) last_pos = i;
+          if (run + (double)blk[i] > target) break;
+          run += (double)blk[i];
+        }
+        if (i >= cntb) i = last_pos;  // rounding left the target past the end
+        pick = lo + i;
+      }
+      idx[c] = (int)pick;
+    }
+    have_mindist = false;
+    last_seed_rows = idx;
+    return init_from_rows(idx.data());
+  }
+  std::vector<int> last_seed_rows;
+
+  int assign() override {
+    KM_HIP_TRY(hipSetDevice(dev));
+    if (!have_data || !have_centroids) return H2O4GPU_KMEANS_ESTATE;
+    PROFILED("assign", launch_assign<T>(stream, opt_assign, X, xnorm, C[cur], cnorm,
+                                        labels, mindist, n, d, k, num_cu, &last_variant));
+    have_mindist = true;
+    return 0;
+  }
+
+  int update_async() {
+    PROFILED("accumulate", launch_accumulate<T>(stream, plan, X, labels, psums, pcounts, n, d, k));
+    int nsp = 0;
+    PROFILED("finalize", launch_finalize<T>(stream, plan, psums, pcounts, C[cur], C[cur ^ 1],
+                                            counts, shift_partials, &nsp, d, k));
+    PROFILED("post_update", launch_post_update<T>(stream, C[cur ^ 1], cnorm, shift_partials,
+                                                  nsp, shift2, d, k));
+    cur ^= 1;
+    return 0;
+  }
+
+  int read_shift2(double *out) {
+    T v;
+    KM_HIP_TRY(hipMemcpyAsync(&v, shift2, sizeof(T), hipMemcpyDeviceToHost, stream));
+    KM_HIP_TRY(hipStreamSynchronize(stream));
+    *out = (double)v;
+    return 0;
+  }
+
+  int update(double *s2) override {
+    KM_HIP_TRY(hipSetDevice(dev));
+    if (!have_data || !have_centroids) return H2O4GPU_KMEANS_ESTATE;
+    KM_TRY(update_async());
+    if (s2) KM_TRY(read_shift2(s2));
+    return 0;
+  }
+
+  // kmeans_impl.h:109-232. The convergence scalar is only fetched when it can
+  // matter (threshold > 0): shift^2 >= 0 can never be below a threshold <= 0,
+  // so a fixed-iteration run has no host synchronisation inside the loop.
+  int fit(int max_iterations, double threshold, int *iters) override {
+    KM_HIP_TRY(hipSetDevice(dev));
+    if (!have_data || !have_centroids) return H2O4GPU_KMEANS_ESTATE;
+    maybe_install_signal_handlers();
+    int updates = 0;
+    for (int i = 0; i < max_iterations; i++) {
+      log_msg(verbose, LOG_VERBOSE, "KMeans - Iteration %d/%d", i, max_iterations);
+      KM_TRY(assign());
+      KM_TRY(update_async());
+      updates++;
+      bool done = false;
+      if (threshold > 0) {
+        double s2 = 0;
+        KM_TRY(read_shift2(&s2));
+        if (s2 < threshold) {
+          log_msg(verbose, LOG_INFO, "Threshold triggered. Terminating early.");
+          done = true;
+        }
+      }
+      if (g_stop_flag) {
+        fprintf(stderr, "Signal caught. Terminated early.\n");
+        g_stop_flag = 0;
+        done = true;
+      }
+      if (done || i == max_iterations - 1) {
+        KM_TRY(assign());  // final relabel with the final centroids
+        break;
+      }
+    }
+    KM_HIP_TRY(hipStreamSynchronize(stream));
+    if (iters) *iters = updates;
+    return 0;
+  }
+
+  int set_labels_host(const int *h) override {
+    KM_HIP_TRY(hipSetDevice(dev));
+    KM_HIP_TRY(hipMemcpyAsync(labels, h, (size_t)n * sizeof(int), hipMemcpyHostToDevice, stream));
+    KM_HIP_TRY(hipStreamSynchronize(stream));
+    return 0;
+  }
+  int d2h(void *dst, const void *src, size_t bytes) {
+    KM_HIP_TRY(hipSetDevice(dev));
+    KM_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, stream));
+    KM_HIP_TRY(hipStreamSynchronize(stream));
+    return 0;
+  }
+  int get_centroids(void *out) override { return d2h(out, C[cur], (size_t)k * d * sizeof(T)); }
+  int get_labels(int *out) override { return d2h(out, labels, (size_t)n * sizeof(int)); }
+  int get_counts(int *out) override { return d2h(out, counts, (size_t)k * sizeof(int)); }
+  int get_min_distances(void *out) override {
+    if (!have_mindist) return H2O4GPU_KMEANS_ESTATE;
+    return d2h(out, mindist, (size_t)n * sizeof(T));
+  }
+  int inertia(double *out) override {
+    KM_HIP_TRY(hipSetDevice(dev));
+    if (!have_mindist) return H2O4GPU_KMEANS_ESTATE;
+    const int np = sum_partials_needed();
+    PROFILED("inertia_sum", launch_sum<T>(stream, mindist, n, sum_partials, np, sum_partials + np));
+    return d2h(out, sum_partials + np, sizeof(double));
+  }
+
+  int predict_host(size_t rows, const void *hX, int *out) override {
+    KM_HIP_TRY(hipSetDevice(dev));
+    if (!have_centroids) return H2O4GPU_KMEANS_ESTATE;
+    if (rows == 0) return 0;
+    T *dX = nullptr, *dxn = nullptr;
+    int *dl = nullptr;
+    int rc = dalloc(&dX, rows * d);
+    if (rc == 0) rc = dalloc(&dxn, rows);
+    if (rc == 0) rc = dalloc(&dl, rows);
+    if (rc == 0) rc = run_predict(rows, hX, out, dX, dxn, dl);
+    (void)hipStreamSynchronize(stream);
+    if (dX) (void)hipFree(dX);
+    if (dxn) (void)hipFree(dxn);
+    if (dl) (void)hipFree(dl);
+    return rc;
+  }
+  int run_predict(size_t rows, const void *hX, int *out, T *dX, T *dxn, int *dl) {
+    KM_HIP_TRY(hipMemcpyAsync(dX, hX, rows * d * sizeof(T), hipMemcpyHostToDevice, stream));
+    PROFILED("row_norms", launch_row_norms<T>(stream, dX, dxn, (int64_t)rows, d));
+    PROFILED("assign", launch_assign<T>(stream, opt_assign, dX, dxn, C[cur], cnorm, dl,
+                                        (T *)nullptr, (int64_t)rows, d, k, num_cu, &last_variant));
+    KM_HIP_TRY(hipMemcpyAsync(out, dl, rows * sizeof(int), hipMemcpyDeviceToHost, stream));
+    KM_HIP_TRY(hipStreamSynchronize(stream));
+    return 0;
+  }
+
+  // The n x k result is produced in row batches of at most ~4 GB so the device
+  // buffer stays bounded; the reference materialises it whole ("TODO batch
+  // this", kmeans_h2o4gpu.cu:936).
+  int transform_host(size_t rows, const void *hX, void *hD) override {
+    KM_HIP_TRY(hipSetDevice(dev));
+    if (!have_centroids) return H2O4GPU_KMEANS_ESTATE;
+    if (rows == 0) return 0;
+    size_t batch = ((size_t)4 << 30) / ((size_t)k * sizeof(T));
+    batch = batch / 128 * 128;
+    if (batch < 128) batch = 128;
+    if (batch > rows) batch = rows;
+    T *dX = nullptr, *dxn = nullptr, *dD = nullptr;
+    int rc = dalloc(&dX, batch * d);
+    if (rc == 0) rc = dalloc(&dxn, batch);
+    if (rc == 0) rc = dalloc(&dD, batch * k);
+    for (size_t lo = 0; rc == 0 && lo < rows; lo += batch) {
+      const size_t cur_rows = std::min(batch, rows - lo);
+      rc = run_transform_batch(lo, cur_rows, rows, hX, hD, dX, dxn, dD);
+    }
+    (void)hipStreamSynchronize(stream);
+    if (dX) (void)hipFree(dX);
+    if (dxn) (void)hipFree(dxn);
+    if (dD) (void)hipFree(dD);
+    return rc;
+  }
+  int run_transform_batch(size_t lo, size_t cur_rows, size_t rows, const void *hX, void *hD,
+                          T *dX, T *dxn, T *dD) {
+    const T *src = static_cast<const T *>(hX) + lo * d;
+    KM_HIP_TRY(hipMemcpyAsync(dX, src, cur_rows * d * sizeof(T), hipMemcpyHostToDevice, stream));
+    PROFILED("row_norms", launch_row_norms<T>(stream, dX, dxn, (int64_t)cur_rows, d));
+    PROFILED("transform", launch_transform<T>(stream, dX, dxn, C[cur], cnorm, dD,
+                                              (int64_t)cur_rows, (int64_t)cur_rows, d, k, num_cu));
+    T *dst = static_cast<T *>(hD) + lo;
+    KM_HIP_TRY(hipMemcpy2DAsync(dst, rows * sizeof(T), dD, cur_rows * sizeof(T),
+                                cur_rows * sizeof(T), (size_t)k, hipMemcpyDeviceToHost, stream));
+    KM_HIP_TRY(hipStreamSynchronize(stream));
+    return 0;
+  }
+  int transform_resident(void *d_dist) override {
+    KM_HIP_TRY(hipSetDevice(dev));
+    if (!have_data || !have_centroids || !d_dist) return H2O4GPU_KMEANS_ESTATE;
+    PROFILED("transform", launch_transform<T>(stream, X, xnorm, C[cur], cnorm,
+                                              static_cast<T *>(d_dist), n, n, d, k, num_cu));
+    KM_HIP_TRY(hipStreamSynchronize(stream));
+    return 0;
+  }
+};
+
+template <typename T>
+static int create_engine(h2o4gpu_kmeans_handle **out, size_t rows, size_t cols, int k,
+                         int gpu_id, int verbose) {
+  const int nvis = visible_devices();
+  if (nvis < 1) {
+    log_msg(verbose ? verbose : LOG_ERROR, LOG_ERROR, "no HIP device visible");
+    return H2O4GPU_KMEANS_EDEVICE;
+  }
+  Engine<T> *e = new (std::nothrow) Engine<T>();
+  if (!e) return H2O4GPU_KMEANS_EALLOC;
+  e->elem_size = sizeof(T);
+  e->n = (int64_t)rows;
+  e->d = (int)cols;
+  e->k = k;
+  e->verbose = verbose;
+  if (gpu_id < 0) gpu_id = 0;
+  e->dev = gpu_id % nvis;  // kmeans_init: gpu_id = gpu_idtry % n_gpuvis
+  int rc = e->create();
+  if (rc != 0) {
+    e->release();
+    delete e;
+    return rc;
+  }
+  *out = e;
+  return 0;
+}
+
+}  // namespace kmhip
+
+#define KM_API __attribute__((visibility("default")))
+extern "C" KM_API int h2o4gpu_kmeans_create(h2o4gpu_kmeans_handle **out, int elem_size, size_t rows,
+                                            size_t cols, int k, int gpu_id, int verbose);
+extern "C" KM_API int h2o4gpu_kmeans_destroy(h2o4gpu_kmeans_handle *h);
+
+__global__ void copy_probe_kernel(const float4 *__restrict__ src, float4 *__restrict__ dst,
+                                  size_t nvec) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += stride)
+    dst[i] = src[i];
+}
+
+// ---------------------------------------------------------------------------
+// C ABI, part 1: the reference's entry points
+// ---------------------------------------------------------------------------
+template <typename T>
+static int fit_entry(int verbose, int seed, int gpu_id, size_t rows, size_t cols, int k,
+                     int max_iterations, int init_from_data, double threshold,
+                     const T *srcdata, const T *centroids, T **pred_centroids,
+                     int **pred_labels) {
+  if (!srcdata || !pred_centroids || !pred_labels || rows < 1 || cols < 1 || k < 1)
+    return H2O4GPU_KMEANS_EARG;
+  if ((size_t)k > rows) {  // kmeans_h2o4gpu.cu:630-635
+    k = (int)rows;
+    fprintf(stderr, "Number of clusters adjusted to be equal to number of rows.\n");
+    fflush(stderr);
+  }
+  h2o4gpu_kmeans_handle *h = nullptr;
+  KM_TRY(h2o4gpu_kmeans_create(&h, sizeof(T), rows, cols, k, gpu_id, verbose));
+  int rc = h->set_data_host(srcdata);
+  if (rc == 0) {
+    if (init_from_data == 0) {
+      rc = h->init_random_rows(seed);
+    } else if (init_from_data == 1) {
+      rc = h->init_plusplus(seed);
+    } else if (init_from_data == 2) {
+      rc = centroids ? h->set_centroids_host(centroids) : H2O4GPU_KMEANS_EARG;
+    } else {
+      // the reference has no branch for other values and runs from all-zero
+      // centroids (kmeans_h2o4gpu.cu:684-740); same here
+      std::vector<T> zeros((size_t)k * cols, (T)0);
+      rc = h->set_centroids_host(zeros.data());
+    }
+  }
+  int iters = 0;
+  if (rc == 0) rc = h->fit(max_iterations, threshold, &iters);
+  T *oc = nullptr;
+  int *ol = nullptr;
+  if (rc == 0) {
+    oc = static_cast<T *>(malloc((size_t)k * cols * sizeof(T)));
+    ol = static_cast<int *>(malloc(rows * sizeof(int)));
+    if (!oc || !ol) rc = H2O4GPU_KMEANS_EALLOC;
+  }
+  if (rc == 0) rc = h->get_centroids(oc);
+  if (rc == 0) rc = h->get_labels(ol);
+  h2o4gpu_kmeans_destroy(h);
+  if (rc != 0) {
+    free(oc);
+    free(ol);
+    log_msg(verbose ? verbose : LOG_ERROR, LOG_ERROR, "KMeans algorithm failed (%d).", rc);
+    return rc;
+  }
+  *pred_centroids = oc;
+  *pred_labels = ol;
+  log_msg(verbose, LOG_INFO, "fit: %d iterations", iters);
+  return 0;
+}
+
+template <typename T>
+static int predict_entry(int verbose, int gpu_id, size_t rows, size_t cols, int k,
+                         const T *srcdata, const T *centroids, int **pred_labels) {
+  if (!srcdata || !centroids || !pred_labels || rows < 1 || cols < 1 || k < 1)
+    return H2O4GPU_KMEANS_EARG;
+  h2o4gpu_kmeans_handle *h = nullptr;
+  // a predict handle needs no resident rows: size its working set for one row
+  KM_TRY(h2o4gpu_kmeans_create(&h, sizeof(T), (size_t)std::max(k, 1), cols, k, gpu_id, verbose));
+  int rc = h->set_centroids_host(centroids);
+  int *ol = nullptr;
+  if (rc == 0) {
+    ol = static_cast<int *>(malloc(rows * sizeof(int)));
+    if (!ol) rc = H2O4GPU_KMEANS_EALLOC;
+  }
+  if (rc == 0) rc = h->predict_host(rows, srcdata, ol);
+  h2o4gpu_kmeans_destroy(h);
+  if (rc != 0) {
+    free(ol);
+    return rc;
+  }
+  *pred_labels = ol;
+  return 0;
+}
+
+template <typename T>
+static int transform_entry(int verbose, int gpu_id, size_t rows, size_t cols, int k,
+                           const T *srcdata, const T *centroids, T **preds) {
+  if (!srcdata || !centroids || !preds || rows < 1 || cols < 1 || k < 1)
+    return H2O4GPU_KMEANS_EARG;
+  h2o4gpu_kmeans_handle *h = nullptr;
+  KM_TRY(h2o4gpu_kmeans_create(&h, sizeof(T), (size_t)std::max(k, 1), cols, k, gpu_id, verbose));
+  int rc = h->set_centroids_host(centroids);
+  T *out = nullptr;
+  if (rc == 0) {
+    out = static_cast<T *>(malloc(rows * (size_t)k * sizeof(T)));
+    if (!out) rc = H2O4GPU_KMEANS_EALLOC;
+  }
+  if (rc == 0) rc = h->transform_host(rows, srcdata, out);
+  h2o4gpu_kmeans_destroy(h);
+  if (rc != 0) {
+    free(out);
+    return rc;
+  }
+  *preds = out;
+  return 0;
+}
+
+
+// ---------------------------------------------------------------------------
+// C ABI, part 3
+// ---------------------------------------------------------------------------
+extern "C" {
+
+#define KM_CHECK_HANDLE(h) \
+  if (!(h)) return H2O4GPU_KMEANS_EARG
+
+KM_API int h2o4gpu_kmeans_create(h2o4gpu_kmeans_handle **out, int elem_size, size_t rows,
+                                 size_t cols, int k, int gpu_id, int verbose) {
+  if (!out) return H2O4GPU_KMEANS_EARG;
+  *out = nullptr;
+  // rows must fit int32 (labels and row indices are int32, as in kmeans_init
+  // kmeans_h2o4gpu.cu:574-579, which exits instead)
+  if (rows < 1 || cols < 1 || k < 1 || rows > 2147483647ull || cols > 1000000ull ||
+      (size_t)k > rows)
+    return H2O4GPU_KMEANS_EARG;
+  if (elem_size == 4) return create_engine<float>(out, rows, cols, k, gpu_id, verbose);
+  if (elem_size == 8) return create_engine<double>(out, rows, cols, k, gpu_id, verbose);
+  return H2O4GPU_KMEANS_EARG;
+}
+KM_API int h2o4gpu_kmeans_destroy(h2o4gpu_kmeans_handle *h) {
+  KM_CHECK_HANDLE(h);
+  h->release();
+  delete h;
+  return 0;
+}
+KM_API int h2o4gpu_kmeans_set_data_host(h2o4gpu_kmeans_handle *h, const void *X) {
+  KM_CHECK_HANDLE(h);
+  return h->set_data_host(X);
+}
+KM_API int h2o4gpu_kmeans_set_data_device(h2o4gpu_kmeans_handle *h, const void *dX) {
+  KM_CHECK_HANDLE(h);
+  return h->set_data_device(dX);
+}
+KM_API int h2o4gpu_kmeans_set_centroids_host(h2o4gpu_kmeans_handle *h, const void *C) {
+  KM_CHECK_HANDLE(h);
+  return h->set_centroids_host(C);
+}
+KM_API int h2o4gpu_kmeans_init_random_rows(h2o4gpu_kmeans_handle *h, int seed) {
+  KM_CHECK_HANDLE(h);
+  return h->init_random_rows(seed);
+}
+KM_API int h2o4gpu_kmeans_init_plusplus(h2o4gpu_kmeans_handle *h, int seed) {
+  KM_CHECK_HANDLE(h);
+  return h->init_plusplus(seed);
+}
+KM_API int h2o4gpu_kmeans_fit(h2o4gpu_kmeans_handle *h, int max_iterations, double threshold,
+                              int *iterations_run) {
+  KM_CHECK_HANDLE(h);
+  return h->fit(max_iterations, threshold, iterations_run);
+}
+KM_API int h2o4gpu_kmeans_assign(h2o4gpu_kmeans_handle *h) {
+  KM_CHECK_HANDLE(h);
+  int rc = h->assign();
+  if (rc == 0 && hipStreamSynchronize(h->stream) != hipSuccess) rc = H2O4GPU_KMEANS_EDEVICE;
+  return rc;
+}
+KM_API int h2o4gpu_kmeans_update(h2o4gpu_kmeans_handle *h, double *shift2) {
+  KM_CHECK_HANDLE(h);
+  int rc = h->update(shift2);
+  if (rc == 0 && hipStreamSynchronize(h->stream) != hipSuccess) rc = H2O4GPU_KMEANS_EDEVICE;
+  return rc;
+}
+KM_API int h2o4gpu_kmeans_set_labels_host(h2o4gpu_kmeans_handle *h, const int *labels) {
+  KM_CHECK_HANDLE(h);
+  if (!labels) return H2O4GPU_KMEANS_EARG;
+  return h->set_labels_host(labels);
+}
+KM_API int h2o4gpu_kmeans_get_centroids(h2o4gpu_kmeans_handle *h, void *C) {
+  KM_CHECK_HANDLE(h);
+  return C ? h->get_centroids(C) : H2O4GPU_KMEANS_EARG;
+}
+KM_API int h2o4gpu_kmeans_get_labels(h2o4gpu_kmeans_handle *h, int *labels) {
+  KM_CHECK_HANDLE(h);
+  return labels ? h->get_labels(labels) : H2O4GPU_KMEANS_EARG;
+}
+KM_API int h2o4gpu_kmeans_get_counts(h2o4gpu_kmeans_handle *h, int *counts) {
+  KM_CHECK_HANDLE(h);
+  return counts ? h->get_counts(counts) : H2O4GPU_KMEANS_EARG;
+}
+KM_API int h2o4gpu_kmeans_get_min_distances(h2o4gpu_kmeans_handle *h, void *m) {
+  KM_CHECK_HANDLE(h);
+  return m ? h->get_min_distances(m) : H2O4GPU_KMEANS_EARG;
+}
+KM_API int h2o4gpu_kmeans_inertia(h2o4gpu_kmeans_handle *h, double *inertia) {
+  KM_CHECK_HANDLE(h);
+  return inertia ? h->inertia(inertia) : H2O4GPU_KMEANS_EARG;
+}
+KM_API int h2o4gpu_kmeans_predict_host(h2o4gpu_kmeans_handle *h, size_t rows, const void *X,
+                                       int *labels) {
+  KM_CHECK_HANDLE(h);
+  if (rows > 0 && (!X || !labels)) return H2O4GPU_KMEANS_EARG;
+  if (rows > 2147483647ull) return H2O4GPU_KMEANS_EARG;
+  return h->predict_host(rows, X, labels);
+}
+KM_API int h2o4gpu_kmeans_transform_host(h2o4gpu_kmeans_handle *h, size_t rows, const void *X,
+                                         void *dist) {
+  KM_CHECK_HANDLE(h);
+  if (rows > 0 && (!X || !dist)) return H2O4GPU_KMEANS_EARG;
+  if (rows > 2147483647ull) return H2O4GPU_KMEANS_EARG;
+  return h->transform_host(rows, X, dist);
+}
+KM_API int h2o4gpu_kmeans_transform_resident(h2o4gpu_kmeans_handle *h, void *d_dist) {
+  KM_CHECK_HANDLE(h);
+  return h->transform_resident(d_dist);
+}
+KM_API int h2o4gpu_kmeans_set_option(h2o4gpu_kmeans_handle *h, const char *name, int value) {
+  KM_CHECK_HANDLE(h);
+  if (!name) return H2O4GPU_KMEANS_EARG;
+  if (strcmp(name, "assign") == 0) {
+    if (value < ASSIGN_AUTO || value > ASSIGN_TILED) return H2O4GPU_KMEANS_EARG;
+    h->opt_assign = value;
+    return 0;
+  }
+  if (strcmp(name, "update") == 0) return value == 0 ? 0 : H2O4GPU_KMEANS_EARG;
+  return H2O4GPU_KMEANS_EARG;
+}
+KM_API int h2o4gpu_kmeans_timer_start(h2o4gpu_kmeans_handle *h) {
+  KM_CHECK_HANDLE(h);
+  KM_HIP_TRY(hipSetDevice(h->dev));
+  if (!h->t0) KM_HIP_TRY(hipEventCreate(&h->t0));
+  if (!h->t1) KM_HIP_TRY(hipEventCreate(&h->t1));
+  KM_HIP_TRY(hipEventRecord(h->t0, h->stream));
+  return 0;
+}
+KM_API int h2o4gpu_kmeans_timer_stop(h2o4gpu_kmeans_handle *h, float *ms) {
+  KM_CHECK_HANDLE(h);
+  if (!h->t0 || !h->t1 || !ms) return H2O4GPU_KMEANS_ESTATE;
+  KM_HIP_TRY(hipSetDevice(h->dev));
+  KM_HIP_TRY(hipEventRecord(h->t1, h->stream));
+  KM_HIP_TRY(hipEventSynchronize(h->t1));
+  KM_HIP_TRY(hipEventElapsedTime(ms, h->t0, h->t1));
+  return 0;
+}
+KM_API int h2o4gpu_kmeans_profile(h2o4gpu_kmeans_handle *h, int on) {
+  KM_CHECK_HANDLE(h);
+  KM_HIP_TRY(hipSetDevice(h->dev));
+  KM_TRY(h->prof_resolve());
+  h->prof_on = on != 0;
+  if (on) h->prof.clear();
+  return 0;
+}
+KM_API int h2o4gpu_kmeans_kernel_time(h2o4gpu_kmeans_handle *h, const char *kernel,
+                                      int *launches, double *ms) {
+  KM_CHECK_HANDLE(h);
+  if (!kernel) return H2O4GPU_KMEANS_EARG;
+  KM_HIP_TRY(hipSetDevice(h->dev));
+  KM_TRY(h->prof_resolve());
+  auto it = h->prof.find(kernel);
+  if (launches) *launches = it == h->prof.end() ? 0 : it->second.first;
+  if (ms) *ms = it == h->prof.end() ? 0.0 : it->second.second;
+  return 0;
+}
+KM_API const char *h2o4gpu_kmeans_assign_variant(h2o4gpu_kmeans_handle *h) {
+  if (!h) return "";
+  int v = h->elem_size == 4 ? pick_assign_variant<float>(h->opt_assign, h->n, h->d, h->k)
+                            : pick_assign_variant<double>(h->opt_assign, h->n, h->d, h->k);
+  return v < 0 ? "unsupported" : assign_variant_name(v);
+}
+
+KM_API int h2o4gpu_kmeans_copy_probe(int gpu_id, size_t bytes, int reps, float *ms) {
+  if (!ms || reps < 1 || bytes < 16) return H2O4GPU_KMEANS_EARG;
+  const int nvis = visible_devices();
+  if (nvis < 1) return H2O4GPU_KMEANS_EDEVICE;
+  KM_HIP_TRY(hipSetDevice((gpu_id < 0 ? 0 : gpu_id) % nvis));
+  void *a = nullptr, *b = nullptr;
+  if (hipMalloc(&a, bytes) != hipSuccess || hipMalloc(&b, bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    if (a) (void)hipFree(a);
+    return H2O4GPU_KMEANS_EALLOC;
+  }
+  hipEvent_t e0, e1;
+  int rc = 0;
+  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) rc = H2O4GPU_KMEANS_EDEVICE;
+  if (rc == 0) {
+    (void)hipMemset(a, 1, bytes);
+    (void)hipMemset(b, 0, bytes);
+    const size_t nvec = bytes / 16;
+    hipLaunchKernelGGL(copy_probe_kernel, dim3(256 * 8), dim3(256), 0, 0, (const float4 *)a, (float4 *)b, nvec);
+    (void)hipDeviceSynchronize();
+    (void)hipEventRecord(e0, 0);
+    for (int r = 0; r < reps; r++)
+      hipLaunchKernelGGL(copy_probe_kernel, dim3(256 * 8), dim3(256), 0, 0, (const float4 *)a, (float4 *)b, nvec);
+    (void)hipEventRecord(e1, 0);
+    if (hipEventSynchronize(e1) != hipSuccess) rc = H2O4GPU_KMEANS_EDEVICE;
+    float t = 0;
+    if (rc == 0 && hipEventElapsedTime(&t, e0, e1) == hipSuccess) *ms = t / reps;
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+  }
+  (void)hipFree(a);
+  (void)hipFree(b);
+  return rc;
+}
+
+KM_API int make_ptr_float_kmeans(int dopredict, int verbose, int seed, int gpu_id, int n_gpu,
+                                 size_t mTrain, size_t n, int k, int max_iterations,
+                                 int init_from_data, float threshold, const float *srcdata,
+                                 const float *centroids, float **pred_centroids,
+                                 int **pred_labels) {
+  (void)n_gpu;
+  if (dopredict == 0)
+    return fit_entry<float>(verbose, seed, gpu_id, mTrain, n, k, max_iterations, init_from_data,
+                            (double)threshold, srcdata, centroids, pred_centroids, pred_labels);
+  return predict_entry<float>(verbose, gpu_id, mTrain, n, k, srcdata, centroids, pred_labels);
+}
+KM_API int make_ptr_double_kmeans(int dopredict, int verbose, int seed, int gpu_id, int n_gpu,
+                                  size_t mTrain, size_t n, int k, int max_iterations,
+                                  int init_from_data, double threshold, const double *srcdata,
+                                  const double *centroids, double **pred_centroids,
+                                  int **pred_labels) {
+  (void)n_gpu;
+  if (dopredict == 0)
+    return fit_entry<double>(verbose, seed, gpu_id, mTrain, n, k, max_iterations, init_from_data,
+                             threshold, srcdata, centroids, pred_centroids, pred_labels);
+  return predict_entry<double>(verbose, gpu_id, mTrain, n, k, srcdata, centroids, pred_labels);
+}
+KM_API int kmeans_transform_float(int verbose, int gpu_id, int n_gpu, size_t m, size_t n, int k,
+                                  const float *srcdata, const float *centroids, float **preds) {
+  (void)n_gpu;
+  return transform_entry<float>(verbose, gpu_id, m, n, k, srcdata, centroids, preds);
+}
+KM_API int kmeans_transform_double(int verbose, int gpu_id, int n_gpu, size_t m, size_t n, int k,
+                                   const double *srcdata, const double *centroids,
+                                   double **preds) {
+  (void)n_gpu;
+  return transform_entry<double>(verbose, gpu_id, m, n, k, srcdata, centroids, preds);
+}
+
+// ---------------------------------------------------------------------------
+// C ABI, part 2: device information
+// ---------------------------------------------------------------------------
+KM_API int h2o4gpu_kmeans_device_count(void) { return visible_devices(); }
+
+KM_API int get_gpu_info_c(int verbose, int return_memory, int return_name, int return_usage,
+                          int return_free_memory, int return_capability,
+                          int return_memory_by_pid, int return_usage_by_pid, int return_all,
+                          unsigned int *n_gpus, int *gpu_percent_usage,
+                          unsigned long long *gpu_total_memory,
+                          unsigned long long *gpu_free_memory, char **gpu_name, int *majors,
+                          int *minors, unsigned int *num_pids, unsigned int *pids,
+                          unsigned long long *usedGpuMemorys, unsigned int *num_pids_usage,
+                          unsigned int *pids_usage, unsigned long long *usedGpuUsage) {
+  (void)pids;
+  (void)usedGpuMemorys;
+  (void)pids_usage;
+  (void)usedGpuUsage;
+  const int nvis = visible_devices();
+  if (n_gpus) *n_gpus = (unsigned)nvis;
+  if (nvis < 1) {
+    log_msg(verbose, LOG_FATAL, "no HIP device visible");
+    return 1;
+  }
+  for (int i = 0; i < nvis; i++) {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, i) != hipSuccess) continue;
+    if ((return_memory || return_all) && gpu_total_memory) gpu_total_memory[i] = prop.totalGlobalMem;
+    if ((return_free_memory || return_all) && gpu_free_memory) {
+      size_t fr = 0, tot = 0;
+      if (hipSetDevice(i) == hipSuccess && hipMemGetInfo(&fr, &tot) == hipSuccess) gpu_free_memory[i] = fr;
+    }
+    if ((return_name || return_all) && gpu_name && gpu_name[i]) {
+      strncpy(gpu_name[i], prop.name, 29);
+      gpu_name[i][29] = '\0';
+    }
+    if ((return_capability || return_all) && majors && minors) {
+      majors[i] = prop.major;
+      minors[i] = prop.minor;
+    }
+    if ((return_usage || return_all) && gpu_percent_usage) gpu_percent_usage[i] = 0;
+    if ((return_memory_by_pid || return_all) && num_pids) num_pids[i] = 0;
+    if ((return_usage_by_pid || return_all) && num_pids_usage) num_pids_usage[i] = 0;
+  }
+  return 0;
+}
+KM_API int get_compute_capability(int d_idx, int *major, int *minor, int *ratioperf) {
+  hipDeviceProp_t prop;
+  hipError_t e = hipGetDeviceProperties(&prop, d_idx);
+  if (e != hipSuccess) return (int)e;
+  if (major) *major = prop.major;
+  if (minor) *minor = prop.minor;
+  if (ratioperf) *ratioperf = 2;  // fp32 : fp64 matrix rate on MI355X
+  return 0;
+}
+KM_API int cudaresetdevice(int wDev, int nDev) {
+  (void)nDev;
+  if (hipSetDevice(wDev) != hipSuccess) return 1;
+  return hipDeviceReset() == hipSuccess ? 0 : 1;
+}
+KM_API int cudaresetdevice_bare(void) { return hipDeviceReset() == hipSuccess ? 0 : 1; }
+
+}  // extern "C"

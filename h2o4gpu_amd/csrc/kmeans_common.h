@@ -1,0 +1,123 @@
+// Shared declarations of the gfx950 k-means engine: status codes, logging,
+// launch-parameter structs and the kernel launchers each .hip file provides.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/h2o4gpu_kmeans.h"
+
+namespace kmhip {
+
+// Logger levels as the reference defines them (src/common/logger.h:10-25):
+// a message of level L is printed when 0 < L <= verbose.
+enum LogLevel {
+  LOG_NOTHING = 0,
+  LOG_FATAL = 100,
+  LOG_ERROR = 200,
+  LOG_INFO = 300,
+  LOG_WARN = 400,
+  LOG_DEBUG = 500,
+  LOG_VERBOSE = 600
+};
+void log_msg(int verbose, int level, const char *fmt, ...)
+    __attribute__((format(printf, 3, 4)));
+
+#define KM_HIP_TRY(expr)                                                     \
+  do {                                                                       \
+    hipError_t _e = (expr);                                                  \
+    if (_e != hipSuccess) {                                                  \
+      ::kmhip::log_msg(LOG_ERROR, LOG_ERROR, "%s:%d %s failed: %s", __FILE__, \
+                       __LINE__, #expr, hipGetErrorString(_e));              \
+      return (_e == hipErrorOutOfMemory) ? H2O4GPU_KMEANS_EALLOC              \
+                                         : H2O4GPU_KMEANS_EDEVICE;           \
+    }                                                                        \
+  } while (0)
+
+#define KM_TRY(expr)            \
+  do {                          \
+    int _rc = (expr);           \
+    if (_rc != 0) return _rc;   \
+  } while (0)
+
+// Assign-kernel variants (value of the "assign" option).
+enum AssignVariant {
+  ASSIGN_AUTO = 0,
+  ASSIGN_VALU = 1,     // one thread per row, centroids broadcast from LDS
+  ASSIGN_ROWSTAT = 2,  // MFMA, row tile stationary in registers, all centroids in LDS
+  ASSIGN_TILED = 3     // MFMA, both operands staged through LDS over a d-loop
+};
+
+// Fused distance + argmin. labels[i] = argmin_c |(xx_i + cc_c) - 2 x_i.c_c|,
+// strict '<', lowest index wins, -1 when no distance is below FLT_MAX.
+// mindist (nullable) receives the minimum. Returns the variant actually used
+// through *used (nullable).
+template <typename T>
+int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
+                  const T *C, const T *cnorm, int *labels, T *mindist,
+                  int64_t n, int d, int k, int num_cu, int *used);
+template <typename T>
+int pick_assign_variant(int requested, int64_t n, int d, int k);
+const char *assign_variant_name(int variant);
+
+// Full squared-distance matrix, centroid-major: D[c * ldn + i], i < n.
+template <typename T>
+int launch_transform(hipStream_t s, const T *X, const T *xnorm, const T *C,
+                     const T *cnorm, T *D, int64_t n, int64_t ldn, int d, int k,
+                     int num_cu);
+
+// out[i] = sum_j X[i][j]^2, j ascending, no contraction.
+template <typename T>
+int launch_row_norms(hipStream_t s, const T *X, T *out, int64_t n, int d);
+
+// Centroid update, pass 1: per-row-block partial sums and counts.
+struct UpdatePlan {
+  int row_blocks;   // partial slots along rows
+  int kc;           // centroids per LDS chunk
+  int k_chunks;     // ceil(k / kc)
+  int vec;          // elements per load (1, 2 or 4)
+  size_t lds_bytes;
+};
+template <typename T>
+UpdatePlan plan_update(int64_t n, int d, int k, int num_cu);
+template <typename T>
+int launch_accumulate(hipStream_t s, const UpdatePlan &p, const T *X,
+                      const int *labels, T *psums, int *pcounts, int64_t n,
+                      int d, int k);
+// Pass 2: fixed-order reduction of the partials, empty clusters keep the old
+// centroid, mean = sum * (1/count), per-block partial of sum((old-new)^2).
+template <typename T>
+int launch_finalize(hipStream_t s, const UpdatePlan &p, const T *psums,
+                    const int *pcounts, const T *c_old, T *c_new, int *counts,
+                    T *shift_partials, int *n_shift_partials, int d, int k);
+// Pass 3: cnorm of the new centroids and the fixed-order sum of the shift
+// partials into *shift2.
+template <typename T>
+int launch_post_update(hipStream_t s, const T *c_new, T *cnorm,
+                       const T *shift_partials, int n_shift_partials, T *shift2,
+                       int d, int k);
+
+// Deterministic sum of n values (two fixed-order stages), result in double.
+template <typename T>
+int launch_sum(hipStream_t s, const T *v, int64_t n, double *partials,
+               int n_partials, double *out);
+int sum_partials_needed();
+
+// k-means++ seeding: mind[i] = min(mind[i], |xx_i + cc - 2 x_i.c|) against one
+// centre (row `centre_row` of X; init != 0 overwrites instead of taking the
+// min), then bsums[b] = sum of mind over rows [b*KPP_BLOCK, (b+1)*KPP_BLOCK) in
+// double with a fixed tree.
+static const int KPP_BLOCK = 1024;
+template <typename T>
+int launch_min_dist_update(hipStream_t s, const T *X, const T *xnorm,
+                           int64_t centre_row, T *mind, double *bsums, int64_t n,
+                           int d, int init);
+
+// Copy rows idx[0..k-1] of X into C ([k][d]).
+template <typename T>
+int launch_gather_rows(hipStream_t s, const T *X, const int *idx, T *C, int k,
+                       int d);
+
+}  // namespace kmhip

@@ -1,0 +1,456 @@
+// Row norms, centroid update and reductions.
+//
+// The centroid update replaces the reference's find_centroids
+// (src/gpu/kmeans/kmeans_centroids.h:108-189: copy old centroids, sort (label,
+// index) pairs, zero, 30-block run-length accumulate with global atomics,
+// revert empties, scale) by
+//   pass 1  accumulate : every workgroup owns a contiguous block of rows and a
+//           chunk of centroids, keeps that chunk's sums and counts in LDS and
+//           writes them to its own slot of a partials buffer (no global
+//           atomics, no sort);
+//   pass 2  finalize   : sums the slots in slot order, applies the reference's
+//           rules (count < 1 keeps the old centroid; mean = sum * (1/count)),
+//           and emits per-block partials of sum((old-new)^2);
+//   pass 3  post_update: centroid norms for the next assign and the ordered
+//           sum of the shift partials.
+#include "kmeans_common.h"
+
+namespace kmhip {
+
+static constexpr int WG = 256;
+
+// LDS floating-point add without return value (ds_add_f32 / ds_add_f64).
+__device__ __forceinline__ void lds_add(float *p, float v) {
+  __builtin_amdgcn_ds_faddf((__attribute__((address_space(3))) float *)p, v, 0, 0, false);
+}
+__device__ __forceinline__ void lds_add(double *p, double v) {
+  unsafeAtomicAdd(p, v);
+}
+
+// ---------------------------------------------------------------------------
+// out[i] = sum_j X[i][j]^2, j ascending, multiply and add rounded separately
+// (what self_dots does, kmeans_labels.h:187-199). One thread per row; used once
+// per fit on the data and on k rows per iteration.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(WG) void row_norms_kernel(const T *__restrict__ X,
+                                                      T *__restrict__ out,
+                                                      int64_t n, int d) {
+#pragma clang fp contract(off)
+  const int64_t i = (int64_t)blockIdx.x * WG + threadIdx.x;
+  if (i >= n) return;
+  const T *x = X + i * (int64_t)d;
+  T acc = 0;
+  for (int j = 0; j < d; j++) {
+    const T v = x[j];
+    acc = acc + v * v;
+  }
+  out[i] = acc;
+}
+
+// Same result, but a group of LPR lanes cooperates on a row so that global
+// loads are coalesced; the partial products are exchanged and then added in j
+// order by one lane, which keeps the sum bit-identical to the scalar loop.
+// Used for the large one-off pass over the data (d <= 64 * VEC).
+template <typename T, int LPR>
+__global__ __launch_bounds__(WG) void row_norms_coalesced_kernel(
+    const T *__restrict__ X, T *__restrict__ out, int64_t n, int d) {
+#pragma clang fp contract(off)
+  constexpr int ROWS = WG / LPR;
+  __shared__ T sq[ROWS][LPR + 1];
+  const int sub = threadIdx.x / LPR, col = threadIdx.x % LPR;
+  const int64_t row0 = (int64_t)blockIdx.x * ROWS;
+  const int64_t row = row0 + sub;
+  T acc = 0;
+  for (int j0 = 0; j0 < d; j0 += LPR) {
+    const int j = j0 + col;
+    T v = (row < n && j < d) ? X[row * (int64_t)d + j] : (T)0;
+    sq[sub][col] = v * v;
+    __syncthreads();
+    if (col == 0) {
+      const int lim = min(LPR, d - j0);
+      for (int e = 0; e < lim; e++) acc = acc + sq[sub][e];
+    }
+    __syncthreads();
+  }
+  if (col == 0 && row < n) out[row] = acc;
+}
+
+template <typename T>
+int launch_row_norms(hipStream_t s, const T *X, T *out, int64_t n, int d) {
+  if (n <= 0) return 0;
+  if (n >= 65536 && d >= 8) {
+    if (d <= 16) {
+      constexpr int LPR = 16;
+      hipLaunchKernelGGL((row_norms_coalesced_kernel<T, LPR>),
+                         dim3((unsigned)((n + WG / LPR - 1) / (WG / LPR))), dim3(WG), 0,
+                         s, X, out, n, d);
+    } else if (d <= 32) {
+      constexpr int LPR = 32;
+      hipLaunchKernelGGL((row_norms_coalesced_kernel<T, LPR>),
+                         dim3((unsigned)((n + WG / LPR - 1) / (WG / LPR))), dim3(WG), 0,
+                         s, X, out, n, d);
+    } else {
+      constexpr int LPR = 64;
+      hipLaunchKernelGGL((row_norms_coalesced_kernel<T, LPR>),
+                         dim3((unsigned)((n + WG / LPR - 1) / (WG / LPR))), dim3(WG), 0,
+                         s, X, out, n, d);
+    }
+  } else {
+    hipLaunchKernelGGL((row_norms_kernel<T>), dim3((unsigned)((n + WG - 1) / WG)),
+                       dim3(WG), 0, s, X, out, n, d);
+  }
+  KM_HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// pass 1: accumulate
+// grid (row_blocks, k_chunks). LDS: sums[kc][d] + counts[kc].
+// A wavefront reads 64 labels at a time, then serves the matching rows one
+// group at a time: LPR lanes (each VEC consecutive features per step) per row,
+// 64/LPR rows in flight. With a single centroid chunk every row matches and
+// the ballot is skipped.
+// ---------------------------------------------------------------------------
+template <typename T, int VEC>
+struct VecOf;
+template <> struct VecOf<float, 4> { typedef float type __attribute__((ext_vector_type(4))); };
+template <> struct VecOf<float, 2> { typedef float type __attribute__((ext_vector_type(2))); };
+template <> struct VecOf<double, 2> { typedef double type __attribute__((ext_vector_type(2))); };
+
+template <typename T, int VEC>
+__device__ __forceinline__ void add_row_slice(T *srow, const T *xrow, int col,
+                                              int lpr, int d) {
+  // lanes col, col+lpr, ... each take VEC consecutive features
+  for (int j = col * VEC; j < d; j += lpr * VEC) {
+    if constexpr (VEC == 1) {
+      lds_add(srow + j, xrow[j]);
+    } else {
+      typedef typename VecOf<T, VEC>::type vt;
+      const vt v = *reinterpret_cast<const vt *>(xrow + j);
+#pragma unroll
+      for (int e = 0; e < VEC; e++) lds_add(srow + j + e, v[e]);
+    }
+  }
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(WG) void accumulate_kernel(
+    const T *__restrict__ X, const int *__restrict__ labels,
+    T *__restrict__ psums, int *__restrict__ pcounts, int64_t n, int d, int k,
+    int kc, int64_t rows_per_block, int lpr) {
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  T *sums = reinterpret_cast<T *>(smem_raw);                  // [kc][d]
+  int *cnt = reinterpret_cast<int *>(sums + (size_t)kc * d);  // [kc]
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int k0 = blockIdx.y * kc;
+  const int nk = min(kc, k - k0);
+  for (int e = tid; e < nk * d; e += WG) sums[e] = (T)0;
+  for (int c = tid; c < nk; c += WG) cnt[c] = 0;
+  __syncthreads();
+
+  const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
+  const int64_t r1 = min(n, r0 + rows_per_block);
+  const int rps = 64 / lpr;  // rows served per wavefront step
+  const int sub = lane / lpr, col = lane % lpr;
+  const bool single_chunk = gridDim.y == 1;
+
+  for (int64_t g0 = r0 + (int64_t)wave * 64; g0 < r1; g0 += (WG / 64) * 64) {
+    const int64_t myrow = g0 + lane;
+    int lab = -1;
+    if (myrow < r1) lab = labels[myrow] - k0;
+    const bool match = lab >= 0 && lab < nk;
+    if (match) atomicAdd(&cnt[lab], 1);
+    if (single_chunk) {
+      // dense: rows g0 .. g0+63 in steps of rps rows
+      for (int b = 0; b < 64; b += rps) {
+        const int src = b + sub;
+        const int l = __shfl(lab, src, 64);
+        const int64_t row = g0 + src;
+        if (l >= 0 && l < nk && row < r1)
+          add_row_slice<T, VEC>(sums + (size_t)l * d, X + row * (int64_t)d, col, lpr, d);
+      }
+    } else {
+      unsigned long long mask = __ballot(match);
+      while (mask) {
+        // take up to rps set bits; sub-group `sub` serves the sub-th of them
+        int src = -1;
+        unsigned long long m = mask;
+        for (int q = 0; q < rps; q++) {
+          if (!m) break;
+          const int b = __ffsll((long long)m) - 1;
+          if (q == sub) src = b;
+          m &= m - 1;
+        }
+        mask = m;
+        const int l = __shfl(lab, src < 0 ? 0 : src, 64);
+        if (src >= 0) {
+          const int64_t row = g0 + src;
+          add_row_slice<T, VEC>(sums + (size_t)l * d, X + row * (int64_t)d, col, lpr, d);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  T *dst = psums + ((size_t)blockIdx.x * k + k0) * d;
+  for (int e = tid; e < nk * d; e += WG) dst[e] = sums[e];
+  int *cdst = pcounts + (size_t)blockIdx.x * k + k0;
+  for (int c = tid; c < nk; c += WG) cdst[c] = cnt[c];
+}
+
+template <typename T>
+UpdatePlan plan_update(int64_t n, int d, int k, int num_cu) {
+  UpdatePlan p;
+  const size_t per_centroid = (size_t)d * sizeof(T) + sizeof(int);
+  const size_t budget = 64 * 1024;
+  int kc = (int)(budget / per_centroid);
+  if (kc < 1) kc = 1;
+  if (kc > k) kc = k;
+  p.kc = kc;
+  p.k_chunks = (k + kc - 1) / kc;
+  p.lds_bytes = (size_t)kc * per_centroid;
+  p.vec = 1;
+  if (sizeof(T) == 4 && d % 4 == 0) p.vec = 4;
+  else if (d % 2 == 0) p.vec = 2;
+  // enough workgroups to cover the machine a few times, but bounded so the
+  // partials buffer (row_blocks * k * d) stays small next to the data
+  int64_t want = (int64_t)num_cu * 4 / p.k_chunks;
+  if (want < 1) want = 1;
+  int64_t max_by_rows = (n + 1023) / 1024;  // at least 1024 rows per block
+  if (max_by_rows < 1) max_by_rows = 1;
+  if (want > max_by_rows) want = max_by_rows;
+  // partials traffic 2*rb*k*d should stay below ~1/8 of the data n*d
+  int64_t max_by_bytes = n / ((int64_t)16 * k);
+  if (max_by_bytes < 1) max_by_bytes = 1;
+  if (want > max_by_bytes) want = max_by_bytes;
+  p.row_blocks = (int)want;
+  return p;
+}
+
+template <typename T, int VEC>
+static int launch_accumulate_vec(hipStream_t s, const UpdatePlan &p, const T *X,
+                                 const int *labels, T *psums, int *pcounts,
+                                 int64_t n, int d, int k) {
+  const int64_t rows_per_block = ((n + p.row_blocks - 1) / p.row_blocks + 63) / 64 * 64;
+  int groups = (d + VEC - 1) / VEC;  // lanes wanted per row
+  int lpr = 1;
+  while (lpr < groups && lpr < 64) lpr <<= 1;
+  auto kern = accumulate_kernel<T, VEC>;
+  if (p.lds_bytes > 64 * 1024)
+    KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)p.lds_bytes));
+  hipLaunchKernelGGL(kern, dim3(p.row_blocks, p.k_chunks), dim3(WG), p.lds_bytes, s,
+                     X, labels, psums, pcounts, n, d, k, p.kc, rows_per_block, lpr);
+  KM_HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+template <>
+int launch_accumulate<float>(hipStream_t s, const UpdatePlan &p, const float *X,
+                             const int *labels, float *psums, int *pcounts,
+                             int64_t n, int d, int k) {
+  const bool aligned = (reinterpret_cast<uintptr_t>(X) & 15) == 0;
+  if (p.vec == 4 && aligned) return launch_accumulate_vec<float, 4>(s, p, X, labels, psums, pcounts, n, d, k);
+  if (p.vec >= 2 && aligned && d % 2 == 0) return launch_accumulate_vec<float, 2>(s, p, X, labels, psums, pcounts, n, d, k);
+  return launch_accumulate_vec<float, 1>(s, p, X, labels, psums, pcounts, n, d, k);
+}
+template <>
+int launch_accumulate<double>(hipStream_t s, const UpdatePlan &p, const double *X,
+                              const int *labels, double *psums, int *pcounts,
+                              int64_t n, int d, int k) {
+  const bool aligned = (reinterpret_cast<uintptr_t>(X) & 15) == 0;
+  if (p.vec >= 2 && aligned) return launch_accumulate_vec<double, 2>(s, p, X, labels, psums, pcounts, n, d, k);
+  return launch_accumulate_vec<double, 1>(s, p, X, labels, psums, pcounts, n, d, k);
+}
+
+// ---------------------------------------------------------------------------
+// pass 2: finalize. One thread per centroid coordinate.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(WG) void finalize_kernel(
+    const T *__restrict__ psums, const int *__restrict__ pcounts, int row_blocks,
+    const T *__restrict__ c_old, T *__restrict__ c_new, int *__restrict__ counts,
+    T *__restrict__ shift_partials, int d, int k) {
+#pragma clang fp contract(off)
+  __shared__ T red[WG];
+  const int tid = threadIdx.x;
+  const int64_t e = (int64_t)blockIdx.x * WG + tid;
+  const int64_t kd = (int64_t)k * d;
+  T diff2 = 0;
+  if (e < kd) {
+    const int c = (int)(e / d);
+    int cnt = 0;
+    T s = 0;
+    for (int rb = 0; rb < row_blocks; rb++) {
+      cnt += pcounts[(size_t)rb * k + c];
+      s = s + psums[(size_t)rb * kd + e];
+    }
+    const T oldv = c_old[e];
+    T newv;
+    if (cnt < 1) {
+      newv = oldv;  // revert_zeroed_centroids, kmeans_centroids.h:77-88
+    } else {
+      const T scale = (T)1.0 / (T)cnt;  // scale_centroids, kmeans_centroids.h:90-105
+      newv = s * scale;
+    }
+    c_new[e] = newv;
+    if (e - (int64_t)c * d == 0) counts[c] = cnt;
+    const T df = oldv - newv;
+    diff2 = df * df;
+  }
+  red[tid] = diff2;
+  __syncthreads();
+  for (int off = WG / 2; off > 0; off >>= 1) {
+    if (tid < off) red[tid] = red[tid] + red[tid + off];
+    __syncthreads();
+  }
+  if (tid == 0) shift_partials[blockIdx.x] = red[0];
+}
+
+template <typename T>
+int launch_finalize(hipStream_t s, const UpdatePlan &p, const T *psums,
+                    const int *pcounts, const T *c_old, T *c_new, int *counts,
+                    T *shift_partials, int *n_shift_partials, int d, int k) {
+  const int64_t kd = (int64_t)k * d;
+  const int blocks = (int)((kd + WG - 1) / WG);
+  hipLaunchKernelGGL((finalize_kernel<T>), dim3(blocks), dim3(WG), 0, s, psums,
+                     pcounts, p.row_blocks, c_old, c_new, counts, shift_partials, d, k);
+  KM_HIP_TRY(hipGetLastError());
+  *n_shift_partials = blocks;
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// pass 3: centroid norms + ordered sum of shift partials.
+// Blocks 0 .. ceil(k/WG)-1 compute norms; the last block sums the partials
+// with one wavefront in a fixed order.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(WG) void post_update_kernel(
+    const T *__restrict__ c_new, T *__restrict__ cnorm,
+    const T *__restrict__ shift_partials, int n_partials, T *__restrict__ shift2,
+    int d, int k) {
+#pragma clang fp contract(off)
+  const int tid = threadIdx.x;
+  if (blockIdx.x == gridDim.x - 1) {
+    __shared__ T red[WG];
+    T acc = 0;
+    for (int i = tid; i < n_partials; i += WG) acc = acc + shift_partials[i];
+    red[tid] = acc;
+    __syncthreads();
+    for (int off = WG / 2; off > 0; off >>= 1) {
+      if (tid < off) red[tid] = red[tid] + red[tid + off];
+      __syncthreads();
+    }
+    if (tid == 0) *shift2 = red[0];
+    return;
+  }
+  const int c = blockIdx.x * WG + tid;
+  if (c >= k) return;
+  const T *x = c_new + (size_t)c * d;
+  T acc = 0;
+  for (int j = 0; j < d; j++) {
+    const T v = x[j];
+    acc = acc + v * v;
+  }
+  cnorm[c] = acc;
+}
+
+template <typename T>
+int launch_post_update(hipStream_t s, const T *c_new, T *cnorm,
+                       const T *shift_partials, int n_shift_partials, T *shift2,
+                       int d, int k) {
+  const int blocks = (k + WG - 1) / WG + 1;
+  hipLaunchKernelGGL((post_update_kernel<T>), dim3(blocks), dim3(WG), 0, s, c_new,
+                     cnorm, shift_partials, n_shift_partials, shift2, d, k);
+  KM_HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Deterministic sum of n values in double: stage 1 gives every block a fixed
+// contiguous range and a fixed tree, stage 2 adds the block results in order.
+// ---------------------------------------------------------------------------
+static const int SUM_BLOCKS = 1024;
+int sum_partials_needed() { return SUM_BLOCKS; }
+
+template <typename T>
+__global__ __launch_bounds__(WG) void sum_stage1_kernel(const T *__restrict__ v,
+                                                       int64_t n,
+                                                       double *__restrict__ partials) {
+  __shared__ double red[WG];
+  const int tid = threadIdx.x;
+  const int64_t per = (n + gridDim.x - 1) / gridDim.x;
+  const int64_t lo = (int64_t)blockIdx.x * per;
+  const int64_t hi = min(n, lo + per);
+  double acc = 0;
+  for (int64_t i = lo + tid; i < hi; i += WG) acc += (double)v[i];
+  red[tid] = acc;
+  __syncthreads();
+  for (int off = WG / 2; off > 0; off >>= 1) {
+    if (tid < off) red[tid] += red[tid + off];
+    __syncthreads();
+  }
+  if (tid == 0) partials[blockIdx.x] = red[0];
+}
+__global__ __launch_bounds__(WG) void sum_stage2_kernel(const double *__restrict__ partials,
+                                                       int np, double *__restrict__ out) {
+  __shared__ double red[WG];
+  const int tid = threadIdx.x;
+  double acc = 0;
+  for (int i = tid; i < np; i += WG) acc += partials[i];
+  red[tid] = acc;
+  __syncthreads();
+  for (int off = WG / 2; off > 0; off >>= 1) {
+    if (tid < off) red[tid] += red[tid + off];
+    __syncthreads();
+  }
+  if (tid == 0) *out = red[0];
+}
+
+template <typename T>
+int launch_sum(hipStream_t s, const T *v, int64_t n, double *partials,
+               int n_partials, double *out) {
+  int blocks = n_partials < SUM_BLOCKS ? n_partials : SUM_BLOCKS;
+  if (blocks < 1) return H2O4GPU_KMEANS_EARG;
+  hipLaunchKernelGGL((sum_stage1_kernel<T>), dim3(blocks), dim3(WG), 0, s, v, n, partials);
+  hipLaunchKernelGGL(sum_stage2_kernel, dim3(1), dim3(WG), 0, s, partials, blocks, out);
+  KM_HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+template <typename T>
+__global__ void gather_rows_kernel(const T *__restrict__ X, const int *__restrict__ idx,
+                                   T *__restrict__ C, int k, int d) {
+  const int64_t e = (int64_t)blockIdx.x * WG + threadIdx.x;
+  if (e >= (int64_t)k * d) return;
+  const int c = (int)(e / d), j = (int)(e - (int64_t)c * d);
+  C[e] = X[(int64_t)idx[c] * d + j];
+}
+template <typename T>
+int launch_gather_rows(hipStream_t s, const T *X, const int *idx, T *C, int k, int d) {
+  const int64_t kd = (int64_t)k * d;
+  hipLaunchKernelGGL((gather_rows_kernel<T>), dim3((unsigned)((kd + WG - 1) / WG)),
+                     dim3(WG), 0, s, X, idx, C, k, d);
+  KM_HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+#define KM_INSTANTIATE(T)                                                            \
+  template int launch_row_norms<T>(hipStream_t, const T *, T *, int64_t, int);       \
+  template UpdatePlan plan_update<T>(int64_t, int, int, int);                        \
+  template int launch_finalize<T>(hipStream_t, const UpdatePlan &, const T *,        \
+                                  const int *, const T *, T *, int *, T *, int *,    \
+                                  int, int);                                         \
+  template int launch_post_update<T>(hipStream_t, const T *, T *, const T *, int,    \
+                                     T *, int, int);                                 \
+  template int launch_sum<T>(hipStream_t, const T *, int64_t, double *, int,         \
+                             double *);                                              \
+  template int launch_gather_rows<T>(hipStream_t, const T *, const int *, T *, int,  \
+                                     int);
+KM_INSTANTIATE(float)
+KM_INSTANTIATE(double)
+
+}  // namespace kmhip

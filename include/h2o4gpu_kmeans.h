@@ -1,0 +1,187 @@
+/*
+ * C ABI of the MI355X (gfx950) k-means engine, libh2o4gpu_kmeans_hip.so.
+ *
+ * Part 1 are the entry points h2o4gpu's language bindings already call for
+ * k-means; a binding built against this header works unchanged. Part 2 is the
+ * small device-information surface the Python estimator touches before it
+ * fits. Part 3 is a handle API that keeps the data set resident in HBM between
+ * calls (the reference has no counterpart; it re-uploads on every call).
+ *
+ * All pointers are plain host pointers unless a parameter is named d_*.
+ * Matrices are dense, row-major, contiguous. Every function returns 0 on
+ * success and a negative code on failure (no exit(), no exceptions).
+ */
+#ifndef H2O4GPU_KMEANS_H
+#define H2O4GPU_KMEANS_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* error codes */
+#define H2O4GPU_KMEANS_OK 0
+#define H2O4GPU_KMEANS_EALLOC (-1)   /* allocation failed (the reference's -1) */
+#define H2O4GPU_KMEANS_EARG (-2)     /* bad argument */
+#define H2O4GPU_KMEANS_EDEVICE (-3)  /* HIP runtime error / no usable device */
+#define H2O4GPU_KMEANS_ESTATE (-4)   /* call order (e.g. fit before data) */
+
+/* ---------------------------------------------------------------------------
+ * Part 1 - drop-in entry points.
+ * Replaces: src/include/solver/kmeans.h:56-76 (declarations),
+ *           src/gpu/kmeans/kmeans_h2o4gpu.cu:1060-1097 (definitions).
+ *
+ * dopredict == 0: fit.   srcdata [mTrain][n]; result buffers are allocated
+ *   with malloc() and handed to the caller through *pred_centroids ([k][n])
+ *   and *pred_labels ([mTrain] int32); the caller owns them.
+ *   init_from_data: 0 = seeded random distinct rows (std::shuffle with
+ *   std::default_random_engine(seed), as the reference), 1 = k-means++
+ *   seeding on the device, 2 = start from `centroids` ([k][n], extension:
+ *   the reference ignores `centroids` when fitting).
+ *   threshold: absolute bound on sum((C_old - C_new)^2); the loop stops when
+ *   the sum is below it. Exactly as the reference, a run of N iterations
+ *   makes N centroid updates and N+1 assignment passes, the last one with the
+ *   final centroids.
+ * dopredict != 0: predict. Labels of srcdata against `centroids`; only
+ *   *pred_labels is set.
+ * gpu_id selects the device as (gpu_id mod visible devices); n_gpu is
+ * accepted for compatibility, one device is used.
+ * If k > mTrain, k is clamped to mTrain (message on stderr) as in the reference.
+ * ------------------------------------------------------------------------- */
+int make_ptr_float_kmeans(int dopredict, int verbose, int seed, int gpu_id,
+                          int n_gpu, size_t mTrain, size_t n, int k,
+                          int max_iterations, int init_from_data,
+                          float threshold, const float *srcdata,
+                          const float *centroids, float **pred_centroids,
+                          int **pred_labels);
+
+int make_ptr_double_kmeans(int dopredict, int verbose, int seed, int gpu_id,
+                           int n_gpu, size_t mTrain, size_t n, int k,
+                           int max_iterations, int init_from_data,
+                           double threshold, const double *srcdata,
+                           const double *centroids, double **pred_centroids,
+                           int **pred_labels);
+
+/* Squared distances |xx + cc - 2 x.c| of every row to every centroid, no
+ * sqrt, centroid-major: (*preds)[c * m + i]. malloc()ed, caller owns.
+ * Replaces: kmeans_transform<T>, src/gpu/kmeans/kmeans_h2o4gpu.cu:891-975. */
+int kmeans_transform_float(int verbose, int gpu_id, int n_gpu, size_t m,
+                           size_t n, int k, const float *srcdata,
+                           const float *centroids, float **preds);
+
+int kmeans_transform_double(int verbose, int gpu_id, int n_gpu, size_t m,
+                            size_t n, int k, const double *srcdata,
+                            const double *centroids, double **preds);
+
+/* ---------------------------------------------------------------------------
+ * Part 2 - device information used by the estimator's constructor.
+ * Replaces: get_gpu_info_c, src/gpu/utils.cu:57-304 (NVML based; argument
+ * list kept, see src/swig/util/gpu.i:64-93), get_compute_capability
+ * (src/gpu/utils.cu:40-55), cudaresetdevice / cudaresetdevice_bare.
+ * Arrays must hold at least *n_gpus entries; per-process usage arrays are
+ * zero-filled (ROCm has no NVML process table here). Returns 0, or 1 when no
+ * device is visible (as the reference does when NVML fails).
+ * ------------------------------------------------------------------------- */
+int get_gpu_info_c(int verbose, int return_memory, int return_name,
+                   int return_usage, int return_free_memory,
+                   int return_capability, int return_memory_by_pid,
+                   int return_usage_by_pid, int return_all,
+                   unsigned int *n_gpus, int *gpu_percent_usage,
+                   unsigned long long *gpu_total_memory,
+                   unsigned long long *gpu_free_memory, char **gpu_name,
+                   int *majors, int *minors, unsigned int *num_pids,
+                   unsigned int *pids, unsigned long long *usedGpuMemorys,
+                   unsigned int *num_pids_usage, unsigned int *pids_usage,
+                   unsigned long long *usedGpuUsage);
+int get_compute_capability(int d_idx, int *major, int *minor, int *ratioperf);
+int cudaresetdevice(int wDev, int nDev);
+int cudaresetdevice_bare(void);
+/* Number of visible HIP devices (0 if the runtime cannot be initialised). */
+int h2o4gpu_kmeans_device_count(void);
+
+/* ---------------------------------------------------------------------------
+ * Part 3 - resident-data handle API (no counterpart in the reference).
+ * One handle = one data set [rows][cols] of one precision on one device plus
+ * the working set of a k-cluster model. Calls on one handle are serialised by
+ * the caller; different handles are independent.
+ * ------------------------------------------------------------------------- */
+typedef struct h2o4gpu_kmeans_handle h2o4gpu_kmeans_handle;
+
+/* elem_size: 4 = float, 8 = double. */
+int h2o4gpu_kmeans_create(h2o4gpu_kmeans_handle **out, int elem_size,
+                          size_t rows, size_t cols, int k, int gpu_id,
+                          int verbose);
+int h2o4gpu_kmeans_destroy(h2o4gpu_kmeans_handle *h);
+
+/* Upload rows from host memory (copies) / adopt a device pointer (no copy,
+ * caller keeps it alive). Row norms are computed on the device either way. */
+int h2o4gpu_kmeans_set_data_host(h2o4gpu_kmeans_handle *h, const void *X);
+int h2o4gpu_kmeans_set_data_device(h2o4gpu_kmeans_handle *h, const void *d_X);
+
+/* Initial centroids: given ([k][cols] host), seeded random distinct rows
+ * (the reference's std::shuffle rule), or k-means++ on the device. */
+int h2o4gpu_kmeans_set_centroids_host(h2o4gpu_kmeans_handle *h, const void *C);
+int h2o4gpu_kmeans_init_random_rows(h2o4gpu_kmeans_handle *h, int seed);
+int h2o4gpu_kmeans_init_plusplus(h2o4gpu_kmeans_handle *h, int seed);
+
+/* The reference's loop (kmeans_impl.h:109-232): up to max_iterations of
+ * assign + update, stop when shift^2 < threshold, final assignment with the
+ * final centroids. *iterations_run receives the number of centroid updates. */
+int h2o4gpu_kmeans_fit(h2o4gpu_kmeans_handle *h, int max_iterations,
+                       double threshold, int *iterations_run);
+
+/* Single steps (for lock-step checks and custom loops). assign: labels (and
+ * per-row minimum squared distance) against the current centroids. update:
+ * centroids <- per-label means of the current labels (empty clusters keep
+ * their centroid); *shift2 (may be NULL) = sum((C_old - C_new)^2). */
+int h2o4gpu_kmeans_assign(h2o4gpu_kmeans_handle *h);
+int h2o4gpu_kmeans_update(h2o4gpu_kmeans_handle *h, double *shift2);
+int h2o4gpu_kmeans_set_labels_host(h2o4gpu_kmeans_handle *h, const int *labels);
+
+/* Results to host memory. */
+int h2o4gpu_kmeans_get_centroids(h2o4gpu_kmeans_handle *h, void *C);
+int h2o4gpu_kmeans_get_labels(h2o4gpu_kmeans_handle *h, int *labels);
+int h2o4gpu_kmeans_get_counts(h2o4gpu_kmeans_handle *h, int *counts);
+int h2o4gpu_kmeans_get_min_distances(h2o4gpu_kmeans_handle *h, void *mind);
+/* Sum over rows of the minimum squared distance found by the last assign. */
+int h2o4gpu_kmeans_inertia(h2o4gpu_kmeans_handle *h, double *inertia);
+
+/* Labels / squared distances of other rows against the handle's centroids.
+ * X: [rows][cols] host memory. dist: [k][rows] host memory. */
+int h2o4gpu_kmeans_predict_host(h2o4gpu_kmeans_handle *h, size_t rows,
+                                const void *X, int *labels);
+int h2o4gpu_kmeans_transform_host(h2o4gpu_kmeans_handle *h, size_t rows,
+                                  const void *X, void *dist);
+/* Same on the handle's own resident rows, output left on the device:
+ * d_dist [k][rows] device memory provided by the caller. */
+int h2o4gpu_kmeans_transform_resident(h2o4gpu_kmeans_handle *h, void *d_dist);
+
+/* Kernel selection: "assign" = 0 auto, 1 VALU, 2 MFMA row-stationary,
+ * 3 MFMA tiled; "update" = 0 auto. Unknown names return EARG. */
+int h2o4gpu_kmeans_set_option(h2o4gpu_kmeans_handle *h, const char *name,
+                              int value);
+
+/* Timing on the handle's stream with HIP events. timer_start/timer_stop
+ * bracket any sequence of calls; with kernel profiling on, every kernel launch
+ * is bracketed by its own event pair and kernel_time() returns the launch count
+ * and summed milliseconds since profiling was switched on, by kernel name
+ * ("assign", "accumulate", "finalize", "row_norms", "transform", ...). */
+int h2o4gpu_kmeans_timer_start(h2o4gpu_kmeans_handle *h);
+int h2o4gpu_kmeans_timer_stop(h2o4gpu_kmeans_handle *h, float *milliseconds);
+int h2o4gpu_kmeans_profile(h2o4gpu_kmeans_handle *h, int on);
+int h2o4gpu_kmeans_kernel_time(h2o4gpu_kmeans_handle *h, const char *kernel,
+                               int *launches, double *milliseconds);
+/* Name of the assign kernel variant the handle's shape dispatches to. */
+const char *h2o4gpu_kmeans_assign_variant(h2o4gpu_kmeans_handle *h);
+
+/* Device-to-device copy bandwidth probe: copies `bytes` from one scratch
+ * buffer to another `reps` times and returns the average milliseconds of one
+ * copy (used to calibrate byte counters and to report achievable HBM rate). */
+int h2o4gpu_kmeans_copy_probe(int gpu_id, size_t bytes, int reps,
+                              float *milliseconds);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* H2O4GPU_KMEANS_H */

@@ -1,0 +1,410 @@
+// TEST INFRASTRUCTURE ONLY -- CPU restatement of the k-means (Lloyd) path of
+// h2oai/h2o4gpu, used as the parity checker and as the CPU baseline in the
+// benchmark. Nothing in the shipped engine (h2o4gpu_amd/) links, loads or
+// calls this file.
+//
+// Every function cites the reference text it restates (paths relative to the
+// reference checkout). Arithmetic is done in T (float or double) with
+// floating-point contraction switched off at build time, so a sum written
+// "a*b + c" is a rounded multiply followed by a rounded add.
+//
+// Pinning status (what independent evidence fixes each function):
+//   row_norms, distances, assign  : brute-force float64 closed form on tiny
+//       inputs, D(x,x)=0 after fabs, tie rule, the reference's gtest
+//       known-answer cases CountsPerCentroids / CentroidPerDataPoint.
+//   update                        : the reference's gtest cases
+//       CalculateCentroids, CalculateCentroids2GPU (shard additivity),
+//       RevertCentroidZeroing, CentroidsScaling; mass invariants.
+//   lloyd                         : k=1 closed form, k=n fixed point, an
+//       independent Lloyd implementation (scikit-learn, explicit init) on
+//       data without empty clusters, labels == argmin against final centroids.
+//   random_rows                   : the two standard-library calls the
+//       reference makes, compiled as written; distinctness, determinism.
+//   transform                     : scipy cdist(sqeuclidean), transposed.
+//   kmeanspp_*                    : parity unpinned against the reference (the
+//       reference seeds with k-means|| whose candidate stream needs a CUDA
+//       build); pinned only against the textbook D^2-sampling definition.
+//
+// Build: make -C oracle   (g++ -O3 -fopenmp -ffp-contract=off)
+
+#include <algorithm>
+#include <cfloat>
+#include <cmath>
+#include <cstdint>
+#include <cstdlib>
+#include <cstring>
+#include <limits>
+#include <numeric>
+#include <random>
+#include <vector>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+namespace {
+
+// ---------------------------------------------------------------------------
+// self_dots: dots[i] = sum_j data[i,j]^2, accumulated in T, j ascending.
+// Reference: src/gpu/kmeans/kmeans_labels.h:187-199.
+// ---------------------------------------------------------------------------
+template <typename T>
+void row_norms(int64_t n, int d, const T *X, T *out, int threads) {
+#pragma omp parallel for num_threads(threads) schedule(static)
+  for (int64_t i = 0; i < n; i++) {
+    T acc = 0;
+    const T *x = X + i * (int64_t)d;
+    for (int j = 0; j < d; j++) {
+      T v = x[j];
+      acc += v * v;
+    }
+    out[i] = acc;
+  }
+}
+
+// Centroids transposed to [d][kp] so the inner loop runs over centroids while
+// each (row, centroid) dot product is still summed over j in ascending order.
+template <typename T>
+std::vector<T> transpose_centroids(int d, int k, const T *C) {
+  std::vector<T> Ct((size_t)d * k);
+  for (int c = 0; c < k; c++)
+    for (int j = 0; j < d; j++) Ct[(size_t)j * k + c] = C[(size_t)c * d + j];
+  return Ct;
+}
+
+// dist(row, c) = | (xx + cc[c]) - 2 * dot(x, C[c]) |
+// Reference: all_dots writes xx + cc (kmeans_labels.h:216-244); the GEMM then
+// forms alpha*dot + beta*D with alpha=-2, beta=1 (kmeans_labels.cu:183-228);
+// absolute_value is applied in place (kmeans_labels.cu:236-239).
+// The summation order inside the reference's GEMM is a cuBLAS internal; this
+// restatement uses j ascending.
+template <typename T>
+__attribute__((target_clones("avx2", "default"))) void
+dist_row(int d, int k, const T *x, T xx, const T *Ct, const T *cc, T *acc) {
+  for (int c = 0; c < k; c++) acc[c] = 0;
+  for (int j = 0; j < d; j++) {
+    const T xj = x[j];
+    const T *ct = Ct + (size_t)j * k;
+    for (int c = 0; c < k; c++) acc[c] += xj * ct[c];
+  }
+  for (int c = 0; c < k; c++) {
+    T t = xx + cc[c];
+    T v = t - (T)2 * acc[c];
+    acc[c] = std::fabs(v);
+  }
+}
+
+// argmin with the reference's rule: running minimum starts at FLT_MAX (also for
+// double), strict '<', first (lowest) index wins, index -1 if nothing is below
+// the start value. Reference: kmeans_labels.h:360-377.
+template <typename T>
+inline int argmin_row(int k, const T *dist, T *best_out) {
+  T best = (T)FLT_MAX;
+  int idx = -1;
+  for (int c = 0; c < k; c++) {
+    if (dist[c] < best) {
+      best = dist[c];
+      idx = c;
+    }
+  }
+  if (best_out) *best_out = best;
+  return idx;
+}
+
+template <typename T>
+void assign(int64_t n, int d, int k, const T *X, const T *C, int *labels,
+            T *mindist, int threads) {
+  std::vector<T> Ct = transpose_centroids(d, k, C);
+  std::vector<T> cc(k);
+  row_norms<T>(k, d, C, cc.data(), 1);
+#pragma omp parallel num_threads(threads)
+  {
+    std::vector<T> acc(k);
+#pragma omp for schedule(static)
+    for (int64_t i = 0; i < n; i++) {
+      const T *x = X + i * (int64_t)d;
+      T xx = 0;
+      for (int j = 0; j < d; j++) xx += x[j] * x[j];
+      dist_row<T>(d, k, x, xx, Ct.data(), cc.data(), acc.data());
+      T best;
+      labels[i] = argmin_row<T>(k, acc.data(), &best);
+      if (mindist) mindist[i] = best;
+    }
+  }
+}
+
+// Full distance matrix, centroid-major [k][n] (index c*n + i), squared
+// distances, no sqrt. Reference: kmeans_transform, kmeans_h2o4gpu.cu:891-975;
+// layout kmeans_labels.h:241.
+template <typename T>
+void distances(int64_t n, int d, int k, const T *X, const T *C, T *D,
+               int threads) {
+  std::vector<T> Ct = transpose_centroids(d, k, C);
+  std::vector<T> cc(k);
+  row_norms<T>(k, d, C, cc.data(), 1);
+#pragma omp parallel num_threads(threads)
+  {
+    std::vector<T> acc(k);
+#pragma omp for schedule(static)
+    for (int64_t i = 0; i < n; i++) {
+      const T *x = X + i * (int64_t)d;
+      T xx = 0;
+      for (int j = 0; j < d; j++) xx += x[j] * x[j];
+      dist_row<T>(d, k, x, xx, Ct.data(), cc.data(), acc.data());
+      for (int c = 0; c < k; c++) D[(size_t)c * n + i] = acc[c];
+    }
+  }
+}
+
+// Centroid update. Reference: find_centroids, kmeans_centroids.h:108-189:
+//   keep a copy of the old centroids, zero sums and counts, add every row to
+//   the sum of its label (calculate_centroids :40-75), restore the old
+//   centroid where count < 1 (revert_zeroed_centroids :77-88), multiply by
+//   1/T(max(count,1)) (scale_centroids :90-105; reciprocal then multiply).
+// The reference adds with floating-point atomics in no fixed order; this
+// restatement adds rows in ascending row order. With several threads each
+// thread sums a contiguous block of rows and blocks are combined in thread
+// order. Rows with a negative label are skipped.
+template <typename T>
+void update_sums(int64_t n, int d, int k, const T *X, const int *labels,
+                 T *sums, int *counts, int threads) {
+  std::fill(sums, sums + (size_t)k * d, (T)0);
+  std::fill(counts, counts + k, 0);
+  if (threads <= 1) {
+    for (int64_t i = 0; i < n; i++) {
+      int l = labels[i];
+      if (l < 0 || l >= k) continue;
+      counts[l]++;
+      T *s = sums + (size_t)l * d;
+      const T *x = X + i * (int64_t)d;
+      for (int j = 0; j < d; j++) s[j] += x[j];
+    }
+    return;
+  }
+  std::vector<std::vector<T>> psum(threads);
+  std::vector<std::vector<int>> pcnt(threads);
+#pragma omp parallel num_threads(threads)
+  {
+    int t = 0, nt = 1;
+#ifdef _OPENMP
+    t = omp_get_thread_num();
+    nt = omp_get_num_threads();
+#endif
+    psum[t].assign((size_t)k * d, (T)0);
+    pcnt[t].assign(k, 0);
+    int64_t lo = n * t / nt, hi = n * (t + 1) / nt;
+    for (int64_t i = lo; i < hi; i++) {
+      int l = labels[i];
+      if (l < 0 || l >= k) continue;
+      pcnt[t][l]++;
+      T *s = psum[t].data() + (size_t)l * d;
+      const T *x = X + i * (int64_t)d;
+      for (int j = 0; j < d; j++) s[j] += x[j];
+    }
+  }
+  for (int t = 0; t < threads; t++) {
+    if (psum[t].empty()) continue;
+    for (size_t e = 0; e < (size_t)k * d; e++) sums[e] += psum[t][e];
+    for (int c = 0; c < k; c++) counts[c] += pcnt[t][c];
+  }
+}
+
+template <typename T>
+void finalize_centroids(int d, int k, const T *sums, const int *counts,
+                        const T *old_c, T *new_c) {
+  for (int c = 0; c < k; c++) {
+    int count = counts[c];
+    if (count < 1) {
+      for (int j = 0; j < d; j++) new_c[(size_t)c * d + j] = old_c[(size_t)c * d + j];
+      // scale_centroids multiplies by 1/T(1) == 1 here: value unchanged.
+    } else {
+      T scale = (T)1.0 / (T)count;
+      for (int j = 0; j < d; j++) new_c[(size_t)c * d + j] = sums[(size_t)c * d + j] * scale;
+    }
+  }
+}
+
+template <typename T>
+void update(int64_t n, int d, int k, const T *X, const int *labels, T *C,
+            int *counts, int threads) {
+  std::vector<T> old_c(C, C + (size_t)k * d);
+  std::vector<T> sums((size_t)k * d);
+  update_sums<T>(n, d, k, X, labels, sums.data(), counts, threads);
+  finalize_centroids<T>(d, k, sums.data(), counts, old_c.data(), C);
+}
+
+// The Lloyd loop. Reference: kmeans::kmeans, kmeans_impl.h:109-232.
+//   for i in [0, max_iterations): old = C; relabel; update; shift2 = sum
+//   (old-new)^2 accumulated in T; done = shift2 < threshold (threshold is held
+//   as double there); if done or last iteration: relabel once more with the
+//   final centroids and stop. Returns i as the reference does (the index of
+//   the iteration at which the loop was left; max_iterations-1 when it ran
+//   to the end, max_iterations if max_iterations <= 0).
+template <typename T>
+int lloyd(int64_t n, int d, int k, const T *X, T *C, int *labels,
+          int max_iterations, double threshold, int threads, double *shift_hist) {
+  std::vector<T> old_c((size_t)k * d);
+  std::vector<int> counts(k);
+  int i = 0;
+  for (; i < max_iterations; i++) {
+    std::copy(C, C + (size_t)k * d, old_c.begin());
+    assign<T>(n, d, k, X, C, labels, nullptr, threads);
+    update<T>(n, d, k, X, labels, C, counts.data(), threads);
+    T shift2 = 0;
+    for (size_t e = 0; e < (size_t)k * d; e++) {
+      T diff = old_c[e] - C[e];
+      shift2 += diff * diff;
+    }
+    if (shift_hist) shift_hist[i] = (double)shift2;
+    bool done = (double)shift2 < threshold;
+    if (done || i == max_iterations - 1) {
+      assign<T>(n, d, k, X, C, labels, nullptr, threads);
+      break;
+    }
+  }
+  return i;
+}
+
+// Exact squared distances ||x - c||^2 in double, direct form (no expansion),
+// returning best index, best and second-best value per row: used by the tests
+// to decide whether a label mismatch sits on a near-tie. Not part of the
+// reference; mathematics only.
+template <typename T>
+void top2_exact(int64_t n, int d, int k, const T *X, const T *C, int *best_idx,
+                double *d1, double *d2, int threads) {
+#pragma omp parallel for num_threads(threads) schedule(static)
+  for (int64_t i = 0; i < n; i++) {
+    const T *x = X + i * (int64_t)d;
+    double b1 = std::numeric_limits<double>::infinity(), b2 = b1;
+    int bi = -1;
+    for (int c = 0; c < k; c++) {
+      const T *cp = C + (size_t)c * d;
+      double s = 0;
+      for (int j = 0; j < d; j++) {
+        double df = (double)x[j] - (double)cp[j];
+        s += df * df;
+      }
+      if (s < b1) {
+        b2 = b1;
+        b1 = s;
+        bi = c;
+      } else if (s < b2) {
+        b2 = s;
+      }
+    }
+    best_idx[i] = bi;
+    d1[i] = b1;
+    d2[i] = b2;
+  }
+}
+
+// Exact squared distance of every row to two given centroids per row
+// (labels a[i], b[i]) in double: lets a test price a mismatch without a full
+// n*k pass.
+template <typename T>
+void pair_dist_exact(int64_t n, int d, const T *X, const T *C, const int *a,
+                     const int *b, double *da, double *db, int threads) {
+#pragma omp parallel for num_threads(threads) schedule(static)
+  for (int64_t i = 0; i < n; i++) {
+    const T *x = X + i * (int64_t)d;
+    const T *ca = C + (size_t)a[i] * d;
+    const T *cb = C + (size_t)b[i] * d;
+    double sa = 0, sb = 0;
+    for (int j = 0; j < d; j++) {
+      double u = (double)x[j] - (double)ca[j];
+      double v = (double)x[j] - (double)cb[j];
+      sa += u * u;
+      sb += v * v;
+    }
+    da[i] = sa;
+    db[i] = sb;
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+#define ORACLE_EXPORT __attribute__((visibility("default")))
+
+ORACLE_EXPORT int oracle_max_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
+#define DEFINE_FOR(T, SUF)                                                        \
+  ORACLE_EXPORT void oracle_row_norms_##SUF(int64_t n, int d, const T *X, T *out, \
+                                            int threads) {                        \
+    row_norms<T>(n, d, X, out, threads);                                          \
+  }                                                                               \
+  ORACLE_EXPORT void oracle_assign_##SUF(int64_t n, int d, int k, const T *X,     \
+                                         const T *C, int *labels, T *mindist,     \
+                                         int threads) {                           \
+    assign<T>(n, d, k, X, C, labels, mindist, threads);                           \
+  }                                                                               \
+  ORACLE_EXPORT void oracle_distances_##SUF(int64_t n, int d, int k, const T *X,  \
+                                            const T *C, T *D, int threads) {      \
+    distances<T>(n, d, k, X, C, D, threads);                                      \
+  }                                                                               \
+  ORACLE_EXPORT void oracle_update_sums_##SUF(int64_t n, int d, int k,            \
+                                              const T *X, const int *labels,      \
+                                              T *sums, int *counts,               \
+                                              int threads) {                      \
+    update_sums<T>(n, d, k, X, labels, sums, counts, threads);                    \
+  }                                                                               \
+  ORACLE_EXPORT void oracle_finalize_##SUF(int d, int k, const T *sums,           \
+                                           const int *counts, const T *old_c,     \
+                                           T *new_c) {                            \
+    finalize_centroids<T>(d, k, sums, counts, old_c, new_c);                      \
+  }                                                                               \
+  ORACLE_EXPORT void oracle_update_##SUF(int64_t n, int d, int k, const T *X,     \
+                                         const int *labels, T *C, int *counts,    \
+                                         int threads) {                           \
+    update<T>(n, d, k, X, labels, C, counts, threads);                            \
+  }                                                                               \
+  ORACLE_EXPORT int oracle_lloyd_##SUF(int64_t n, int d, int k, const T *X, T *C, \
+                                       int *labels, int max_iterations,           \
+                                       double threshold, int threads,             \
+                                       double *shift_hist) {                      \
+    return lloyd<T>(n, d, k, X, C, labels, max_iterations, threshold, threads,    \
+                    shift_hist);                                                  \
+  }                                                                               \
+  ORACLE_EXPORT void oracle_top2_exact_##SUF(int64_t n, int d, int k, const T *X, \
+                                             const T *C, int *best, double *d1,   \
+                                             double *d2, int threads) {           \
+    top2_exact<T>(n, d, k, X, C, best, d1, d2, threads);                          \
+  }                                                                               \
+  ORACLE_EXPORT void oracle_pair_dist_exact_##SUF(                                \
+      int64_t n, int d, const T *X, const T *C, const int *a, const int *b,       \
+      double *da, double *db, int threads) {                                      \
+    pair_dist_exact<T>(n, d, X, C, a, b, da, db, threads);                        \
+  }
+
+DEFINE_FOR(float, f32)
+DEFINE_FOR(double, f64)
+
+// Seeded random-row initialisation: a permutation of 0..n-1 by
+// std::shuffle(v.begin(), v.end(), std::default_random_engine(seed)); the
+// initial centroids are rows v[0..k-1]. These are the two standard-library
+// calls the reference makes (kmeans_h2o4gpu.cu:662-669, rows taken at :79-84
+// and :692-693); the permutation depends on the C++ standard library in use.
+ORACLE_EXPORT void oracle_random_rows(int seed, int64_t n, int k, int *idx_out) {
+  std::vector<int> v((size_t)n);
+  std::iota(v.begin(), v.end(), 0);
+  std::shuffle(v.begin(), v.end(), std::default_random_engine(seed));
+  for (int c = 0; c < k; c++) idx_out[c] = v[c];
+}
+
+// First k-means++ centre: std::mt19937 gen(seed); uniform_int_distribution<>
+// dis(0, rows-1); dis(gen). Reference: kmeans_parallel picks its first centre
+// this way (kmeans_h2o4gpu.cu:343-347).
+ORACLE_EXPORT int oracle_kmeanspp_first(int seed, int64_t n) {
+  std::mt19937 gen(seed);
+  std::uniform_int_distribution<> dis(0, (int)(n - 1));
+  return dis(gen);
+}
+
+}  // extern "C"

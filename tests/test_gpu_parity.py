@@ -1,0 +1,137 @@
+"""GPU parity: every kernel of the engine against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+
+from parity import assert_centroids_close, label_report
+
+pytestmark = pytest.mark.gpu
+
+RNG = np.random.default_rng(20240607)
+
+
+def blobs(n, d, k, dtype, spread=5.0, sigma=1.0, seed=0):
+    rng = np.random.default_rng(seed)
+    centers = rng.uniform(-spread, spread, size=(k, d))
+    lab = rng.integers(0, k, size=n)
+    X = centers[lab] + sigma * rng.standard_normal((n, d))
+    return np.ascontiguousarray(X.astype(dtype))
+
+
+ASSIGN_CASES = [
+    # (n, d, k) covering padding of rows, features and centroids in every variant
+    (1000, 16, 8), (777, 5, 3), (4096, 32, 256), (5000, 32, 100), (3001, 64, 64),
+    (2000, 24, 33), (1500, 128, 40), (2500, 100, 70), (1200, 256, 130), (900, 300, 257),
+    (64, 8, 64), (1, 4, 1), (130, 2, 2),
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("variant", ["valu", "mfma_rowstat", "mfma_tiled"])
+@pytest.mark.parametrize("n,d,k", ASSIGN_CASES)
+def test_assign_matches_oracle(hip, oracle, n, d, k, variant, dtype):
+    X = blobs(n, d, max(k, 2), dtype, seed=n + d + k)
+    C = np.ascontiguousarray(X[RNG.choice(n, size=k, replace=False)]) if k <= n else None
+    with hip.Handle(n, d, k, dtype) as h:
+        h.set_data(X)
+        h.set_centroids(C)
+        try:
+            h.set_option("assign", variant)
+        except hip.KMeansHipError:
+            pytest.skip("variant not available")
+        if h.assign_variant() == "unsupported":
+            pytest.skip("shape outside %s" % variant)
+        h.assign()
+        got = h.labels()
+        mind = h.min_distances()
+    want, wmind = oracle.assign(X, C, return_mindist=True)
+    if variant == "valu":
+        # same association as the scalar loop: bit-exact
+        assert np.array_equal(got, want)
+        assert np.array_equal(mind, wmind)
+    else:
+        rep = label_report(oracle, X, C, got, want)
+        scale = (X.astype(np.float64) ** 2).sum(1).max() + (C.astype(np.float64) ** 2).sum(1).max()
+        eps = np.finfo(dtype).eps
+        assert np.max(np.abs(mind.astype(np.float64) - wmind)) <= 4 * np.sqrt(d) * eps * scale
+        print("assign %s %s n=%d d=%d k=%d: %s" % (variant, np.dtype(dtype).name, n, d, k, rep))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n,d,k", [(5000, 32, 256), (3000, 16, 8), (2000, 7, 5), (4000, 256, 300),
+                                   (1000, 784, 130), (70000, 64, 64), (300, 3, 300)])
+def test_update_matches_oracle(hip, oracle, n, d, k, dtype):
+    X = blobs(n, d, k, dtype, seed=7 * n + k)
+    C = np.ascontiguousarray(X[RNG.choice(n, size=k, replace=False)])
+    labels = RNG.integers(0, k, size=n).astype(np.int32)
+    labels[labels == 1] = 0  # cluster 1 empty: must keep its old centroid
+    with hip.Handle(n, d, k, dtype) as h:
+        h.set_data(X)
+        h.set_centroids(C)
+        h.set_labels(labels)
+        shift2 = h.update()
+        got = h.centroids()
+        counts = h.counts()
+    want, wcounts = oracle.update(X, labels, C)
+    assert np.array_equal(counts, wcounts)
+    if k > 1:
+        assert np.array_equal(got[1], C[1])
+    tol = 1e-5 if dtype == np.float32 else 1e-12
+    assert np.allclose(got, want, rtol=tol, atol=tol * np.abs(want).max())
+    ws2 = ((C.astype(np.float64) - want.astype(np.float64)) ** 2).sum()
+    assert abs(shift2 - ws2) <= 1e-4 * ws2 + 1e-30
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("variant", ["auto", "mfma_rowstat", "mfma_tiled"])
+def test_lloyd_end_to_end(hip, oracle, variant, dtype):
+    n, d, k, iters = 20000, 32, 40, 12
+    X = blobs(n, d, k, dtype, spread=10.0, seed=5)
+    C0 = np.ascontiguousarray(X[RNG.choice(n, size=k, replace=False)])
+    with hip.Handle(n, d, k, dtype) as h:
+        h.set_data(X)
+        h.set_centroids(C0)
+        h.set_option("assign", variant)
+        done = h.fit(iters, 0.0)
+        C = h.centroids()
+        labels = h.labels()
+    assert done == iters
+    wC, wlabels, it, _ = oracle.lloyd(X, C0, iters, 0.0, threads=4)
+    assert it == iters - 1
+    assert_centroids_close(C, wC, dtype)
+    rep = label_report(oracle, X, wC, labels, wlabels)
+    print("lloyd %s %s: %s" % (variant, np.dtype(dtype).name, rep))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_threshold_stop(hip, oracle, dtype):
+    n, d, k = 6000, 8, 5
+    # one start per blob (true centre + offset): no blob is split, so no row sits
+    # on a boundary and a last-bit difference cannot flip a label
+    rng = np.random.default_rng(11)
+    centers = rng.uniform(-20.0, 20.0, size=(k, d))
+    X = np.ascontiguousarray((centers[rng.integers(0, k, size=n)] + rng.standard_normal((n, d))).astype(dtype))
+    C0 = np.ascontiguousarray((centers + 0.5).astype(dtype))
+    thr = 1e-3
+    with hip.Handle(n, d, k, dtype) as h:
+        h.set_data(X)
+        h.set_centroids(C0)
+        done = h.fit(200, thr)
+        C = h.centroids()
+    wC, _, it, hist = oracle.lloyd(X, C0, 200, thr, threads=2)
+    assert done == it + 1 and done < 200
+    assert_centroids_close(C, wC, dtype)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n,d,k", [(1000, 16, 8), (3000, 64, 70), (700, 300, 130), (129, 5, 17)])
+def test_transform_matches_oracle(hip, oracle, n, d, k, dtype):
+    X = blobs(n, d, k, dtype, seed=n)
+    C = np.ascontiguousarray(X[RNG.choice(n, size=k, replace=False)])
+    with hip.Handle(k, d, k, dtype) as h:
+        h.set_centroids(C)
+        got = h.transform(X)
+    want = oracle.distances(X, C, threads=2)
+    scale = (X.astype(np.float64) ** 2).sum(1).max() * 2
+    eps = np.finfo(dtype).eps
+    assert got.shape == (k, n)
+    assert np.max(np.abs(got.astype(np.float64) - want)) <= 4 * np.sqrt(d) * eps * scale
