@@ -1,0 +1,169 @@
+#!/usr/bin/env python3
+"""Lloyd-iteration throughput of the gfx950 k-means engine on one MI355X.
+
+A step is one Lloyd iteration (fused distance+argmin pass, then the centroid
+update) over the whole resident data set. The default workload is the headline
+shape: 10,000,000 x 32 float32 Gaussian blobs, k = 256, seeded-random row
+initialisation. Prints one JSON line.
+
+    python bench.py [--gpus 1] [--steps 30] [--warmup 3] [--workload C3]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from h2o4gpu_amd import datasets  # noqa: E402
+from h2o4gpu_amd.libs import kmeans_hip  # noqa: E402
+
+PEAK_HBM_GBPS = 8000.0
+PEAK_MFMA_TFLOPS = {"f32": 157.3, "f64": 78.6}
+
+
+def log(msg):
+    print("[bench] " + msg, file=sys.stderr, flush=True)
+
+
+def cpu_baseline(X, C0, iters):
+    """The CPU restatement (oracle port) timed on this host's cores: `iters` full
+    Lloyd iterations (assign + update) over all rows, all hardware threads."""
+    from oracle import load_oracle
+    orc = load_oracle()
+    threads = min(os.cpu_count() or 1, orc.max_threads)
+    C = C0.copy()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        labels = orc.assign(X, C, threads=threads)
+        C, _ = orc.update(X, labels, C, threads=threads)
+    dt = time.perf_counter() - t0
+    return {"value": iters / dt, "unit": "iter/s", "cores": threads, "kind": "port",
+            "sample": "%d full Lloyd iterations (assign+update) over all %d rows, "
+                      "C++/OpenMP restatement of the reference semantics" % (iters, X.shape[0]),
+            "seconds": dt}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="C3", choices=sorted(datasets.SHAPES))
+    ap.add_argument("--scale", type=float, default=1.0, help="row-count scale (1.0 = full shape)")
+    ap.add_argument("--dtype", default="f32", choices=["f32", "f64"])
+    ap.add_argument("--assign", default="auto", choices=sorted(kmeans_hip.ASSIGN_VARIANTS))
+    ap.add_argument("--no-fuse", action="store_true",
+                    help="keep assignment and accumulation as separate kernels")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-iters", type=int, default=0, help="CPU baseline iterations (0 = auto)")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py: this engine runs on one GPU; --gpus %d is not supported "
+              "(collectives and sharding are not part of this build)" % args.gpus, file=sys.stderr)
+        return 2
+    if kmeans_hip.device_count() < 1:
+        print("bench.py: no HIP device visible", file=sys.stderr)
+        return 3
+
+    dtype = np.float32 if args.dtype == "f32" else np.float64
+    t0 = time.perf_counter()
+    X, k, _ = datasets.make(args.workload, args.scale, dtype)
+    n, d = X.shape
+    C0 = datasets.seeded_row_init(X, k, datasets.SHAPES[args.workload][3])
+    log("generated %s: %d x %d %s, k=%d in %.1f s" % (args.workload, n, d, X.dtype, k,
+                                                    time.perf_counter() - t0))
+    s = X.dtype.itemsize
+    flops_per_iter = 2.0 * n * k * d
+    bytes_per_iter = float(n) * d * s + 4.0 * n + 2.0 * k * d * s
+
+    h = kmeans_hip.Handle(n, d, k, dtype)
+    t0 = time.perf_counter()
+    h.set_data(X)
+    h2d_s = time.perf_counter() - t0
+    h.set_centroids(C0)
+    h.set_option("assign", args.assign)
+    if args.no_fuse:
+        h.set_option("fuse", 0)
+    variant = h.assign_variant()
+    log("upload %.2f s (%.1f GB/s incl. pageable staging); assign variant %s"
+        % (h2d_s, n * d * s / h2d_s / 1e9, variant))
+
+    # warm-up, then exactly K timed steps between stream events
+    h.iterate(args.warmup)
+    h.timer_start()
+    h.timer_stop()
+    h.timer_start()
+    h.iterate(args.steps)
+    ms_total = h.timer_stop()
+    ms_step = ms_total / args.steps
+
+    # per-kernel durations: same K steps again with an event pair round every launch
+    h.profile(True)
+    h.iterate(args.steps)
+    kern = {}
+    for name in ("assign", "accumulate", "assign_accumulate", "finalize", "post_update"):
+        cnt, ms = h.kernel_time(name)
+        if cnt:
+            kern[name] = {"launches": cnt, "avg_ms": ms / cnt}
+    h.profile(False)
+
+    fused = "assign_accumulate" in kern
+    dom = "assign_accumulate" if fused else "assign"
+    assign_ms = kern[dom]["avg_ms"]
+    tflops = flops_per_iter / (assign_ms * 1e-3) / 1e12
+    peak = PEAK_MFMA_TFLOPS[args.dtype]
+    mfma_bound = variant != "valu"
+    if mfma_bound:
+        roofline = {"bound": "mfma", "kernel": "%s (%s)" % (dom, variant), "achieved": tflops,
+                    "peak": peak, "unit": "TFLOP/s", "frac": tflops / peak, "traffic": None}
+    else:
+        gbps = (float(n) * d * s + 8.0 * n) / (assign_ms * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "kernel": "assign (valu)", "achieved": gbps,
+                    "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": gbps / PEAK_HBM_GBPS,
+                    "traffic": None}
+    iter_gbps = bytes_per_iter / (ms_step * 1e-3) / 1e9
+    copy_bytes = 1 << 30
+    copy_ms = kmeans_hip.copy_probe(copy_bytes, 10)
+
+    inertia = None
+    h.assign()
+    inertia = h.inertia()
+    h.close()
+
+    out = {
+        "metric": "lloyd_iterations_per_second", "value": 1000.0 / ms_step, "unit": "iter/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic",
+        "config": {"workload": "%s: %d x %d %s Gaussian blobs, k=%d, seeded-random row init, "
+                               "one step = assign + centroid update" % (args.workload, n, d, args.dtype, k),
+                   "rows": n, "cols": d, "k": k, "assign_variant": variant},
+        "roofline": roofline,
+        "iteration": {"algorithmic_bytes": bytes_per_iter, "algorithmic_flops": flops_per_iter,
+                      "gbps": iter_gbps, "hbm_frac": iter_gbps / PEAK_HBM_GBPS,
+                      "tflops": flops_per_iter / (ms_step * 1e-3) / 1e12,
+                      "mfma_frac": flops_per_iter / (ms_step * 1e-3) / 1e12 / peak},
+        "kernels_avg_ms": {kname: round(v["avg_ms"], 5) for kname, v in kern.items()},
+        "copy_probe_gbps": 2.0 * copy_bytes / (copy_ms * 1e-3) / 1e9,
+        "h2d_seconds": h2d_s,
+        "inertia": inertia,
+    }
+    if not args.no_cpu:
+        iters = args.cpu_iters
+        if iters <= 0:
+            # ~10-30 s of CPU work: assume ~5 GFLOP/s per core for the estimate
+            est = flops_per_iter / (5e9 * (os.cpu_count() or 1))
+            iters = int(max(1, min(5, round(20.0 / max(est, 1e-3)))))
+        out["cpu_baseline"] = cpu_baseline(X, C0, iters)
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

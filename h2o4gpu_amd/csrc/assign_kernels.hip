@@ -88,12 +88,19 @@ __global__ __launch_bounds__(WG) void assign_valu_kernel(
 // (min, index). Lane groups holding different centroid subsets of the same row
 // are merged with one (f32) or two (f64) cross-lane exchanges per row tile.
 // ---------------------------------------------------------------------------
-template <typename T, int DP, int ROWT, bool VECLOAD>
-__global__ __launch_bounds__(WG) void assign_rowstat_kernel(
+//
+// FUSE: the workgroup also keeps per-centroid sums and counts of the rows it
+// labels in LDS (row stride DP+1 words so that different centroids start on
+// different banks) and writes them to its own slot psums[blockIdx.x][k][d],
+// pcounts[blockIdx.x][k] when it has walked all its row tiles: the centroid
+// update then needs no second pass over the data.
+template <typename T, int DP, int ROWT, bool VECLOAD, bool FUSE, int NW>
+__global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
     const T *__restrict__ X, const T *__restrict__ xnorm,
     const T *__restrict__ C, const T *__restrict__ cnorm,
     int *__restrict__ labels, T *__restrict__ mindist, int64_t n, int d, int k,
-    int kp) {
+    int kp, double *__restrict__ psums, int *__restrict__ pcounts) {
+  constexpr int TPB = NW * 64;
   typedef Mfma<T> M;
   constexpr int MT = M::MT, KL = M::KL, NACC = M::NACC, VW = M::VW;
   constexpr int DCH = DP / KL;  // features per lane group
@@ -105,6 +112,10 @@ __global__ __launch_bounds__(WG) void assign_rowstat_kernel(
   extern __shared__ __align__(16) unsigned char smem_raw[];
   T *Cs = reinterpret_cast<T *>(smem_raw);  // [KT][NV][64][VW]
   T *ccs = Cs + (size_t)kp * DP;            // [kp]
+  constexpr int SD = DP + 1;
+  // (FUSE) sums in double: ds_add_f64 is the fast LDS floating-point atomic on gfx950
+  double *sums = reinterpret_cast<double *>(ccs + kp + (kp & 1));  // [k][SD], 8-byte aligned
+  int *cnt = reinterpret_cast<int *>(sums + (size_t)k * SD);       // [k]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -113,17 +124,22 @@ __global__ __launch_bounds__(WG) void assign_rowstat_kernel(
   const int g = lane / MT;
   const int KT = kp / MT;
 
-  for (int e = tid; e < kp * DP; e += WG) {
+  if (FUSE) {
+    for (int e = tid; e < k * SD; e += TPB) sums[e] = 0.0;
+    for (int c = tid; c < k; c += TPB) cnt[c] = 0;
+  }
+
+  for (int e = tid; e < kp * DP; e += TPB) {
     const int c = e / DP, j = e - c * DP;
     const T v = (c < k && j < d) ? (T)-2 * C[(size_t)c * d + j] : (T)0;
     const int t = c / MT, i = c - t * MT, gg = j / DCH, s = j - gg * DCH;
     Cs[((size_t)(t * NV + s / VW) * 64 + gg * MT + i) * VW + (s % VW)] = v;
   }
-  for (int c = tid; c < kp; c += WG) ccs[c] = c < k ? cnorm[c] : pos_inf<T>();
+  for (int c = tid; c < kp; c += TPB) ccs[c] = c < k ? cnorm[c] : pos_inf<T>();
   __syncthreads();
 
   constexpr int ROWS_PER_WAVE = ROWT * MT;
-  constexpr int ROWS_PER_WG = (WG / 64) * ROWS_PER_WAVE;
+  constexpr int ROWS_PER_WG = NW * ROWS_PER_WAVE;
   for (int64_t base = (int64_t)blockIdx.x * ROWS_PER_WG; base < n;
        base += (int64_t)gridDim.x * ROWS_PER_WG) {
     const int64_t wrow0 = base + (int64_t)wave * ROWS_PER_WAVE;
@@ -204,7 +220,23 @@ __global__ __launch_bounds__(WG) void assign_rowstat_kernel(
         labels[row] = bidx[rt];
         if (mindist) mindist[row] = best[rt];
       }
+      if (FUSE && row < n && bidx[rt] >= 0) {
+        double *srow = sums + (size_t)bidx[rt] * SD + g * DCH;
+#pragma unroll
+        for (int s = 0; s < DCH; s++) unsafeAtomicAdd(srow + s, (double)x[rt][s]);
+        if (g == 0) atomicAdd(&cnt[bidx[rt]], 1);
+      }
     }
+  }
+  if (FUSE) {
+    __syncthreads();
+    double *dst = psums + (size_t)blockIdx.x * k * d;
+    for (int e = tid; e < k * d; e += TPB) {
+      const int c = e / d, j = e - c * d;
+      dst[e] = sums[(size_t)c * SD + j];
+    }
+    int *cdst = pcounts + (size_t)blockIdx.x * k;
+    for (int c = tid; c < k; c += TPB) cdst[c] = cnt[c];
   }
 }
 
@@ -504,68 +536,116 @@ static int launch_valu(hipStream_t s, const T *X, const T *xnorm, const T *C,
   return 0;
 }
 
-template <typename T, int DP, int ROWT>
-static int launch_rowstat_dp(hipStream_t s, const T *X, const T *xnorm,
-                             const T *C, const T *cnorm, int *labels,
-                             T *mindist, int64_t n, int d, int k, int num_cu) {
+template <typename T>
+static size_t rowstat_fused_lds(int d, int k) {
+  const int dp = rowstat_dp<T>(d);
+  return rowstat_lds<T>(d, k) + 8 + (size_t)k * (dp + 1) * sizeof(double) + (size_t)k * sizeof(int);
+}
+
+// Persistent grid of the row-stationary kernels: as many workgroups as stay
+// resident (two 4-wave workgroups per CU while two LDS images fit, otherwise
+// one 8-wave workgroup per CU), never more than there are row tiles.
+static bool rowstat_two_per_cu(size_t lds) { return lds <= 80 * 1024; }
+
+template <typename T, int DP, int ROWT, bool FUSE, int NW>
+static int launch_rowstat_nw(hipStream_t s, const T *X, const T *xnorm, const T *C,
+                             const T *cnorm, int *labels, T *mindist, int64_t n, int d,
+                             int k, int num_cu, double *psums, int *pcounts, int *slots,
+                             size_t lds) {
   const int MT = Mfma<T>::MT;
   const int kp = (k + MT - 1) / MT * MT;
-  const size_t lds = ((size_t)kp * DP + kp) * sizeof(T);
-  const int rows_per_wg = (WG / 64) * ROWT * MT;
+  const int rows_per_wg = NW * ROWT * MT;
   const int64_t tiles = (n + rows_per_wg - 1) / rows_per_wg;
-  const int wg_per_cu = lds <= 72 * 1024 ? 2 : 1;
-  int64_t grid = (int64_t)num_cu * wg_per_cu;
+  int64_t grid = (int64_t)num_cu * (NW == 4 ? 2 : 1);
   if (grid > tiles) grid = tiles;
   if (grid < 1) grid = 1;
+  if (slots) *slots = (int)grid;
   const bool vec = (d == DP) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0);
   if (vec) {
-    auto kern = assign_rowstat_kernel<T, DP, ROWT, true>;
+    auto kern = assign_rowstat_kernel<T, DP, ROWT, true, FUSE, NW>;
     if (lds > 64 * 1024)
       KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(WG), lds, s, X, xnorm, C,
-                       cnorm, labels, mindist, n, d, k, kp);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), lds, s, X, xnorm, C,
+                       cnorm, labels, mindist, n, d, k, kp, psums, pcounts);
   } else {
-    auto kern = assign_rowstat_kernel<T, DP, ROWT, false>;
+    auto kern = assign_rowstat_kernel<T, DP, ROWT, false, FUSE, NW>;
     if (lds > 64 * 1024)
       KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(WG), lds, s, X, xnorm, C,
-                       cnorm, labels, mindist, n, d, k, kp);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), lds, s, X, xnorm, C,
+                       cnorm, labels, mindist, n, d, k, kp, psums, pcounts);
   }
   KM_HIP_TRY(hipGetLastError());
   return 0;
 }
 
-template <typename T>
+template <typename T, int DP, int ROWT, bool FUSE>
+static int launch_rowstat_dp(hipStream_t s, const T *X, const T *xnorm,
+                             const T *C, const T *cnorm, int *labels,
+                             T *mindist, int64_t n, int d, int k, int num_cu,
+                             double *psums, int *pcounts, int *slots) {
+  const size_t lds = FUSE ? rowstat_fused_lds<T>(d, k) : rowstat_lds<T>(d, k);
+  if (rowstat_two_per_cu(lds))
+    return launch_rowstat_nw<T, DP, ROWT, FUSE, 4>(s, X, xnorm, C, cnorm, labels, mindist, n, d,
+                                                   k, num_cu, psums, pcounts, slots, lds);
+  return launch_rowstat_nw<T, DP, ROWT, FUSE, 8>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k,
+                                                 num_cu, psums, pcounts, slots, lds);
+}
+
+template <typename T, bool FUSE>
 struct RowstatDispatch;
-template <>
-struct RowstatDispatch<float> {
+#define KM_ROWSTAT_CASE(T, DP, ROWT)                                                  \
+  case DP:                                                                            \
+    return launch_rowstat_dp<T, DP, ROWT, FUSE>(s, X, xnorm, C, cnorm, labels, mindist, \
+                                                n, d, k, num_cu, psums, pcounts, slots)
+template <bool FUSE>
+struct RowstatDispatch<float, FUSE> {
   static int run(hipStream_t s, const float *X, const float *xnorm, const float *C,
                  const float *cnorm, int *labels, float *mindist, int64_t n, int d,
-                 int k, int num_cu) {
+                 int k, int num_cu, double *psums, int *pcounts, int *slots) {
     switch (rowstat_dp<float>(d)) {
-      case 16: return launch_rowstat_dp<float, 16, 2>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu);
-      case 32: return launch_rowstat_dp<float, 32, 2>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu);
-      case 64: return launch_rowstat_dp<float, 64, 2>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu);
-      case 128: return launch_rowstat_dp<float, 128, 1>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu);
+      KM_ROWSTAT_CASE(float, 16, 2);
+      KM_ROWSTAT_CASE(float, 32, 2);
+      KM_ROWSTAT_CASE(float, 64, 2);
+      KM_ROWSTAT_CASE(float, 128, 1);
     }
     return H2O4GPU_KMEANS_EARG;
   }
 };
-template <>
-struct RowstatDispatch<double> {
+template <bool FUSE>
+struct RowstatDispatch<double, FUSE> {
   static int run(hipStream_t s, const double *X, const double *xnorm, const double *C,
                  const double *cnorm, int *labels, double *mindist, int64_t n, int d,
-                 int k, int num_cu) {
+                 int k, int num_cu, double *psums, int *pcounts, int *slots) {
     switch (rowstat_dp<double>(d)) {
-      case 16: return launch_rowstat_dp<double, 16, 4>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu);
-      case 32: return launch_rowstat_dp<double, 32, 4>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu);
-      case 64: return launch_rowstat_dp<double, 64, 2>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu);
+      KM_ROWSTAT_CASE(double, 16, 4);
+      KM_ROWSTAT_CASE(double, 32, 4);
+      KM_ROWSTAT_CASE(double, 64, 2);
     }
     return H2O4GPU_KMEANS_EARG;
   }
 };
+#undef KM_ROWSTAT_CASE
+
+// Fused assign + accumulate is offered where the row-stationary kernel applies
+// and centroids plus the double-precision sums fit in one CU's LDS.
+template <typename T>
+int fused_slots(int requested_variant, int64_t n, int d, int k, int num_cu) {
+  if (pick_assign_variant<T>(requested_variant, n, d, k) != ASSIGN_ROWSTAT) return 0;
+  const size_t lds = rowstat_fused_lds<T>(d, k);
+  if (lds > 150 * 1024) return 0;
+  return 2 * num_cu;  // upper bound of the grid = number of partial slots
+}
+
+template <typename T>
+int launch_assign_accumulate(hipStream_t s, const T *X, const T *xnorm, const T *C,
+                             const T *cnorm, int *labels, T *mindist, int64_t n, int d,
+                             int k, int num_cu, double *psums, int *pcounts, int *slots) {
+  if (n <= 0 || d < 1 || k < 1) return H2O4GPU_KMEANS_EARG;
+  return RowstatDispatch<T, true>::run(s, X, xnorm, C, cnorm, labels, mindist, n, d, k,
+                                       num_cu, psums, pcounts, slots);
+}
 
 template <typename T, int MODE>
 static int launch_tiled(hipStream_t s, const T *X, const T *xnorm, const T *C,
@@ -600,7 +680,8 @@ int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
     case ASSIGN_VALU:
       return launch_valu<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k);
     case ASSIGN_ROWSTAT:
-      return RowstatDispatch<T>::run(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu);
+      return RowstatDispatch<T, false>::run(s, X, xnorm, C, cnorm, labels, mindist, n, d, k,
+                                            num_cu, nullptr, nullptr, nullptr);
     case ASSIGN_TILED:
       return launch_tiled<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k);
   }
@@ -619,6 +700,14 @@ int launch_transform(hipStream_t s, const T *X, const T *xnorm, const T *C,
   return launch_tiled<T, 1>(s, X, xnorm, C, cnorm, nullptr, nullptr, D, n, ldn, d, k);
 }
 
+template int fused_slots<float>(int, int64_t, int, int, int);
+template int fused_slots<double>(int, int64_t, int, int, int);
+template int launch_assign_accumulate<float>(hipStream_t, const float *, const float *,
+                                             const float *, const float *, int *, float *,
+                                             int64_t, int, int, int, double *, int *, int *);
+template int launch_assign_accumulate<double>(hipStream_t, const double *, const double *,
+                                              const double *, const double *, int *, double *,
+                                              int64_t, int, int, int, double *, int *, int *);
 template int pick_assign_variant<float>(int, int64_t, int, int);
 template int pick_assign_variant<double>(int, int64_t, int, int);
 template int launch_assign<float>(hipStream_t, int, const float *, const float *,

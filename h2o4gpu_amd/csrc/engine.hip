@@ -87,6 +87,7 @@ struct h2o4gpu_kmeans_handle {
   int num_cu = 0;
   hipStream_t stream = nullptr;
   int opt_assign = ASSIGN_AUTO;
+  int opt_fuse = 1;  // 1: use the fused assign+accumulate kernel where the shape allows
   int last_variant = ASSIGN_AUTO;
 
   // profiling
@@ -110,6 +111,7 @@ struct h2o4gpu_kmeans_handle {
   virtual int assign() = 0;
   virtual int update(double *shift2) = 0;
   virtual int set_labels_host(const int *labels) = 0;
+  virtual int iterate(int steps) = 0;
   virtual int get_centroids(void *C) = 0;
   virtual int get_labels(int *labels) = 0;
   virtual int get_counts(int *counts) = 0;
@@ -195,7 +197,7 @@ struct Engine : h2o4gpu_kmeans_handle {
   T *mindist = nullptr;
   int *counts = nullptr;
   UpdatePlan plan;
-  T *psums = nullptr;
+  double *psums = nullptr;
   int *pcounts = nullptr;
   T *shift_partials = nullptr;
   T *shift2 = nullptr;
@@ -233,9 +235,12 @@ struct Engine : h2o4gpu_kmeans_handle {
     KM_TRY(dalloc(&labels, n));
     KM_TRY(dalloc(&xnorm, n));
     KM_TRY(dalloc(&mindist, n));
-    KM_TRY(dalloc(&psums, (size_t)plan.row_blocks * kd));
-    KM_TRY(dalloc(&pcounts, (size_t)plan.row_blocks * k));
-    KM_TRY(dalloc(&shift_partials, (kd + 255) / 256 + 1));
+    int slots = plan.row_blocks;
+    const int fs = fused_slots<T>(ASSIGN_AUTO, n, d, k, num_cu);
+    if (fs > slots) slots = fs;
+    KM_TRY(dalloc(&psums, (size_t)slots * kd));
+    KM_TRY(dalloc(&pcounts, (size_t)slots * k));
+    KM_TRY(dalloc(&shift_partials, (kd + 31) / 32 + 1));
     KM_TRY(dalloc(&shift2, 1));
     KM_TRY(dalloc(&sum_partials, sum_partials_needed() + 1));
     KM_TRY(dalloc(&kpp_bsums, (n + KPP_BLOCK - 1) / KPP_BLOCK + 1));
@@ -409,8 +414,27 @@ struct Engine : h2o4gpu_kmeans_handle {
 
   int update_async() {
     PROFILED("accumulate", launch_accumulate<T>(stream, plan, X, labels, psums, pcounts, n, d, k));
+    return finish_update(plan.row_blocks);
+  }
+
+  // one Lloyd step: labels against the current centroids, then the update
+  int step_async() {
+    if (opt_fuse && fused_slots<T>(opt_assign, n, d, k, num_cu) > 0) {
+      int slots = 0;
+      PROFILED("assign_accumulate",
+               launch_assign_accumulate<T>(stream, X, xnorm, C[cur], cnorm, labels, mindist, n, d,
+                                           k, num_cu, psums, pcounts, &slots));
+      last_variant = ASSIGN_ROWSTAT;
+      have_mindist = true;
+      return finish_update(slots);
+    }
+    KM_TRY(assign());
+    return update_async();
+  }
+
+  int finish_update(int slots) {
     int nsp = 0;
-    PROFILED("finalize", launch_finalize<T>(stream, plan, psums, pcounts, C[cur], C[cur ^ 1],
+    PROFILED("finalize", launch_finalize<T>(stream, slots, psums, pcounts, C[cur], C[cur ^ 1],
                                             counts, shift_partials, &nsp, d, k));
     PROFILED("post_update", launch_post_update<T>(stream, C[cur ^ 1], cnorm, shift_partials,
                                                   nsp, shift2, d, k));
@@ -444,8 +468,7 @@ struct Engine : h2o4gpu_kmeans_handle {
     int updates = 0;
     for (int i = 0; i < max_iterations; i++) {
       log_msg(verbose, LOG_VERBOSE, "KMeans - Iteration %d/%d", i, max_iterations);
-      KM_TRY(assign());
-      KM_TRY(update_async());
+      KM_TRY(step_async());
       updates++;
       bool done = false;
       if (threshold > 0) {
@@ -468,6 +491,13 @@ struct Engine : h2o4gpu_kmeans_handle {
     }
     KM_HIP_TRY(hipStreamSynchronize(stream));
     if (iters) *iters = updates;
+    return 0;
+  }
+
+  int iterate(int steps) override {
+    KM_HIP_TRY(hipSetDevice(dev));
+    if (!have_data || !have_centroids) return H2O4GPU_KMEANS_ESTATE;
+    for (int i = 0; i < steps; i++) KM_TRY(step_async());
     return 0;
   }
 
@@ -786,6 +816,10 @@ KM_API int h2o4gpu_kmeans_set_labels_host(h2o4gpu_kmeans_handle *h, const int *l
   if (!labels) return H2O4GPU_KMEANS_EARG;
   return h->set_labels_host(labels);
 }
+KM_API int h2o4gpu_kmeans_iterate(h2o4gpu_kmeans_handle *h, int steps) {
+  KM_CHECK_HANDLE(h);
+  return h->iterate(steps);
+}
 KM_API int h2o4gpu_kmeans_get_centroids(h2o4gpu_kmeans_handle *h, void *C) {
   KM_CHECK_HANDLE(h);
   return C ? h->get_centroids(C) : H2O4GPU_KMEANS_EARG;
@@ -832,7 +866,11 @@ KM_API int h2o4gpu_kmeans_set_option(h2o4gpu_kmeans_handle *h, const char *name,
     h->opt_assign = value;
     return 0;
   }
-  if (strcmp(name, "update") == 0) return value == 0 ? 0 : H2O4GPU_KMEANS_EARG;
+  if (strcmp(name, "fuse") == 0) {
+    if (value != 0 && value != 1) return H2O4GPU_KMEANS_EARG;
+    h->opt_fuse = value;
+    return 0;
+  }
   return H2O4GPU_KMEANS_EARG;
 }
 KM_API int h2o4gpu_kmeans_timer_start(h2o4gpu_kmeans_handle *h) {

@@ -62,6 +62,18 @@ template <typename T>
 int pick_assign_variant(int requested, int64_t n, int d, int k);
 const char *assign_variant_name(int variant);
 
+// Fused assign + accumulate (row-stationary shapes only): labels/mindist as
+// launch_assign, plus per-workgroup partial sums psums[slot][k][d] and counts
+// pcounts[slot][k]; *slots receives the number of slots written. fused_slots()
+// returns the largest slot count the launch can use, or 0 when the shape (or a
+// forced assign variant) rules the fused kernel out.
+template <typename T>
+int fused_slots(int requested_variant, int64_t n, int d, int k, int num_cu);
+template <typename T>
+int launch_assign_accumulate(hipStream_t s, const T *X, const T *xnorm, const T *C,
+                             const T *cnorm, int *labels, T *mindist, int64_t n, int d,
+                             int k, int num_cu, double *psums, int *pcounts, int *slots);
+
 // Full squared-distance matrix, centroid-major: D[c * ldn + i], i < n.
 template <typename T>
 int launch_transform(hipStream_t s, const T *X, const T *xnorm, const T *C,
@@ -72,24 +84,25 @@ int launch_transform(hipStream_t s, const T *X, const T *xnorm, const T *C,
 template <typename T>
 int launch_row_norms(hipStream_t s, const T *X, T *out, int64_t n, int d);
 
-// Centroid update, pass 1: per-row-block partial sums and counts.
+// Centroid update, pass 1: per-row-block partial sums (always double) and counts.
 struct UpdatePlan {
   int row_blocks;   // partial slots along rows
   int kc;           // centroids per LDS chunk
   int k_chunks;     // ceil(k / kc)
   int vec;          // elements per load (1, 2 or 4)
+  int sd;           // LDS row stride of the sums, in elements
   size_t lds_bytes;
 };
 template <typename T>
 UpdatePlan plan_update(int64_t n, int d, int k, int num_cu);
 template <typename T>
 int launch_accumulate(hipStream_t s, const UpdatePlan &p, const T *X,
-                      const int *labels, T *psums, int *pcounts, int64_t n,
+                      const int *labels, double *psums, int *pcounts, int64_t n,
                       int d, int k);
 // Pass 2: fixed-order reduction of the partials, empty clusters keep the old
 // centroid, mean = sum * (1/count), per-block partial of sum((old-new)^2).
 template <typename T>
-int launch_finalize(hipStream_t s, const UpdatePlan &p, const T *psums,
+int launch_finalize(hipStream_t s, int slots, const double *psums,
                     const int *pcounts, const T *c_old, T *c_new, int *counts,
                     T *shift_partials, int *n_shift_partials, int d, int k);
 // Pass 3: cnorm of the new centroids and the fixed-order sum of the shift

@@ -19,13 +19,12 @@ namespace kmhip {
 
 static constexpr int WG = 256;
 
-// LDS floating-point add without return value (ds_add_f32 / ds_add_f64).
-__device__ __forceinline__ void lds_add(float *p, float v) {
-  __builtin_amdgcn_ds_faddf((__attribute__((address_space(3))) float *)p, v, 0, 0, false);
-}
-__device__ __forceinline__ void lds_add(double *p, double v) {
-  unsafeAtomicAdd(p, v);
-}
+// Sums are kept in double in LDS for both precisions and added with ds_add_f64:
+// measured on gfx950, ds_add_f32 retires about 0.33 lane-operations per clock
+// per CU whatever the address pattern, ds_add_f64 about 8. As a side effect a
+// float32 column whose values span fewer than ~14 binades is summed exactly, so
+// the result does not depend on the order in which wavefronts arrive.
+__device__ __forceinline__ void lds_add(double *p, double v) { unsafeAtomicAdd(p, v); }
 
 // ---------------------------------------------------------------------------
 // out[i] = sum_j X[i][j]^2, j ascending, multiply and add rounded separately
@@ -119,34 +118,50 @@ template <> struct VecOf<float, 2> { typedef float type __attribute__((ext_vecto
 template <> struct VecOf<double, 2> { typedef double type __attribute__((ext_vector_type(2))); };
 
 template <typename T, int VEC>
-__device__ __forceinline__ void add_row_slice(T *srow, const T *xrow, int col,
-                                              int lpr, int d) {
-  // lanes col, col+lpr, ... each take VEC consecutive features
-  for (int j = col * VEC; j < d; j += lpr * VEC) {
-    if constexpr (VEC == 1) {
-      lds_add(srow + j, xrow[j]);
-    } else {
-      typedef typename VecOf<T, VEC>::type vt;
-      const vt v = *reinterpret_cast<const vt *>(xrow + j);
+struct RowVec {
+  typedef typename VecOf<T, VEC>::type type;
+};
+template <typename T>
+struct RowVec<T, 1> {
+  typedef T type;
+};
+template <typename T, int VEC>
+__device__ __forceinline__ typename RowVec<T, VEC>::type load_vec(const T *p) {
+  return *reinterpret_cast<const typename RowVec<T, VEC>::type *>(p);
+}
+template <typename T, int VEC>
+__device__ __forceinline__ void lds_add_vec(double *dst, typename RowVec<T, VEC>::type v) {
+  if constexpr (VEC == 1) {
+    lds_add(dst, (double)v);
+  } else {
 #pragma unroll
-      for (int e = 0; e < VEC; e++) lds_add(srow + j + e, v[e]);
-    }
+    for (int e = 0; e < VEC; e++) lds_add(dst + e, (double)v[e]);
   }
 }
 
 template <typename T, int VEC>
+__device__ __forceinline__ void add_row_slice(double *srow, const T *xrow, int col,
+                                              int lpr, int d) {
+  // lanes col, col+lpr, ... each take VEC consecutive features
+  for (int j = col * VEC; j < d; j += lpr * VEC)
+    lds_add_vec<T, VEC>(srow + j, load_vec<T, VEC>(xrow + j));
+}
+
+// sd = LDS row stride of the sums (>= d): chosen odd-ish by the host so that
+// rows of different centroids do not all start on the same bank.
+template <typename T, int VEC>
 __global__ __launch_bounds__(WG) void accumulate_kernel(
     const T *__restrict__ X, const int *__restrict__ labels,
-    T *__restrict__ psums, int *__restrict__ pcounts, int64_t n, int d, int k,
-    int kc, int64_t rows_per_block, int lpr) {
+    double *__restrict__ psums, int *__restrict__ pcounts, int64_t n, int d, int k,
+    int kc, int64_t rows_per_block, int lpr, int sd) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  T *sums = reinterpret_cast<T *>(smem_raw);                  // [kc][d]
-  int *cnt = reinterpret_cast<int *>(sums + (size_t)kc * d);  // [kc]
+  double *sums = reinterpret_cast<double *>(smem_raw);         // [kc][sd]
+  int *cnt = reinterpret_cast<int *>(sums + (size_t)kc * sd);  // [kc]
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int k0 = blockIdx.y * kc;
   const int nk = min(kc, k - k0);
-  for (int e = tid; e < nk * d; e += WG) sums[e] = (T)0;
+  for (int e = tid; e < nk * sd; e += WG) sums[e] = 0.0;
   for (int c = tid; c < nk; c += WG) cnt[c] = 0;
   __syncthreads();
 
@@ -155,6 +170,8 @@ __global__ __launch_bounds__(WG) void accumulate_kernel(
   const int rps = 64 / lpr;  // rows served per wavefront step
   const int sub = lane / lpr, col = lane % lpr;
   const bool single_chunk = gridDim.y == 1;
+  const bool narrow = d <= lpr * VEC;  // one vector per lane covers a row
+  constexpr int U = 8;
 
   for (int64_t g0 = r0 + (int64_t)wave * 64; g0 < r1; g0 += (WG / 64) * 64) {
     const int64_t myrow = g0 + lane;
@@ -162,14 +179,31 @@ __global__ __launch_bounds__(WG) void accumulate_kernel(
     if (myrow < r1) lab = labels[myrow] - k0;
     const bool match = lab >= 0 && lab < nk;
     if (match) atomicAdd(&cnt[lab], 1);
-    if (single_chunk) {
-      // dense: rows g0 .. g0+63 in steps of rps rows
+    if (single_chunk && narrow) {
+      // all loads of U row groups are issued before the first LDS add
+      const bool has = col * VEC < d;
+      for (int b = 0; b < 64; b += rps * U) {
+        typename RowVec<T, VEC>::type v[U];
+        int l[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+          const int src = b + u * rps + sub;
+          l[u] = src < 64 ? __shfl(lab, src & 63, 64) : -1;
+          const int64_t row = g0 + src;
+          if (!(l[u] >= 0 && l[u] < nk && row < r1 && has)) l[u] = -1;
+          v[u] = load_vec<T, VEC>(X + (l[u] >= 0 ? row : r0) * (int64_t)d + (has ? col * VEC : 0));
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++)
+          if (l[u] >= 0) lds_add_vec<T, VEC>(sums + (size_t)l[u] * sd + col * VEC, v[u]);
+      }
+    } else if (single_chunk) {
       for (int b = 0; b < 64; b += rps) {
         const int src = b + sub;
         const int l = __shfl(lab, src, 64);
         const int64_t row = g0 + src;
         if (l >= 0 && l < nk && row < r1)
-          add_row_slice<T, VEC>(sums + (size_t)l * d, X + row * (int64_t)d, col, lpr, d);
+          add_row_slice<T, VEC>(sums + (size_t)l * sd, X + row * (int64_t)d, col, lpr, d);
       }
     } else {
       unsigned long long mask = __ballot(match);
@@ -187,22 +221,30 @@ __global__ __launch_bounds__(WG) void accumulate_kernel(
         const int l = __shfl(lab, src < 0 ? 0 : src, 64);
         if (src >= 0) {
           const int64_t row = g0 + src;
-          add_row_slice<T, VEC>(sums + (size_t)l * d, X + row * (int64_t)d, col, lpr, d);
+          add_row_slice<T, VEC>(sums + (size_t)l * sd, X + row * (int64_t)d, col, lpr, d);
         }
       }
     }
   }
   __syncthreads();
-  T *dst = psums + ((size_t)blockIdx.x * k + k0) * d;
-  for (int e = tid; e < nk * d; e += WG) dst[e] = sums[e];
+  double *dst = psums + ((size_t)blockIdx.x * k + k0) * d;
+  for (int e = tid; e < nk * d; e += WG) {
+    const int c = e / d, j = e - c * d;
+    dst[e] = sums[(size_t)c * sd + j];
+  }
   int *cdst = pcounts + (size_t)blockIdx.x * k + k0;
   for (int c = tid; c < nk; c += WG) cdst[c] = cnt[c];
 }
 
+// LDS row stride of the sums (in doubles): odd, so that the rows of different
+// centroids start on different banks.
+static int update_lds_stride(int d) { return d | 1; }
+
 template <typename T>
 UpdatePlan plan_update(int64_t n, int d, int k, int num_cu) {
   UpdatePlan p;
-  const size_t per_centroid = (size_t)d * sizeof(T) + sizeof(int);
+  p.sd = update_lds_stride(d);
+  const size_t per_centroid = (size_t)p.sd * sizeof(double) + sizeof(int);
   const size_t budget = 64 * 1024;
   int kc = (int)(budget / per_centroid);
   if (kc < 1) kc = 1;
@@ -230,7 +272,7 @@ UpdatePlan plan_update(int64_t n, int d, int k, int num_cu) {
 
 template <typename T, int VEC>
 static int launch_accumulate_vec(hipStream_t s, const UpdatePlan &p, const T *X,
-                                 const int *labels, T *psums, int *pcounts,
+                                 const int *labels, double *psums, int *pcounts,
                                  int64_t n, int d, int k) {
   const int64_t rows_per_block = ((n + p.row_blocks - 1) / p.row_blocks + 63) / 64 * 64;
   int groups = (d + VEC - 1) / VEC;  // lanes wanted per row
@@ -242,14 +284,14 @@ static int launch_accumulate_vec(hipStream_t s, const UpdatePlan &p, const T *X,
                                    hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)p.lds_bytes));
   hipLaunchKernelGGL(kern, dim3(p.row_blocks, p.k_chunks), dim3(WG), p.lds_bytes, s,
-                     X, labels, psums, pcounts, n, d, k, p.kc, rows_per_block, lpr);
+                     X, labels, psums, pcounts, n, d, k, p.kc, rows_per_block, lpr, p.sd);
   KM_HIP_TRY(hipGetLastError());
   return 0;
 }
 
 template <>
 int launch_accumulate<float>(hipStream_t s, const UpdatePlan &p, const float *X,
-                             const int *labels, float *psums, int *pcounts,
+                             const int *labels, double *psums, int *pcounts,
                              int64_t n, int d, int k) {
   const bool aligned = (reinterpret_cast<uintptr_t>(X) & 15) == 0;
   if (p.vec == 4 && aligned) return launch_accumulate_vec<float, 4>(s, p, X, labels, psums, pcounts, n, d, k);
@@ -268,55 +310,89 @@ int launch_accumulate<double>(hipStream_t s, const UpdatePlan &p, const double *
 // ---------------------------------------------------------------------------
 // pass 2: finalize. One thread per centroid coordinate.
 // ---------------------------------------------------------------------------
+// A workgroup takes EPW = 32 consecutive coordinates; RS = 8 thread groups each
+// sum a contiguous range of the row-block slots for those coordinates (slot
+// order), then group 0 adds the 8 range sums in range order.
 template <typename T>
 __global__ __launch_bounds__(WG) void finalize_kernel(
-    const T *__restrict__ psums, const int *__restrict__ pcounts, int row_blocks,
+    const double *__restrict__ psums, const int *__restrict__ pcounts, int row_blocks,
     const T *__restrict__ c_old, T *__restrict__ c_new, int *__restrict__ counts,
     T *__restrict__ shift_partials, int d, int k) {
 #pragma clang fp contract(off)
-  __shared__ T red[WG];
+  constexpr int EPW = 32, RS = WG / EPW;
+  __shared__ double part[RS][EPW];
+  __shared__ int cpart[RS][EPW];
+  __shared__ T red[EPW];
   const int tid = threadIdx.x;
-  const int64_t e = (int64_t)blockIdx.x * WG + tid;
+  const int slice = tid / EPW, el = tid % EPW;
   const int64_t kd = (int64_t)k * d;
-  T diff2 = 0;
-  if (e < kd) {
-    const int c = (int)(e / d);
-    int cnt = 0;
-    T s = 0;
-    for (int rb = 0; rb < row_blocks; rb++) {
-      cnt += pcounts[(size_t)rb * k + c];
+  const int64_t e = (int64_t)blockIdx.x * EPW + el;
+  const bool valid = e < kd;
+  const int c = valid ? (int)(e / d) : 0;
+  const int per = (row_blocks + RS - 1) / RS;
+  const int lo = slice * per, hi = min(row_blocks, lo + per);
+  double s = 0;
+  int cnt = 0;
+  if (valid) {
+    int rb = lo;
+    for (; rb + 4 <= hi; rb += 4) {
+      const double a0 = psums[(size_t)rb * kd + e], a1 = psums[(size_t)(rb + 1) * kd + e];
+      const double a2 = psums[(size_t)(rb + 2) * kd + e], a3 = psums[(size_t)(rb + 3) * kd + e];
+      const int b0 = pcounts[(size_t)rb * k + c], b1 = pcounts[(size_t)(rb + 1) * k + c];
+      const int b2 = pcounts[(size_t)(rb + 2) * k + c], b3 = pcounts[(size_t)(rb + 3) * k + c];
+      s = s + a0;
+      s = s + a1;
+      s = s + a2;
+      s = s + a3;
+      cnt += b0 + b1 + b2 + b3;
+    }
+    for (; rb < hi; rb++) {
       s = s + psums[(size_t)rb * kd + e];
+      cnt += pcounts[(size_t)rb * k + c];
+    }
+  }
+  part[slice][el] = s;
+  cpart[slice][el] = cnt;
+  __syncthreads();
+  T diff2 = 0;
+  if (slice == 0 && valid) {
+    double tot = part[0][el];
+    int ctot = cpart[0][el];
+#pragma unroll
+    for (int q = 1; q < RS; q++) {
+      tot = tot + part[q][el];
+      ctot += cpart[q][el];
     }
     const T oldv = c_old[e];
     T newv;
-    if (cnt < 1) {
+    if (ctot < 1) {
       newv = oldv;  // revert_zeroed_centroids, kmeans_centroids.h:77-88
     } else {
-      const T scale = (T)1.0 / (T)cnt;  // scale_centroids, kmeans_centroids.h:90-105
-      newv = s * scale;
+      const T scale = (T)1.0 / (T)ctot;  // scale_centroids, kmeans_centroids.h:90-105
+      newv = (T)tot * scale;
     }
     c_new[e] = newv;
-    if (e - (int64_t)c * d == 0) counts[c] = cnt;
+    if (e - (int64_t)c * d == 0) counts[c] = ctot;
     const T df = oldv - newv;
     diff2 = df * df;
   }
-  red[tid] = diff2;
+  if (slice == 0) red[el] = diff2;
   __syncthreads();
-  for (int off = WG / 2; off > 0; off >>= 1) {
-    if (tid < off) red[tid] = red[tid] + red[tid + off];
-    __syncthreads();
+  if (tid == 0) {
+    T acc = 0;
+    for (int q = 0; q < EPW; q++) acc = acc + red[q];
+    shift_partials[blockIdx.x] = acc;
   }
-  if (tid == 0) shift_partials[blockIdx.x] = red[0];
 }
 
 template <typename T>
-int launch_finalize(hipStream_t s, const UpdatePlan &p, const T *psums,
+int launch_finalize(hipStream_t s, int slots, const double *psums,
                     const int *pcounts, const T *c_old, T *c_new, int *counts,
                     T *shift_partials, int *n_shift_partials, int d, int k) {
   const int64_t kd = (int64_t)k * d;
-  const int blocks = (int)((kd + WG - 1) / WG);
+  const int blocks = (int)((kd + 31) / 32);
   hipLaunchKernelGGL((finalize_kernel<T>), dim3(blocks), dim3(WG), 0, s, psums,
-                     pcounts, p.row_blocks, c_old, c_new, counts, shift_partials, d, k);
+                     pcounts, slots, c_old, c_new, counts, shift_partials, d, k);
   KM_HIP_TRY(hipGetLastError());
   *n_shift_partials = blocks;
   return 0;
@@ -441,7 +517,7 @@ int launch_gather_rows(hipStream_t s, const T *X, const int *idx, T *C, int k, i
 #define KM_INSTANTIATE(T)                                                            \
   template int launch_row_norms<T>(hipStream_t, const T *, T *, int64_t, int);       \
   template UpdatePlan plan_update<T>(int64_t, int, int, int);                        \
-  template int launch_finalize<T>(hipStream_t, const UpdatePlan &, const T *,        \
+  template int launch_finalize<T>(hipStream_t, int, const double *,                  \
                                   const int *, const T *, T *, int *, T *, int *,    \
                                   int, int);                                         \
   template int launch_post_update<T>(hipStream_t, const T *, T *, const T *, int,    \

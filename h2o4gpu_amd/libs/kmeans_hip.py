@@ -49,6 +49,7 @@ PROTOTYPES = {
     "h2o4gpu_kmeans_assign": (c_int, [c_void_p]),
     "h2o4gpu_kmeans_update": (c_int, [c_void_p, P(c_double)]),
     "h2o4gpu_kmeans_set_labels_host": (c_int, [c_void_p, c_void_p]),
+    "h2o4gpu_kmeans_iterate": (c_int, [c_void_p, c_int]),
     "h2o4gpu_kmeans_get_centroids": (c_int, [c_void_p, c_void_p]),
     "h2o4gpu_kmeans_get_labels": (c_int, [c_void_p, c_void_p]),
     "h2o4gpu_kmeans_get_counts": (c_int, [c_void_p, c_void_p]),
@@ -184,6 +185,10 @@ class Handle:
         s = c_double(0.0)
         _check("update", lib().h2o4gpu_kmeans_update(self._h, ctypes.byref(s) if want_shift else None))
         return s.value
+
+    def iterate(self, steps):
+        """Enqueue `steps` x (assign + update); returns without waiting."""
+        _check("iterate", lib().h2o4gpu_kmeans_iterate(self._h, int(steps)))
 
     def set_labels(self, labels):
         labels = np.ascontiguousarray(labels, np.int32)

@@ -138,6 +138,9 @@ int h2o4gpu_kmeans_fit(h2o4gpu_kmeans_handle *h, int max_iterations,
 int h2o4gpu_kmeans_assign(h2o4gpu_kmeans_handle *h);
 int h2o4gpu_kmeans_update(h2o4gpu_kmeans_handle *h, double *shift2);
 int h2o4gpu_kmeans_set_labels_host(h2o4gpu_kmeans_handle *h, const int *labels);
+/* Enqueue `steps` iterations (assign + update each) on the handle's stream
+ * without convergence test or host synchronisation (timing loops). */
+int h2o4gpu_kmeans_iterate(h2o4gpu_kmeans_handle *h, int steps);
 
 /* Results to host memory. */
 int h2o4gpu_kmeans_get_centroids(h2o4gpu_kmeans_handle *h, void *C);
@@ -158,7 +161,9 @@ int h2o4gpu_kmeans_transform_host(h2o4gpu_kmeans_handle *h, size_t rows,
 int h2o4gpu_kmeans_transform_resident(h2o4gpu_kmeans_handle *h, void *d_dist);
 
 /* Kernel selection: "assign" = 0 auto, 1 VALU, 2 MFMA row-stationary,
- * 3 MFMA tiled; "update" = 0 auto. Unknown names return EARG. */
+ * 3 MFMA tiled; "fuse" = 1 (default) lets fit/iterate run assignment and the
+ * per-centroid accumulation as one kernel where the shape allows, 0 keeps them
+ * separate. Unknown names return EARG. */
 int h2o4gpu_kmeans_set_option(h2o4gpu_kmeans_handle *h, const char *name,
                               int value);
 
@@ -166,7 +171,8 @@ int h2o4gpu_kmeans_set_option(h2o4gpu_kmeans_handle *h, const char *name,
  * bracket any sequence of calls; with kernel profiling on, every kernel launch
  * is bracketed by its own event pair and kernel_time() returns the launch count
  * and summed milliseconds since profiling was switched on, by kernel name
- * ("assign", "accumulate", "finalize", "row_norms", "transform", ...). */
+ * ("assign", "accumulate", "assign_accumulate", "finalize", "post_update",
+ * "row_norms", "transform", "min_dist_update", "inertia_sum"). */
 int h2o4gpu_kmeans_timer_start(h2o4gpu_kmeans_handle *h);
 int h2o4gpu_kmeans_timer_stop(h2o4gpu_kmeans_handle *h, float *milliseconds);
 int h2o4gpu_kmeans_profile(h2o4gpu_kmeans_handle *h, int on);
