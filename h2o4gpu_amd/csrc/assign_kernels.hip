@@ -76,6 +76,14 @@ __global__ __launch_bounds__(WG) void assign_valu_kernel(
   }
 }
 
+__device__ __forceinline__ unsigned umin3(unsigned a, unsigned b, unsigned c) {
+  return min(a, min(b, c));  // v_min3_u32
+}
+// centroid row of accumulator v (runtime v) of the 32x32 float tile
+__device__ __forceinline__ int key_row(unsigned v, int g) {
+  return (int)((v >> 2) * 8 + (unsigned)g * 4 + (v & 3));
+}
+
 // ---------------------------------------------------------------------------
 // MFMA row-stationary variant (d <= DP, all centroids resident in LDS).
 //
@@ -147,36 +155,41 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
     T xx[ROWT];
 #pragma unroll
     for (int rt = 0; rt < ROWT; rt++) {
-      const int64_t row = wrow0 + rt * MT + r;
-      const bool valid = row < n;
+      // rows past the end re-read the last row; their results are never stored
+      const int64_t row = min(wrow0 + rt * MT + r, n - 1);
       if (VECLOAD) {
-        const vec_t *src = reinterpret_cast<const vec_t *>(
-            X + (valid ? row : 0) * (int64_t)DP + g * DCH);
+        const vec_t *src = reinterpret_cast<const vec_t *>(X + row * (int64_t)DP + g * DCH);
 #pragma unroll
         for (int q = 0; q < NV; q++) {
           vec_t v = src[q];
 #pragma unroll
-          for (int e = 0; e < VW; e++) x[rt][q * VW + e] = valid ? v[e] : (T)0;
+          for (int e = 0; e < VW; e++) x[rt][q * VW + e] = v[e];
         }
       } else {
-        const T *src = X + (valid ? row : 0) * (int64_t)d;
+        const T *src = X + row * (int64_t)d;
 #pragma unroll
         for (int s = 0; s < DCH; s++) {
           const int j = g * DCH + s;
-          x[rt][s] = (valid && j < d) ? src[j] : (T)0;
+          x[rt][s] = j < d ? src[j] : (T)0;
         }
       }
-      xx[rt] = valid ? xnorm[row] : (T)0;
+      xx[rt] = xnorm[row];
     }
     T best[ROWT];
     int bidx[ROWT];
+    unsigned bkey[ROWT];  // float32 path: running minimum key and its tile
+    int btile[ROWT];
 #pragma unroll
     for (int rt = 0; rt < ROWT; rt++) {
       best[rt] = argmin_start<T>();
       bidx[rt] = -1;
+      bkey[rt] = 0x7F7FFFF0u;  // FLT_MAX with the index bits cleared
+      btile[rt] = -1;
     }
-    for (int t = 0; t < KT; t++) {
-      acc_t acc[ROWT];
+    // Two accumulator sets: the matrix-core work of centroid tile t is issued
+    // together with the argmin epilogue of tile t-1, so that one wavefront
+    // alone keeps both the MFMA pipe and the VALU busy.
+    auto tile_mma = [&](acc_t (&acc)[ROWT], int t) {
 #pragma unroll
       for (int v = 0; v < NACC; v++) {
         const T cc = ccs[t * MT + M::acc_row(v, g)];
@@ -194,17 +207,71 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
             acc[rt] = M::mma(a[e], x[rt][q * VW + e], acc[rt]);
         }
       }
-#pragma unroll
-      for (int v = 0; v < NACC; v++) {
-        const int cidx = t * MT + M::acc_row(v, g);
+    };
+    auto tile_argmin = [&](const acc_t (&acc)[ROWT], int t) {
+      if constexpr (sizeof(T) == 4) {
+        // float32 MFMA shares the SIMD's FP32 datapath with ordinary vector
+        // instructions, so every epilogue instruction costs matrix time. The
+        // argmin is therefore done on integer keys: |acc| with its four lowest
+        // mantissa bits replaced by the accumulator number v. Keys of one tile are
+        // reduced with 3-input unsigned minima (positive floats order like
+        // unsigned integers), the winner is compared once per tile with the
+        // running key. Distances are thus compared at a resolution of 16 ulp
+        // (1.9e-6 relative); within one key value the lowest centroid index wins.
 #pragma unroll
         for (int rt = 0; rt < ROWT; rt++) {
-          const T dist = fabs(acc[rt][v]);
-          if (dist < best[rt]) {
-            best[rt] = dist;
-            bidx[rt] = cidx;
+          unsigned key[NACC];
+#pragma unroll
+          for (int v = 0; v < NACC; v++)
+            key[v] = (__float_as_uint(acc[rt][v]) & 0x7FFFFFF0u) | (unsigned)v;
+          unsigned m = umin3(key[0], key[1], key[2]);
+#pragma unroll
+          for (int v = 3; v + 1 < NACC; v += 2) m = umin3(m, key[v], key[v + 1]);
+          if ((NACC & 1) == 0) m = min(m, key[NACC - 1]);
+          if (m < bkey[rt]) {
+            bkey[rt] = m;
+            btile[rt] = t;
           }
         }
+      } else {
+        const int cbase = t * MT + M::acc_row(0, g);
+#pragma unroll
+        for (int v = 0; v < NACC; v++) {
+          const int cidx = cbase + (M::acc_row(v, 0) - M::acc_row(0, 0));
+#pragma unroll
+          for (int rt = 0; rt < ROWT; rt++) {
+            const T dist = fabs(acc[rt][v]);
+            if (dist < best[rt]) {
+              best[rt] = dist;
+              bidx[rt] = cidx;
+            }
+          }
+        }
+      }
+    };
+    {
+      acc_t accA[ROWT], accB[ROWT];
+      tile_mma(accA, 0);
+      int t = 1;
+      for (; t + 1 < KT; t += 2) {
+        tile_mma(accB, t);
+        tile_argmin(accA, t - 1);
+        tile_mma(accA, t + 1);
+        tile_argmin(accB, t);
+      }
+      if (t < KT) {
+        tile_mma(accB, t);
+        tile_argmin(accA, t - 1);
+        tile_argmin(accB, t);
+      } else {
+        tile_argmin(accA, t - 1);
+      }
+    }
+    if constexpr (sizeof(T) == 4) {
+#pragma unroll
+      for (int rt = 0; rt < ROWT; rt++) {
+        best[rt] = __uint_as_float(bkey[rt] & 0xFFFFFFF0u);
+        bidx[rt] = btile[rt] < 0 ? -1 : btile[rt] * MT + key_row(bkey[rt] & 15u, g);
       }
     }
 #pragma unroll

@@ -52,7 +52,9 @@ def test_assign_matches_oracle(hip, oracle, n, d, k, variant, dtype):
         rep = label_report(oracle, X, C, got, want)
         scale = (X.astype(np.float64) ** 2).sum(1).max() + (C.astype(np.float64) ** 2).sum(1).max()
         eps = np.finfo(dtype).eps
-        assert np.max(np.abs(mind.astype(np.float64) - wmind)) <= 4 * np.sqrt(d) * eps * scale
+        # MFMA summation order differs from the scalar loop (rounding of order
+        # sqrt(d)*eps*(xx+cc)); the float32 epilogue compares distances at 16 ulp
+        assert np.max(np.abs(mind.astype(np.float64) - wmind)) <= (4 * np.sqrt(d) + 16) * eps * scale
         print("assign %s %s n=%d d=%d k=%d: %s" % (variant, np.dtype(dtype).name, n, d, k, rep))
 
 
