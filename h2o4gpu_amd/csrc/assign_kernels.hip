@@ -249,7 +249,16 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
         }
       }
     };
-    {
+#ifndef KM_PIPE
+#define KM_PIPE 1
+#endif
+    if (!KM_PIPE) {
+      for (int t = 0; t < KT; t++) {
+        acc_t acc[ROWT];
+        tile_mma(acc, t);
+        tile_argmin(acc, t);
+      }
+    } else {
       acc_t accA[ROWT], accB[ROWT];
       tile_mma(accA, 0);
       int t = 1;
@@ -673,7 +682,10 @@ struct RowstatDispatch<float, FUSE> {
                  int k, int num_cu, double *psums, int *pcounts, int *slots) {
     switch (rowstat_dp<float>(d)) {
       KM_ROWSTAT_CASE(float, 16, 2);
-      KM_ROWSTAT_CASE(float, 32, 2);
+#ifndef KM_ROWT_F32_32
+#define KM_ROWT_F32_32 2
+#endif
+      KM_ROWSTAT_CASE(float, 32, KM_ROWT_F32_32);
       KM_ROWSTAT_CASE(float, 64, 2);
       KM_ROWSTAT_CASE(float, 128, 1);
     }

@@ -9,7 +9,8 @@ import os
 import numpy as np
 
 _PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-LIB_PATH = os.path.join(_PKG, "libh2o4gpu_kmeans_hip.so")
+# H2O4GPU_KMEANS_LIB may point at another build of the same library
+LIB_PATH = os.environ.get("H2O4GPU_KMEANS_LIB") or os.path.join(_PKG, "libh2o4gpu_kmeans_hip.so")
 
 c_int = ctypes.c_int
 c_size_t = ctypes.c_size_t

@@ -1,0 +1,367 @@
+"""K-Means estimator with the interface of h2o4gpu.KMeans.
+
+Mirrors src/interface_py/h2o4gpu/solvers/kmeans.py of the reference: the same
+constructor arguments and defaults (:131-148, :685-702), attributes, dtype rule,
+argument order of the native calls (:369-372, :410-418, :485-497) and result shapes,
+on top of the gfx950 engine. Differences, all additive:
+  * `init` may be an ndarray of shape (n_clusters, n_features): it is passed to the
+    engine as starting centroids (init_from_data=2) instead of forcing the
+    scikit-learn backend;
+  * `inertia_` is filled after fit (the reference leaves it None, :187);
+  * when scikit-learn is chosen as backend it is the installed scikit-learn (the
+    reference uses its own renamed copy).
+"""
+import sys
+
+import numpy as np
+
+
+def _to_np(data):
+    """Reference solvers/utils.py:_get_data/_to_np for the dense-matrix case: numpy
+    array, 2-D, float32 unless the data already is float64/float32."""
+    if hasattr(data, "values") and not isinstance(data, np.ndarray):  # pandas
+        data = data.values
+    arr = np.asarray(data)
+    if arr.ndim == 1:
+        arr = arr.reshape(-1, 1)
+    if arr.dtype not in (np.float32, np.float64):
+        arr = arr.astype(np.float32)
+    return arr
+
+
+def _check_data_content(do_check, name, data):
+    """Reference solvers/utils.py:144-158."""
+    if do_check == 1:
+        assert np.isfinite(data).all(), "%s contains Inf" % name
+        assert not np.isnan(data).any(), "%s contains NA" % name
+
+
+def assert_satisfies(value, cond, message):
+    """Reference typecheck.typechecks.assert_satisfies, reduced to what the setters use."""
+    if not cond:
+        raise ValueError("%s (got %r)" % (message, value))
+
+
+class KMeansH2O:
+    """K-Means on the GPU (reference class KMeansH2O, kmeans.py:18-588)."""
+
+    def __init__(self, n_clusters=8, init='k-means++', n_init=1, max_iter=300, tol=1e-4,
+                 precompute_distances='auto', verbose=0, random_state=None, copy_x=True, n_jobs=1,
+                 algorithm='auto', gpu_id=0, n_gpus=-1, do_checks=1):
+        if isinstance(tol, np.floating):
+            tol = tol.item()
+        if isinstance(init, str) and init not in ['random', 'k-means++']:
+            raise ValueError("Invalid initialization method. Should be 'k-means++' or 'random' "
+                             "but got '%s'." % init)
+        self.init = init
+        self._n_clusters = n_clusters
+        self._gpu_id = gpu_id
+        from ..util.gpu import device_count
+        (self.n_gpus, self.devices) = device_count(n_gpus)
+        self._max_iter = max_iter
+        self.tol = tol
+        self._did_sklearn_fit = 0
+        self.verbose = verbose
+        self.do_checks = do_checks
+        self.n_init = n_init
+        self.precompute_distances = precompute_distances
+        self.copy_x = copy_x
+        self.n_jobs = n_jobs
+        self.algorithm = algorithm
+        if random_state is None:
+            import random
+            self.random_state = random.randint(0, 32000)
+        else:
+            self.random_state = random_state
+        self.cluster_centers_ = None
+        self.labels_ = None
+        self.inertia_ = None
+        self.sklearn_model = None
+        self.double_precision = 0
+
+    _PARAMS = ["algorithm", "copy_x", "do_checks", "gpu_id", "init", "max_iter", "n_clusters", "n_gpus",
+               "n_init", "n_jobs", "precompute_distances", "random_state", "tol", "verbose"]
+
+    @classmethod
+    def _get_param_names(cls):
+        return list(cls._PARAMS)
+
+    def get_params(self, deep=True):
+        return {key: getattr(self, key, None) for key in self._get_param_names()}
+
+    def set_params(self, **params):
+        valid = self.get_params(deep=True)
+        for key, value in params.items():
+            if key not in valid:
+                raise ValueError('Invalid parameter %s for estimator %s. Check the list of available '
+                                 'parameters with `estimator.get_params().keys()`.'
+                                 % (key, self.__class__.__name__))
+            setattr(self, key, value)
+        return self
+
+    def fit(self, X, y=None):
+        X_np = _to_np(X)
+        _check_data_content(self.do_checks, "X", X_np)
+        self._fit(X_np)
+        self._did_sklearn_fit = 0
+        return self
+
+    def sklearn_fit(self, X, y=None):
+        assert self.cluster_centers_ is not None, "Centroids are None. Run fit() first."
+        if self._did_sklearn_fit == 0:
+            X_np = _to_np(X)
+            _check_data_content(self.do_checks, "X", X_np)
+            self._did_sklearn_fit = 1
+            import sklearn.cluster as sk_cluster
+            self.sklearn_model = sk_cluster.KMeans(self._n_clusters, max_iter=1,
+                                                   init=self.cluster_centers_, n_init=1)
+            self.sklearn_model.fit(X_np)
+            self.sklearn_model.cluster_centers_ = self.cluster_centers_
+
+    def predict(self, X):
+        lib = self._load_lib()
+        cols, rows = self._validate_centroids(X)
+        X_np = _to_np(X)
+        _check_data_content(self.do_checks, "X", X_np)
+        c_X_np = self._toc(X_np)
+        cluster_centers_ = self._toc(self.cluster_centers_, convert=False)
+        c_res = np.zeros(rows, np.int32)
+        c_kmeans = lib.make_ptr_float_kmeans if self.double_precision == 0 else lib.make_ptr_double_kmeans
+        c_kmeans(1, self.verbose, self.random_state, self._gpu_id, self.n_gpus, rows, cols,
+                 self._n_clusters, self._max_iter, 0, self.tol, c_X_np, cluster_centers_,
+                 np.empty([], X_np.dtype), c_res)
+        return c_res
+
+    def sklearn_predict(self, X, y=None):
+        _check_data_content(self.do_checks, "X", X)
+        self.sklearn_fit(X)
+        return self.sklearn_model.predict(X)
+
+    def transform(self, X, y=None):
+        """Squared distances to every centre, shape (rows, n_clusters) (the reference returns
+        the squared values, kmeans.py:389-422 with kmeans_h2o4gpu.cu:937-950)."""
+        lib = self._load_lib()
+        cols, rows = self._validate_centroids(X)
+        X_np = _to_np(X)
+        c_X_np = self._toc(X_np)
+        cluster_centers_ = self._toc(self.cluster_centers_, convert=False)
+        c_res = np.zeros(rows * self._n_clusters, X_np.dtype)
+        if self.double_precision == 0:
+            lib.kmeans_transform_float(self.verbose, self._gpu_id, self.n_gpus, rows, cols,
+                                       self._n_clusters, c_X_np, cluster_centers_, c_res)
+        else:
+            lib.kmeans_transform_double(self.verbose, self._gpu_id, self.n_gpus, rows, cols,
+                                        self._n_clusters, c_X_np, cluster_centers_, c_res)
+        return np.reshape(c_res, (rows, self._n_clusters), order='F')
+
+    def sklearn_transform(self, X, y=None):
+        _check_data_content(self.do_checks, "X", X)
+        self.sklearn_fit(X)
+        return self.sklearn_model.transform(X)
+
+    def fit_transform(self, X, y=None):
+        return self.fit(X, y).transform(X)
+
+    def fit_predict(self, X, y=None):
+        return self.fit(X, y).labels_
+
+    def _fit(self, data):
+        lib = self._load_lib()
+        c_data = self._toc(data)
+        rows = np.shape(data)[0]
+        cols = np.shape(data)[1]
+        centroids = np.empty([])
+        if isinstance(self.init, np.ndarray):
+            init_arr = np.asarray(self.init)
+            assert init_arr.shape == (self._n_clusters, cols), \
+                "init must have shape (n_clusters, n_features)"
+            c_init = 2
+            centroids = np.ascontiguousarray(init_arr, dtype=data.dtype).flatten()
+        elif self.init == "k-means++":
+            c_init = 1
+        else:
+            c_init = 0
+        pred_centers = np.zeros(cols * self._n_clusters, data.dtype)
+        pred_labels = np.zeros(rows, dtype=np.int32)
+        fn = lib.make_ptr_float_kmeans if self.double_precision == 0 else lib.make_ptr_double_kmeans
+        status = fn(0, self.verbose, self.random_state, self._gpu_id, self.n_gpus, rows, cols,
+                    self._n_clusters, self._max_iter, c_init, self.tol, c_data, centroids,
+                    pred_centers, pred_labels)
+        if status != 0:
+            raise RuntimeError("KMeans fit failed in the native library (status %d)" % status)
+        self.cluster_centers_ = np.reshape(pred_centers, (self._n_clusters, cols))
+        self.labels_ = np.reshape(pred_labels, rows)
+        self.inertia_ = self._inertia(data)
+        return self.cluster_centers_, self.labels_
+
+    def _inertia(self, data):
+        """Sum of squared distances of the rows to their centre, from the fitted result."""
+        diff = data.astype(np.float64) - self.cluster_centers_.astype(np.float64)[self.labels_]
+        return float(np.einsum("ij,ij->", diff, diff))
+
+    def _toc(self, data, convert=True):
+        if convert and data.dtype != np.float64 and data.dtype != np.float32:
+            self._print_verbose(1, "Detected numeric data format which is not supported. "
+                                   "Casting to np.float32.")
+            data = np.asarray(data, dtype=np.float32)
+        if data.dtype == np.float64:
+            self._print_verbose(1, "Detected np.float64 data")
+            self.double_precision = 1
+        elif data.dtype == np.float32:
+            self._print_verbose(1, "Detected np.float32 data")
+            self.double_precision = 0
+        return data.flatten()
+
+    def _print_verbose(self, level, msg):
+        if self.verbose > level:
+            print(msg)
+            sys.stdout.flush()
+
+    def _load_lib(self):
+        """The native module, or None when no GPU can be used (the caller then falls back
+        to scikit-learn, as in the reference kmeans.py:532-546)."""
+        if (self.n_gpus == 0) or (self.devices == 0):
+            self._print_verbose(0, "H2O KMeans for CPU not yet supported.")
+            return None
+        from ..libs import ch2o4gpu_gpu
+        self._print_verbose(0, "\nUsing GPU KMeans solver with %d GPUs.\n" % self.n_gpus)
+        return ch2o4gpu_gpu
+
+    def _validate_centroids(self, X):
+        assert self.cluster_centers_ is not None, "Centroids are None. Run fit() first."
+        rows = np.shape(X)[0]
+        cols = np.shape(X)[1]
+        centroids_dim = np.shape(self.cluster_centers_)[1]
+        assert cols == centroids_dim, \
+            "The dimension of X [%d] and centroids [%d] is not equal." % (cols, centroids_dim)
+        return cols, rows
+
+    @property
+    def n_clusters(self):
+        return self._n_clusters
+
+    @n_clusters.setter
+    def n_clusters(self, value):
+        assert_satisfies(value, value > 0, "Number of clusters must be positive.")
+        self._n_clusters = value
+
+    @property
+    def gpu_id(self):
+        return self._gpu_id
+
+    @gpu_id.setter
+    def gpu_id(self, value):
+        assert_satisfies(value, value >= 0, "GPU ID must be non-negative.")
+        self._gpu_id = value
+
+    @property
+    def max_iter(self):
+        return self._max_iter
+
+    @max_iter.setter
+    def max_iter(self, value):
+        assert_satisfies(value, value > 0, "Number of maximum iterations must be non-negative.")
+        self._max_iter = value
+
+
+class KMeans:
+    """Backend selector (reference class KMeans, kmeans.py:591-829): 'auto' uses the GPU
+    engine when a device is usable, 'sklearn' forces scikit-learn, 'h2o4gpu' forces the
+    engine. The environment variable H2O4GPU_BACKEND overrides the argument."""
+
+    def __init__(self, n_clusters=8, init='k-means++', n_init=1, max_iter=300, tol=1e-4,
+                 precompute_distances='auto', verbose=0, random_state=None, copy_x=True, n_jobs=1,
+                 algorithm='auto', gpu_id=0, n_gpus=-1, do_checks=1, backend='auto'):
+        import os
+        _backend = os.environ.get('H2O4GPU_BACKEND', None)
+        if _backend is not None:
+            backend = _backend
+        self.do_sklearn = backend == 'sklearn'
+        if backend == 'auto' and n_init != 1:
+            KMeans._print_verbose(verbose, 0, "'n_init' not supported. Running h2o4gpu with n_init = 1.")
+        self.model_h2o4gpu = KMeansH2O(n_clusters=n_clusters, init=init, n_init=n_init, max_iter=max_iter,
+                                       tol=tol, precompute_distances=precompute_distances,
+                                       verbose=verbose, random_state=random_state, copy_x=copy_x,
+                                       n_jobs=n_jobs, algorithm=algorithm, gpu_id=gpu_id, n_gpus=n_gpus,
+                                       do_checks=do_checks)
+        self._sk_args = dict(n_clusters=n_clusters, init=init, n_init=n_init, max_iter=max_iter, tol=tol,
+                             verbose=verbose, random_state=random_state, copy_x=copy_x)
+        self.model_sklearn = None
+        # scikit-learn is used only when asked for (backend='sklearn' or n_gpus=0). The
+        # reference also drops to scikit-learn silently when no GPU library or device is
+        # found (kmeans.py:766-773); here that case raises instead, so a missing build or
+        # device is never mistaken for a GPU run.
+        # pylint: disable=protected-access
+        if not self.do_sklearn and n_gpus != 0 and self.model_h2o4gpu._load_lib() is None:
+            raise RuntimeError("KMeans(backend=%r): no usable GPU (visible devices: %d). Pass "
+                               "backend='sklearn' or n_gpus=0 to run scikit-learn on the CPU."
+                               % (backend, self.model_h2o4gpu.devices))
+        if self.do_sklearn or n_gpus == 0:
+            if backend == 'h2o4gpu':
+                raise RuntimeError("backend='h2o4gpu' was requested with n_gpus=0")
+            self.backend = 'sklearn'
+            self.model = self._sklearn()
+            KMeans._print_verbose(verbose, 0, "Using ScikitLearn backend.")
+        else:
+            self.backend = 'h2o4gpu'
+            self.model = self.model_h2o4gpu
+            KMeans._print_verbose(verbose, 0, "Using h2o4gpu backend.")
+        self.cluster_centers_ = None
+        self.labels_ = None
+        self.inertia_ = None
+
+    def _sklearn(self):
+        if self.model_sklearn is None:
+            import sklearn.cluster as sk_cluster
+            self.model_sklearn = sk_cluster.KMeans(**self._sk_args)
+        return self.model_sklearn
+
+    def fit(self, X, y=None):
+        res = self.model.fit(X, y)
+        self.set_attributes()
+        return res
+
+    def fit_predict(self, X, y=None):
+        res = self.model.fit_predict(X, y)
+        self.set_attributes()
+        return res
+
+    def fit_transform(self, X, y=None):
+        res = self.model.fit_transform(X, y)
+        self.set_attributes()
+        return res
+
+    def get_params(self, deep=True):
+        return self.model.get_params(deep)
+
+    def predict(self, X):
+        res = self.model.predict(X)
+        self.set_attributes()
+        return res
+
+    def score(self, X, y=None):
+        """Opposite of the k-means objective on X (scikit-learn's definition)."""
+        if self.backend == 'sklearn':
+            return self.model.score(X, y)
+        D = self.model.transform(X)
+        return -float(np.min(D, axis=1).astype(np.float64).sum())
+
+    def set_params(self, **params):
+        res = self.model.set_params(**params)
+        self.set_attributes()
+        return res
+
+    def transform(self, X):
+        res = self.model.transform(X)
+        self.set_attributes()
+        return res
+
+    def set_attributes(self):
+        for name in ("cluster_centers_", "labels_", "inertia_"):
+            setattr(self, name, getattr(self.model, name, None))
+
+    @staticmethod
+    def _print_verbose(verbose, level, msg):
+        if verbose > level:
+            print(msg)
+            sys.stdout.flush()
