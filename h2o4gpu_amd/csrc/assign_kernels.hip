@@ -320,20 +320,27 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
 // MFMA tiled variant (any d, any k). A workgroup owns BR = 128 data rows and
 // walks over centroid blocks of BC = 128; for each block it runs the d-loop in
 // steps of BK features with both operand tiles staged through LDS in operand
-// order (double buffered). The four wavefronts split the block 2 x 2, each
+// order (double buffered, next stage's global loads in flight during the
+// current stage's matrix work). The four wavefronts split the block 2 x 2, each
 // holding (BC/2/MT) x (BR/2/MT) result tiles in accumulators.
 // MODE 0: running argmin kept in registers across centroid blocks, halves
 // merged through LDS at the end.  MODE 1: |acc| stored to D[c*ldn + i].
+//
+// Preconditions (the engine's buffers satisfy them): C holds round_up(k, BC)
+// rows and cnorm round_up(k, BC) entries, the entries past k being +inf, so the
+// loads need no bounds test on the centroid axis; rows past n re-read row n-1.
+// A feature tail (d not a multiple of BK, DTAIL) re-reads in-bounds features on
+// the data side and zeroes the centroid side.
 // ---------------------------------------------------------------------------
 template <typename T>
 struct TiledCfg {
   static constexpr int BC = 128;
-  static constexpr int BR = 128;
+  static constexpr int BR = sizeof(T) == 4 ? 128 : 64;  // double: half the rows, same register budget
   static constexpr int BK = sizeof(T) == 4 ? 32 : 16;
 };
 
-template <typename T, int MODE, bool VECLOAD>
-__global__ __launch_bounds__(WG) void assign_tiled_kernel(
+template <typename T, int MODE, bool VECLOAD, bool DTAIL>
+__global__ __launch_bounds__(WG, 2) void assign_tiled_kernel(
     const T *__restrict__ X, const T *__restrict__ xnorm,
     const T *__restrict__ C, const T *__restrict__ cnorm,
     int *__restrict__ labels, T *__restrict__ mindist, T *__restrict__ D,
@@ -350,8 +357,9 @@ __global__ __launch_bounds__(WG) void assign_tiled_kernel(
   constexpr int A_ELEMS = (BC / MT) * TILE_ELEMS;   // = BC*BK
   constexpr int B_ELEMS = (BR / MT) * TILE_ELEMS;
   constexpr int VEC_PER_ROW = BK / VW;              // 16-byte vectors per operand row per stage
-  constexpr int A_VECS = BC * VEC_PER_ROW / WG;     // vectors each thread stages for A
-  constexpr int B_VECS = BR * VEC_PER_ROW / WG;
+  constexpr int ROWS_PER_PASS = WG / VEC_PER_ROW;   // operand rows one pass of the workgroup covers
+  constexpr int A_VECS = BC / ROWS_PER_PASS;        // vectors each thread stages for A
+  constexpr int B_VECS = BR / ROWS_PER_PASS;
   typedef typename M::acc_t acc_t;
   typedef typename M::vec_t vec_t;
 
@@ -370,83 +378,82 @@ __global__ __launch_bounds__(WG) void assign_tiled_kernel(
   const int64_t row0 = (int64_t)blockIdx.x * BR;
   const int nstage = (d + BK - 1) / BK;
 
-  // element (row rr of the operand block, features [j0, j0+VW)) goes to
-  // tile rr/MT, lane group (jj/DCH), slot s = jj%DCH as one 16-byte store.
-  auto lds_slot = [&](int rr, int jj) -> int {
+  // staging role of this thread: operand row rr0 + q*ROWS_PER_PASS, features
+  // [jj, jj+VW) of the stage. The 16-byte vector lands in LDS at tile rr/MT,
+  // lane group jj/DCH, slot jj%DCH (operand order).
+  const int rr0 = tid / VEC_PER_ROW;
+  const int jj = (tid - rr0 * VEC_PER_ROW) * VW;
+  int lds_off[A_VECS > B_VECS ? A_VECS : B_VECS];
+#pragma unroll
+  for (int q = 0; q < (A_VECS > B_VECS ? A_VECS : B_VECS); q++) {
+    const int rr = rr0 + q * ROWS_PER_PASS;
     const int t = rr / MT, i = rr - t * MT, gg = jj / DCH, s = jj - gg * DCH;
-    return ((t * NV + s / VW) * 64 + gg * MT + i) * VW;
-  };
+    lds_off[q] = ((t * NV + s / VW) * 64 + gg * MT + i) * VW;
+  }
+  const T *xrow[B_VECS];
+#pragma unroll
+  for (int q = 0; q < B_VECS; q++)
+    xrow[q] = X + min(row0 + rr0 + q * ROWS_PER_PASS, n - 1) * (int64_t)d;
 
   T xx[RT];
 #pragma unroll
-  for (int rt = 0; rt < RT; rt++) {
-    const int64_t row = row0 + (wr * RT + rt) * MT + r;
-    xx[rt] = row < n ? xnorm[row] : (T)0;
-  }
+  for (int rt = 0; rt < RT; rt++)
+    xx[rt] = xnorm[min(row0 + (wr * RT + rt) * MT + r, n - 1)];
   T best[RT];
   int bidx[RT];
+  unsigned bkey[RT];
+  int bblk[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; rt++) {
     best[rt] = argmin_start<T>();
     bidx[rt] = -1;
+    bkey[rt] = 0x7F7FFFF0u;  // first tile start (a multiple of MT) of the best key
+    bblk[rt] = -1;
   }
 
   vec_t areg[A_VECS], breg[B_VECS];
   auto gload = [&](int c0, int st) {
-    const int j0 = st * BK;
+    int j = st * BK + jj;
+    bool jok = true;
+    if (DTAIL) {
+      jok = j < d;
+      j = VECLOAD ? min(j, d - VW) : j;
+    }
+    const T *cbase = C + (size_t)(c0 + rr0) * d;
 #pragma unroll
     for (int q = 0; q < A_VECS; q++) {
-      const int vi = tid + q * WG;
-      const int rr = vi / VEC_PER_ROW, jj = (vi - rr * VEC_PER_ROW) * VW;
-      const int c = c0 + rr, j = j0 + jj;
+      const T *src = cbase + (size_t)q * ROWS_PER_PASS * d;
       vec_t v;
       if (VECLOAD) {
-        if (c < k && j < d)
-          v = *reinterpret_cast<const vec_t *>(C + (size_t)c * d + j);
-        else
+        v = *reinterpret_cast<const vec_t *>(src + j);
+        if (DTAIL && !jok)
 #pragma unroll
           for (int e = 0; e < VW; e++) v[e] = 0;
       } else {
 #pragma unroll
-        for (int e = 0; e < VW; e++)
-          v[e] = (c < k && j + e < d) ? C[(size_t)c * d + j + e] : (T)0;
+        for (int e = 0; e < VW; e++) v[e] = (j + e < d) ? src[min(j + e, d - 1)] : (T)0;
       }
       areg[q] = v * (T)-2;
     }
 #pragma unroll
     for (int q = 0; q < B_VECS; q++) {
-      const int vi = tid + q * WG;
-      const int rr = vi / VEC_PER_ROW, jj = (vi - rr * VEC_PER_ROW) * VW;
-      const int64_t row = row0 + rr;
-      const int j = j0 + jj;
       vec_t v;
       if (VECLOAD) {
-        if (row < n && j < d)
-          v = *reinterpret_cast<const vec_t *>(X + row * (int64_t)d + j);
-        else
-#pragma unroll
-          for (int e = 0; e < VW; e++) v[e] = 0;
+        v = *reinterpret_cast<const vec_t *>(xrow[q] + j);
       } else {
 #pragma unroll
-        for (int e = 0; e < VW; e++)
-          v[e] = (row < n && j + e < d) ? X[row * (int64_t)d + j + e] : (T)0;
+        for (int e = 0; e < VW; e++) v[e] = xrow[q][min(j + e, d - 1)];
       }
       breg[q] = v;
     }
   };
   auto lstore = [&](int buf) {
 #pragma unroll
-    for (int q = 0; q < A_VECS; q++) {
-      const int vi = tid + q * WG;
-      const int rr = vi / VEC_PER_ROW, jj = (vi - rr * VEC_PER_ROW) * VW;
-      *reinterpret_cast<vec_t *>(As + buf * A_ELEMS + lds_slot(rr, jj)) = areg[q];
-    }
+    for (int q = 0; q < A_VECS; q++)
+      *reinterpret_cast<vec_t *>(As + buf * A_ELEMS + lds_off[q]) = areg[q];
 #pragma unroll
-    for (int q = 0; q < B_VECS; q++) {
-      const int vi = tid + q * WG;
-      const int rr = vi / VEC_PER_ROW, jj = (vi - rr * VEC_PER_ROW) * VW;
-      *reinterpret_cast<vec_t *>(Bs + buf * B_ELEMS + lds_slot(rr, jj)) = breg[q];
-    }
+    for (int q = 0; q < B_VECS; q++)
+      *reinterpret_cast<vec_t *>(Bs + buf * B_ELEMS + lds_off[q]) = breg[q];
   };
 
   for (int c0 = 0; c0 < k; c0 += BC) {
@@ -455,8 +462,7 @@ __global__ __launch_bounds__(WG) void assign_tiled_kernel(
     for (int ct = 0; ct < CT; ct++) {
 #pragma unroll
       for (int v = 0; v < NACC; v++) {
-        const int c = c0 + (wc * CT + ct) * MT + M::acc_row(v, g);
-        const T cc = c < k ? cnorm[c] : pos_inf<T>();
+        const T cc = cnorm[c0 + (wc * CT + ct) * MT + M::acc_row(v, g)];
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) acc[ct][rt][v] = xx[rt] + cc;
       }
@@ -493,26 +499,65 @@ __global__ __launch_bounds__(WG) void assign_tiled_kernel(
       }
     }
     // epilogue for this centroid block
+    if (MODE == 1) {
 #pragma unroll
-    for (int ct = 0; ct < CT; ct++) {
+      for (int ct = 0; ct < CT; ct++) {
 #pragma unroll
-      for (int v = 0; v < NACC; v++) {
-        const int c = c0 + (wc * CT + ct) * MT + M::acc_row(v, g);
+        for (int v = 0; v < NACC; v++) {
+          const int c = c0 + (wc * CT + ct) * MT + M::acc_row(v, g);
+#pragma unroll
+          for (int rt = 0; rt < RT; rt++) {
+            const int64_t row = row0 + (wr * RT + rt) * MT + r;
+            if (c < k && row < n) D[(size_t)c * ldn + row] = fabs(acc[ct][rt][v]);
+          }
+        }
+      }
+    } else if constexpr (sizeof(T) == 4) {
+      // integer keys as in the row-stationary kernel (4 index bits, 16 ulp)
+#pragma unroll
+      for (int ct = 0; ct < CT; ct++) {
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
-          const T dist = fabs(acc[ct][rt][v]);
-          if (MODE == 1) {
-            const int64_t row = row0 + (wr * RT + rt) * MT + r;
-            if (c < k && row < n) D[(size_t)c * ldn + row] = dist;
-          } else if (dist < best[rt]) {
-            best[rt] = dist;
-            bidx[rt] = c;
+          unsigned key[NACC];
+#pragma unroll
+          for (int v = 0; v < NACC; v++)
+            key[v] = (__float_as_uint(acc[ct][rt][v]) & 0x7FFFFFF0u) | (unsigned)v;
+          unsigned m = umin3(key[0], key[1], key[2]);
+#pragma unroll
+          for (int v = 3; v + 1 < NACC; v += 2) m = umin3(m, key[v], key[v + 1]);
+          if ((NACC & 1) == 0) m = min(m, key[NACC - 1]);
+          if (m < bkey[rt]) {
+            bkey[rt] = m;
+            bblk[rt] = c0 + (wc * CT + ct) * MT;
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int ct = 0; ct < CT; ct++) {
+#pragma unroll
+        for (int v = 0; v < NACC; v++) {
+          const int c = c0 + (wc * CT + ct) * MT + M::acc_row(v, g);
+#pragma unroll
+          for (int rt = 0; rt < RT; rt++) {
+            const T dist = fabs(acc[ct][rt][v]);
+            if (dist < best[rt]) {
+              best[rt] = dist;
+              bidx[rt] = c;
+            }
           }
         }
       }
     }
   }
   if (MODE == 0) {
+    if constexpr (sizeof(T) == 4) {
+#pragma unroll
+      for (int rt = 0; rt < RT; rt++) {
+        best[rt] = __uint_as_float(bkey[rt] & 0xFFFFFFF0u);
+        bidx[rt] = bblk[rt] < 0 ? -1 : bblk[rt] + key_row(bkey[rt] & 15u, g);
+      }
+    }
     // lane groups of one wavefront, then the two wavefronts sharing the rows
 #pragma unroll
     for (int rt = 0; rt < RT; rt++) {
@@ -736,12 +781,14 @@ static int launch_tiled(hipStream_t s, const T *X, const T *xnorm, const T *C,
   const int vw = Mfma<T>::VW;
   const bool vec = (d % vw == 0) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0) &&
                    ((reinterpret_cast<uintptr_t>(C) & 15) == 0);
-  if (vec)
-    hipLaunchKernelGGL((assign_tiled_kernel<T, MODE, true>), grid, dim3(WG), lds, s,
-                       X, xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k);
-  else
-    hipLaunchKernelGGL((assign_tiled_kernel<T, MODE, false>), grid, dim3(WG), lds, s,
-                       X, xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k);
+  const bool tail = (d % Cfg::BK) != 0;
+#define KM_TILED(VEC, TAIL)                                                               \
+  hipLaunchKernelGGL((assign_tiled_kernel<T, MODE, VEC, TAIL>), grid, dim3(WG), lds, s, X, \
+                     xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k)
+  if (vec && !tail) KM_TILED(true, false);
+  else if (vec) KM_TILED(true, true);
+  else KM_TILED(false, true);
+#undef KM_TILED
   KM_HIP_TRY(hipGetLastError());
   return 0;
 }

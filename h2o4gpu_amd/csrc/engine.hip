@@ -13,6 +13,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <ctime>
+#include <limits>
 #include <map>
 #include <numeric>
 #include <random>
@@ -228,9 +229,20 @@ struct Engine : h2o4gpu_kmeans_handle {
     KM_HIP_TRY(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
     plan = plan_update<T>(n, d, k, num_cu);
     const size_t kd = (size_t)k * d;
-    KM_TRY(dalloc(&C[0], kd));
-    KM_TRY(dalloc(&C[1], kd));
-    KM_TRY(dalloc(&cnorm, k));
+    // Centroid buffers are padded to a multiple of CENTROID_PAD rows (zeros) and the
+    // norms to as many entries (+inf): the tiled MFMA kernels read whole centroid
+    // blocks without bounds tests and the padding can never win an argmin.
+    const size_t kpad = ((size_t)k + CENTROID_PAD - 1) / CENTROID_PAD * CENTROID_PAD;
+    KM_TRY(dalloc(&C[0], kpad * d));
+    KM_TRY(dalloc(&C[1], kpad * d));
+    KM_TRY(dalloc(&cnorm, kpad));
+    KM_HIP_TRY(hipMemsetAsync(C[0], 0, kpad * d * sizeof(T), stream));
+    KM_HIP_TRY(hipMemsetAsync(C[1], 0, kpad * d * sizeof(T), stream));
+    {
+      std::vector<T> inf(kpad, std::numeric_limits<T>::infinity());
+      KM_HIP_TRY(hipMemcpyAsync(cnorm, inf.data(), kpad * sizeof(T), hipMemcpyHostToDevice, stream));
+      KM_HIP_TRY(hipStreamSynchronize(stream));
+    }
     KM_TRY(dalloc(&counts, k));
     KM_TRY(dalloc(&labels, n));
     KM_TRY(dalloc(&xnorm, n));

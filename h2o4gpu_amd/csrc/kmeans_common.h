@@ -50,6 +50,10 @@ enum AssignVariant {
   ASSIGN_TILED = 3     // MFMA, both operands staged through LDS over a d-loop
 };
 
+// Rows the centroid buffer C (zeros) and entries the norm buffer cnorm (+inf) must
+// be padded to: launch_assign / launch_transform may read that far.
+static const int CENTROID_PAD = 128;
+
 // Fused distance + argmin. labels[i] = argmin_c |(xx_i + cc_c) - 2 x_i.c_c|,
 // strict '<', lowest index wins, -1 when no distance is below FLT_MAX.
 // mindist (nullable) receives the minimum. Returns the variant actually used
