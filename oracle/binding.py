@@ -151,6 +151,11 @@ class Oracle:
                                              _int(threads))
         return da, db
 
+    def set_dot_order(self, descending):
+        """Summation order of the distance dot product: features ascending (False,
+        default) or descending (True)."""
+        self.lib.oracle_set_dot_order(_int(1 if descending else 0))
+
     def random_rows(self, seed, n, k):
         idx = np.empty(k, np.int32)
         self.lib.oracle_random_rows(_int(seed), _i64(n), _int(k), _ptr(idx))

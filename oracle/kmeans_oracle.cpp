@@ -72,6 +72,11 @@ std::vector<T> transpose_centroids(int d, int k, const T *C) {
   return Ct;
 }
 
+// Summation order of the dot product: 0 = features ascending (default), 1 =
+// descending. The reference leaves this order to cuBLAS; the switch exists so a
+// test can measure how much a fixed-iteration trajectory depends on it.
+static int g_dot_order = 0;
+
 // dist(row, c) = | (xx + cc[c]) - 2 * dot(x, C[c]) |
 // Reference: all_dots writes xx + cc (kmeans_labels.h:216-244); the GEMM then
 // forms alpha*dot + beta*D with alpha=-2, beta=1 (kmeans_labels.cu:183-228);
@@ -82,7 +87,9 @@ template <typename T>
 __attribute__((target_clones("avx2", "default"))) void
 dist_row(int d, int k, const T *x, T xx, const T *Ct, const T *cc, T *acc) {
   for (int c = 0; c < k; c++) acc[c] = 0;
-  for (int j = 0; j < d; j++) {
+  const int order = g_dot_order;
+  for (int jj = 0; jj < d; jj++) {
+    const int j = order ? d - 1 - jj : jj;
     const T xj = x[j];
     const T *ct = Ct + (size_t)j * k;
     for (int c = 0; c < k; c++) acc[c] += xj * ct[c];
@@ -161,27 +168,17 @@ void distances(int64_t n, int d, int k, const T *X, const T *C, T *D,
 //   the sum of its label (calculate_centroids :40-75), restore the old
 //   centroid where count < 1 (revert_zeroed_centroids :77-88), multiply by
 //   1/T(max(count,1)) (scale_centroids :90-105; reciprocal then multiply).
-// The reference adds with floating-point atomics in no fixed order; this
-// restatement adds rows in ascending row order. With several threads each
-// thread sums a contiguous block of rows and blocks are combined in thread
-// order. Rows with a negative label are skipped.
+// The reference adds with floating-point atomics in no fixed order, so the
+// order of the additions is not part of its semantics. This restatement adds
+// in double and rounds the total to T once: for float data whose column values
+// span fewer than ~20 binades every partial sum is exact, so the result is the
+// correctly rounded sum whatever the order or the number of threads. Rows with
+// a label outside [0, k) are skipped.
 template <typename T>
 void update_sums(int64_t n, int d, int k, const T *X, const int *labels,
                  T *sums, int *counts, int threads) {
-  std::fill(sums, sums + (size_t)k * d, (T)0);
-  std::fill(counts, counts + k, 0);
-  if (threads <= 1) {
-    for (int64_t i = 0; i < n; i++) {
-      int l = labels[i];
-      if (l < 0 || l >= k) continue;
-      counts[l]++;
-      T *s = sums + (size_t)l * d;
-      const T *x = X + i * (int64_t)d;
-      for (int j = 0; j < d; j++) s[j] += x[j];
-    }
-    return;
-  }
-  std::vector<std::vector<T>> psum(threads);
+  if (threads < 1) threads = 1;
+  std::vector<std::vector<double>> psum(threads);
   std::vector<std::vector<int>> pcnt(threads);
 #pragma omp parallel num_threads(threads)
   {
@@ -190,23 +187,26 @@ void update_sums(int64_t n, int d, int k, const T *X, const int *labels,
     t = omp_get_thread_num();
     nt = omp_get_num_threads();
 #endif
-    psum[t].assign((size_t)k * d, (T)0);
+    psum[t].assign((size_t)k * d, 0.0);
     pcnt[t].assign(k, 0);
     int64_t lo = n * t / nt, hi = n * (t + 1) / nt;
     for (int64_t i = lo; i < hi; i++) {
       int l = labels[i];
       if (l < 0 || l >= k) continue;
       pcnt[t][l]++;
-      T *s = psum[t].data() + (size_t)l * d;
+      double *s = psum[t].data() + (size_t)l * d;
       const T *x = X + i * (int64_t)d;
-      for (int j = 0; j < d; j++) s[j] += x[j];
+      for (int j = 0; j < d; j++) s[j] += (double)x[j];
     }
   }
+  std::vector<double> tot((size_t)k * d, 0.0);
+  std::fill(counts, counts + k, 0);
   for (int t = 0; t < threads; t++) {
     if (psum[t].empty()) continue;
-    for (size_t e = 0; e < (size_t)k * d; e++) sums[e] += psum[t][e];
+    for (size_t e = 0; e < (size_t)k * d; e++) tot[e] += psum[t][e];
     for (int c = 0; c < k; c++) counts[c] += pcnt[t][c];
   }
+  for (size_t e = 0; e < (size_t)k * d; e++) sums[e] = (T)tot[e];
 }
 
 template <typename T>
@@ -326,6 +326,8 @@ void pair_dist_exact(int64_t n, int d, const T *X, const T *C, const int *a,
 extern "C" {
 
 #define ORACLE_EXPORT __attribute__((visibility("default")))
+
+ORACLE_EXPORT void oracle_set_dot_order(int order) { g_dot_order = order ? 1 : 0; }
 
 ORACLE_EXPORT int oracle_max_threads(void) {
 #ifdef _OPENMP
