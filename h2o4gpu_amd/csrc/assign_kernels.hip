@@ -148,11 +148,11 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
 
   constexpr int ROWS_PER_WAVE = ROWT * MT;
   constexpr int ROWS_PER_WG = NW * ROWS_PER_WAVE;
-  for (int64_t base = (int64_t)blockIdx.x * ROWS_PER_WG; base < n;
-       base += (int64_t)gridDim.x * ROWS_PER_WG) {
-    const int64_t wrow0 = base + (int64_t)wave * ROWS_PER_WAVE;
-    T x[ROWT][DCH];
-    T xx[ROWT];
+  // The rows of the next tile are fetched while the current tile is swept, so
+  // the only exposed memory latency is that of the first tile.
+  T xn[ROWT][DCH];
+  T xxn[ROWT];
+  auto fetch_rows = [&](int64_t wrow0) {
 #pragma unroll
     for (int rt = 0; rt < ROWT; rt++) {
       // rows past the end re-read the last row; their results are never stored
@@ -163,17 +163,34 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
         for (int q = 0; q < NV; q++) {
           vec_t v = src[q];
 #pragma unroll
-          for (int e = 0; e < VW; e++) x[rt][q * VW + e] = v[e];
+          for (int e = 0; e < VW; e++) xn[rt][q * VW + e] = v[e];
         }
       } else {
         const T *src = X + row * (int64_t)d;
 #pragma unroll
         for (int s = 0; s < DCH; s++) {
           const int j = g * DCH + s;
-          x[rt][s] = j < d ? src[j] : (T)0;
+          xn[rt][s] = j < d ? src[j] : (T)0;
         }
       }
-      xx[rt] = xnorm[row];
+      xxn[rt] = xnorm[row];
+    }
+  };
+  const int64_t base0 = (int64_t)blockIdx.x * ROWS_PER_WG;
+  if (base0 < n) fetch_rows(base0 + (int64_t)wave * ROWS_PER_WAVE);
+  for (int64_t base = base0; base < n; base += (int64_t)gridDim.x * ROWS_PER_WG) {
+    const int64_t wrow0 = base + (int64_t)wave * ROWS_PER_WAVE;
+    T x[ROWT][DCH];
+    T xx[ROWT];
+#pragma unroll
+    for (int rt = 0; rt < ROWT; rt++) {
+#pragma unroll
+      for (int s = 0; s < DCH; s++) x[rt][s] = xn[rt][s];
+      xx[rt] = xxn[rt];
+    }
+    {
+      const int64_t nbase = base + (int64_t)gridDim.x * ROWS_PER_WG;
+      if (nbase < n) fetch_rows(nbase + (int64_t)wave * ROWS_PER_WAVE);
     }
     T best[ROWT];
     int bidx[ROWT];
@@ -250,7 +267,7 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
       }
     };
 #ifndef KM_PIPE
-#define KM_PIPE 1
+#define KM_PIPE 0
 #endif
     if (!KM_PIPE) {
       for (int t = 0; t < KT; t++) {
@@ -710,8 +727,13 @@ static int launch_rowstat_dp(hipStream_t s, const T *X, const T *xnorm,
   if (rowstat_two_per_cu(lds))
     return launch_rowstat_nw<T, DP, ROWT, FUSE, 4>(s, X, xnorm, C, cnorm, labels, mindist, n, d,
                                                    k, num_cu, psums, pcounts, slots, lds);
-  return launch_rowstat_nw<T, DP, ROWT, FUSE, 8>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k,
-                                                 num_cu, psums, pcounts, slots, lds);
+  // one workgroup per CU: as many wavefronts as the register budget allows
+  if constexpr (sizeof(T) == 4 && DP <= 32)
+    return launch_rowstat_nw<T, DP, ROWT, FUSE, 16>(s, X, xnorm, C, cnorm, labels, mindist, n, d,
+                                                    k, num_cu, psums, pcounts, slots, lds);
+  else
+    return launch_rowstat_nw<T, DP, ROWT, FUSE, 8>(s, X, xnorm, C, cnorm, labels, mindist, n, d,
+                                                   k, num_cu, psums, pcounts, slots, lds);
 }
 
 template <typename T, bool FUSE>
