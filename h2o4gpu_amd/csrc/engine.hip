@@ -108,6 +108,7 @@ struct h2o4gpu_kmeans_handle {
   virtual int set_centroids_host(const void *C) = 0;
   virtual int init_random_rows(int seed) = 0;
   virtual int init_plusplus(int seed) = 0;
+  std::vector<int> last_seed_rows;
   virtual int fit(int max_iterations, double threshold, int *iters) = 0;
   virtual int assign() = 0;
   virtual int update(double *shift2) = 0;
@@ -338,6 +339,7 @@ struct Engine : h2o4gpu_kmeans_handle {
       std::random_device rd;
       std::shuffle(v.begin(), v.end(), std::default_random_engine(rd()));
     }
+    last_seed_rows.assign(v.begin(), v.begin() + k);
     return init_from_rows(v.data());
   }
 
@@ -409,11 +411,10 @@ struct Engine : h2o4gpu_kmeans_handle {
       }
       idx[c] = (int)pick;
     }
-    have_mindist = false;
+    have_mindist = true;  // minimum distance of every row to the k chosen centres
     last_seed_rows = idx;
     return init_from_rows(idx.data());
   }
-  std::vector<int> last_seed_rows;
 
   int assign() override {
     KM_HIP_TRY(hipSetDevice(dev));
@@ -805,6 +806,12 @@ KM_API int h2o4gpu_kmeans_init_random_rows(h2o4gpu_kmeans_handle *h, int seed) {
 KM_API int h2o4gpu_kmeans_init_plusplus(h2o4gpu_kmeans_handle *h, int seed) {
   KM_CHECK_HANDLE(h);
   return h->init_plusplus(seed);
+}
+KM_API int h2o4gpu_kmeans_get_seed_rows(h2o4gpu_kmeans_handle *h, int *rows) {
+  KM_CHECK_HANDLE(h);
+  if (!rows || (int)h->last_seed_rows.size() != h->k) return H2O4GPU_KMEANS_ESTATE;
+  memcpy(rows, h->last_seed_rows.data(), (size_t)h->k * sizeof(int));
+  return 0;
 }
 KM_API int h2o4gpu_kmeans_fit(h2o4gpu_kmeans_handle *h, int max_iterations, double threshold,
                               int *iterations_run) {

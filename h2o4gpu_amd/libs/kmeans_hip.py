@@ -46,6 +46,7 @@ PROTOTYPES = {
     "h2o4gpu_kmeans_set_centroids_host": (c_int, [c_void_p, c_void_p]),
     "h2o4gpu_kmeans_init_random_rows": (c_int, [c_void_p, c_int]),
     "h2o4gpu_kmeans_init_plusplus": (c_int, [c_void_p, c_int]),
+    "h2o4gpu_kmeans_get_seed_rows": (c_int, [c_void_p, c_void_p]),
     "h2o4gpu_kmeans_fit": (c_int, [c_void_p, c_int, c_double, P(c_int)]),
     "h2o4gpu_kmeans_assign": (c_int, [c_void_p]),
     "h2o4gpu_kmeans_update": (c_int, [c_void_p, P(c_double)]),
@@ -173,6 +174,11 @@ class Handle:
 
     def init_plusplus(self, seed):
         _check("init_plusplus", lib().h2o4gpu_kmeans_init_plusplus(self._h, seed))
+
+    def seed_rows(self):
+        out = np.empty(self.k, np.int32)
+        _check("get_seed_rows", lib().h2o4gpu_kmeans_get_seed_rows(self._h, _vp(out)))
+        return out
 
     def fit(self, max_iter, threshold=0.0):
         it = c_int(0)

@@ -124,6 +124,8 @@ int h2o4gpu_kmeans_set_data_device(h2o4gpu_kmeans_handle *h, const void *d_X);
 int h2o4gpu_kmeans_set_centroids_host(h2o4gpu_kmeans_handle *h, const void *C);
 int h2o4gpu_kmeans_init_random_rows(h2o4gpu_kmeans_handle *h, int seed);
 int h2o4gpu_kmeans_init_plusplus(h2o4gpu_kmeans_handle *h, int seed);
+/* Row indices the last init_random_rows / init_plusplus call chose ([k] int32). */
+int h2o4gpu_kmeans_get_seed_rows(h2o4gpu_kmeans_handle *h, int *rows);
 
 /* The reference's loop (kmeans_impl.h:109-232): up to max_iterations of
  * assign + update, stop when shift^2 < threshold, final assignment with the

@@ -161,6 +161,16 @@ class Oracle:
         self.lib.oracle_random_rows(_int(seed), _i64(n), _int(k), _ptr(idx))
         return idx
 
+    def kmeanspp(self, X, k, seed):
+        """Rows chosen by k-means++ (D^2 sampling) and the final minimum distances."""
+        X, _ = self._prep(X)
+        n, d = X.shape
+        rows = np.empty(k, np.int32)
+        mind = np.empty(n, X.dtype)
+        self._fn("kmeanspp", X.dtype)(_i64(n), _int(d), _int(k), _ptr(X), _int(seed), _ptr(rows),
+                                      _ptr(mind))
+        return rows, mind
+
     def kmeanspp_first(self, seed, n):
         self.lib.oracle_kmeanspp_first.restype = _int
         return int(self.lib.oracle_kmeanspp_first(_int(seed), _i64(n)))

@@ -321,6 +321,89 @@ void pair_dist_exact(int64_t n, int d, const T *X, const T *C, const int *a,
   }
 }
 
+// k-means++ (D^2 sampling), the textbook algorithm with the draw rule spelled out so
+// that a GPU implementation can follow it to the bit:
+//   first centre: std::mt19937 gen(seed); uniform_int_distribution<>(0, n-1)(gen)
+//     (how the reference draws the first centre of its k-means||,
+//      kmeans_h2o4gpu.cu:343-347);
+//   mind[i] = min over chosen centres of |(xx_i + cc) - 2 x_i.c|  (the distance
+//     form of kmeans_labels.cu:183-244; running minimum as min_calc_functor,
+//     kmeans_h2o4gpu.cu:281-304);
+//   next centre: u = uniform_real_distribution<double>(0,1)(gen); target = u*total,
+//     total = ordered sum of block sums; block sums cover 1024 rows each and are
+//     formed in double by 256 partial sums (rows t, t+256, t+512, t+768) combined by
+//     a halving tree; the block is the first whose running total exceeds the target,
+//     the row the first inside it whose running total exceeds the target (last
+//     positive row if rounding runs past the end).
+// Not part of the reference (it seeds with k-means||); parity unpinned against it.
+template <typename T>
+void kmeanspp(int64_t n, int d, int k, const T *X, int seed, int *rows_out, T *mind_out) {
+  const int BLOCK = 1024, W = 256;
+  std::vector<T> xx((size_t)n), mind((size_t)n);
+  row_norms<T>(n, d, X, xx.data(), 1);
+  std::mt19937 gen((unsigned)seed);
+  std::uniform_int_distribution<> first(0, (int)(n - 1));
+  std::uniform_real_distribution<double> uni(0.0, 1.0);
+  const int64_t nb = (n + BLOCK - 1) / BLOCK;
+  std::vector<double> bs((size_t)nb);
+  rows_out[0] = first(gen);
+  for (int c = 1; c <= k; c++) {
+    const T *cp = X + (int64_t)rows_out[c - 1] * d;
+    const T cc = xx[rows_out[c - 1]];
+    for (int64_t i = 0; i < n; i++) {
+      const T *x = X + i * (int64_t)d;
+      T dot = 0;
+      for (int j = 0; j < d; j++) dot += x[j] * cp[j];
+      T t = xx[i] + cc;
+      T dist = std::fabs(t - (T)2 * dot);
+      mind[i] = (c == 1) ? dist : std::min(dist, mind[i]);
+    }
+    if (c == k) break;
+    for (int64_t b = 0; b < nb; b++) {
+      double part[W];
+      for (int t = 0; t < W; t++) {
+        double acc = 0;
+        for (int q = 0; q < BLOCK / W; q++) {
+          int64_t row = b * BLOCK + t + q * W;
+          if (row < n) acc += (double)mind[row];
+        }
+        part[t] = acc;
+      }
+      for (int off = W / 2; off > 0; off >>= 1)
+        for (int t = 0; t < off; t++) part[t] += part[t + off];
+      bs[b] = part[0];
+    }
+    double total = 0;
+    for (int64_t b = 0; b < nb; b++) total += bs[b];
+    const double u = uni(gen);
+    int64_t pick;
+    if (!(total > 0)) {
+      pick = (int64_t)(u * (double)n);
+      if (pick >= n) pick = n - 1;
+    } else {
+      const double target = u * total;
+      double run = 0;
+      int64_t b = 0;
+      for (; b < nb - 1; b++) {
+        if (run + bs[b] > target) break;
+        run += bs[b];
+      }
+      const int64_t lo = b * BLOCK;
+      const int cnt = (int)std::min<int64_t>(BLOCK, n - lo);
+      int i = 0, last_pos = 0;
+      for (; i < cnt; i++) {
+        if ((double)mind[lo + i] > 0) last_pos = i;
+        if (run + (double)mind[lo + i] > target) break;
+        run += (double)mind[lo + i];
+      }
+      if (i >= cnt) i = last_pos;
+      pick = lo + i;
+    }
+    rows_out[c] = (int)pick;
+  }
+  if (mind_out) std::copy(mind.begin(), mind.end(), mind_out);
+}
+
 }  // namespace
 
 extern "C" {
@@ -387,6 +470,15 @@ ORACLE_EXPORT int oracle_max_threads(void) {
 
 DEFINE_FOR(float, f32)
 DEFINE_FOR(double, f64)
+
+ORACLE_EXPORT void oracle_kmeanspp_f32(int64_t n, int d, int k, const float *X, int seed,
+                                       int *rows_out, float *mind_out) {
+  kmeanspp<float>(n, d, k, X, seed, rows_out, mind_out);
+}
+ORACLE_EXPORT void oracle_kmeanspp_f64(int64_t n, int d, int k, const double *X, int seed,
+                                       int *rows_out, double *mind_out) {
+  kmeanspp<double>(n, d, k, X, seed, rows_out, mind_out);
+}
 
 // Seeded random-row initialisation: a permutation of 0..n-1 by
 // std::shuffle(v.begin(), v.end(), std::default_random_engine(seed)); the

@@ -209,3 +209,36 @@ def test_transform_matches_oracle(hip, oracle, n, d, k, dtype):
     eps = np.finfo(dtype).eps
     assert got.shape == (k, n)
     assert np.max(np.abs(got.astype(np.float64) - want)) <= 4 * np.sqrt(d) * eps * scale
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n,d,k,seed", [(5000, 6, 12, 3), (20000, 32, 40, 11), (3000, 100, 25, 5), (1500, 3, 7, 0)])
+def test_kmeanspp_seeding(hip, oracle, n, d, k, seed, dtype):
+    """k-means++ on the device: same draw rule as the CPU restatement (same generator
+    calls, same fixed-tree block sums), so the chosen rows agree; the minimum distances
+    differ only by summation order."""
+    X = blobs(n, d, k, dtype, spread=30.0, seed=n + k)
+    with hip.Handle(n, d, k, dtype) as h:
+        h.set_data(X)
+        h.init_plusplus(seed)
+        rows = h.seed_rows()
+        C = h.centroids()
+        mind = h.min_distances()
+        h.init_plusplus(seed)
+        assert np.array_equal(rows, h.seed_rows())          # deterministic per seed
+    want_rows, want_mind = oracle.kmeanspp(X, k, seed)
+    assert np.array_equal(C, X[rows])
+    assert len(set(rows.tolist())) == k
+    scale = (X.astype(np.float64) ** 2).sum(1).max() * 2
+    eps = np.finfo(dtype).eps
+    if np.array_equal(rows, want_rows):
+        assert np.max(np.abs(mind.astype(np.float64) - want_mind)) <= 8 * np.sqrt(d) * eps * scale
+    else:
+        # a draw landed within rounding of a boundary between two rows: allowed, but the
+        # first differing pick must be such a boundary case and quality must be the same
+        i = int(np.nonzero(rows != want_rows)[0][0])
+        assert i > 0
+        pot_g = mind.astype(np.float64).sum()
+        pot_o = want_mind.astype(np.float64).sum()
+        assert abs(pot_g - pot_o) <= 0.2 * pot_o
+        print("k-means++ picks diverged at pick %d of %d" % (i, k))

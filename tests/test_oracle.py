@@ -209,3 +209,42 @@ def test_row_norms_sequential_float32(oracle):
         acc = np.float32(acc + np.float32(v * v))
     assert oracle.row_norms(x)[0] == acc
     assert oracle.row_norms(x.astype(np.float64))[0] == 1e8 + 4
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_kmeanspp_is_d2_sampling(oracle, dtype):
+    """Textbook properties of D^2 sampling: chosen rows are distinct (a chosen row has
+    distance 0 and cannot be drawn again), the potential never increases, the draw is a
+    function of the seed, and on far-apart blobs it hits every blob."""
+    rng = np.random.default_rng(8)
+    k, d, n = 12, 6, 5000
+    centers = rng.uniform(-100, 100, size=(k, d))
+    X = (centers[rng.integers(0, k, size=n)] + rng.normal(size=(n, d))).astype(dtype)
+    rows, mind = oracle.kmeanspp(X, k, 3)
+    rows2, _ = oracle.kmeanspp(X, k, 3)
+    rows3, _ = oracle.kmeanspp(X, k, 4)
+    assert np.array_equal(rows, rows2) and not np.array_equal(rows, rows3)
+    assert len(set(rows.tolist())) == k
+    assert rows[0] == oracle.kmeanspp_first(3, n)
+    # minimum distance to the chosen rows, by brute force in float64
+    D = ((X[:, None, :].astype(np.float64) - X[rows][None, :, :]) ** 2).sum(-1).min(1)
+    assert np.allclose(mind, D, rtol=1e-3, atol=1e-2 if dtype == np.float32 else 1e-9)
+    # every blob got a centre: all rows are within a blob diameter of a chosen row
+    assert D.max() < 100.0
+    pots = [oracle.kmeanspp(X, kk, 3)[1].astype(np.float64).sum() for kk in (2, 4, 8, 12)]
+    assert all(b <= a for a, b in zip(pots, pots[1:]))
+
+
+def test_kmeanspp_draw_is_proportional_to_d2(oracle):
+    """Two far clusters of very different spread: after the first centre, the second is
+    drawn with probability proportional to squared distance, so over many seeds it falls
+    in the other cluster almost always (a uniform or D^1 draw would not)."""
+    rng = np.random.default_rng(9)
+    A = rng.normal(size=(900, 2)) * 0.1
+    B = rng.normal(size=(100, 2)) * 0.1 + 50.0
+    X = np.concatenate([A, B]).astype(np.float32)
+    other = 0
+    for seed in range(40):
+        rows, _ = oracle.kmeanspp(X, 2, seed)
+        other += (rows[0] < 900) != (rows[1] < 900)
+    assert other >= 39
