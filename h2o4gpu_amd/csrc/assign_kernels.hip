@@ -410,8 +410,17 @@ __global__ __launch_bounds__(WG, 2) void assign_tiled_kernel(
   for (int q = 0; q < (A_VECS > B_VECS ? A_VECS : B_VECS); q++) {
     const int rr = rr0 + q * ROWS_PER_PASS;
     const int t = rr / MT, i = rr - t * MT, gg = jj / DCH, s = jj - gg * DCH;
-    lds_off[q] = ((t * NV + s / VW) * 64 + gg * MT + i) * VW;
+    // The 8 threads that stage one operand row write 8 different (vector, lane group)
+    // combinations; unswizzled they land 1 KB apart, i.e. on the same banks. XOR-ing the
+    // combination number into the low 3 bits of the lane slot spreads them over all
+    // banks; a reader of vector q applies the same XOR, and since it reads all 64 slots
+    // of the vector its access stays a conflict-free permutation.
+    const int slot = (gg * MT + i) ^ (((s / VW) * KL + gg) & 7);
+    lds_off[q] = ((t * NV + s / VW) * 64 + slot) * VW;
   }
+  int rd_slot[NV];  // this lane's (swizzled) slot when it reads vector q of a tile
+#pragma unroll
+  for (int q = 0; q < NV; q++) rd_slot[q] = lane ^ ((q * KL + g) & 7);
   const T *xrow[B_VECS];
 #pragma unroll
   for (int q = 0; q < B_VECS; q++)
@@ -496,15 +505,15 @@ __global__ __launch_bounds__(WG, 2) void assign_tiled_kernel(
     for (int st = 0; st < nstage; st++) {
       const int buf = st & 1;
       if (st + 1 < nstage) gload(c0, st + 1);
-      const vec_t *ap = reinterpret_cast<const vec_t *>(As + buf * A_ELEMS) + lane;
-      const vec_t *bp = reinterpret_cast<const vec_t *>(Bs + buf * B_ELEMS) + lane;
+      const vec_t *ap = reinterpret_cast<const vec_t *>(As + buf * A_ELEMS);
+      const vec_t *bp = reinterpret_cast<const vec_t *>(Bs + buf * B_ELEMS);
 #pragma unroll
       for (int q = 0; q < NV; q++) {
         vec_t a[CT], b[RT];
 #pragma unroll
-        for (int ct = 0; ct < CT; ct++) a[ct] = ap[((wc * CT + ct) * NV + q) * 64];
+        for (int ct = 0; ct < CT; ct++) a[ct] = ap[((wc * CT + ct) * NV + q) * 64 + rd_slot[q]];
 #pragma unroll
-        for (int rt = 0; rt < RT; rt++) b[rt] = bp[((wr * RT + rt) * NV + q) * 64];
+        for (int rt = 0; rt < RT; rt++) b[rt] = bp[((wr * RT + rt) * NV + q) * 64 + rd_slot[q]];
 #pragma unroll
         for (int e = 0; e < VW; e++) {
 #pragma unroll
