@@ -89,6 +89,7 @@ struct h2o4gpu_kmeans_handle {
   hipStream_t stream = nullptr;
   int opt_assign = ASSIGN_AUTO;
   int opt_fuse = 1;  // 1: use the fused assign+accumulate kernel where the shape allows
+  int opt_buckets = 1;  // 1: bucketed centroid sums where the sums do not fit LDS
   int last_variant = ASSIGN_AUTO;
 
   // profiling
@@ -203,6 +204,9 @@ struct Engine : h2o4gpu_kmeans_handle {
   int *pcounts = nullptr;
   T *shift_partials = nullptr;
   T *shift2 = nullptr;
+  int *order = nullptr, *order_label = nullptr, *bucket_offsets = nullptr, *bucket_cursor = nullptr;
+  int *bucket_counts = nullptr;
+  bool use_buckets = false;
   double *sum_partials = nullptr;  // [sum_partials_needed() + 1]
   double *kpp_bsums = nullptr;
   bool have_data = false, have_centroids = false, have_mindist = false;
@@ -253,6 +257,14 @@ struct Engine : h2o4gpu_kmeans_handle {
     if (fs > slots) slots = fs;
     KM_TRY(dalloc(&psums, (size_t)slots * kd));
     KM_TRY(dalloc(&pcounts, (size_t)slots * k));
+    use_buckets = bucketed_update_applies(plan.k_chunks, k);
+    if (use_buckets) {
+      KM_TRY(dalloc(&order, n));
+      KM_TRY(dalloc(&order_label, n));
+      KM_TRY(dalloc(&bucket_offsets, k));
+      KM_TRY(dalloc(&bucket_cursor, k));
+      KM_TRY(dalloc(&bucket_counts, k));
+    }
     KM_TRY(dalloc(&shift_partials, (kd + 31) / 32 + 1));
     KM_TRY(dalloc(&shift2, 1));
     KM_TRY(dalloc(&sum_partials, sum_partials_needed() + 1));
@@ -276,7 +288,8 @@ struct Engine : h2o4gpu_kmeans_handle {
     if (own_X && X) (void)hipFree(X);
     void *ptrs[] = {xnorm,  C[0],    C[1],           cnorm,  labels,       mindist,
                     counts, psums,   pcounts,        shift_partials, shift2,
-                    sum_partials, kpp_bsums};
+                    sum_partials, kpp_bsums, order, order_label, bucket_offsets,
+                    bucket_cursor, bucket_counts};
     for (void *p : ptrs)
       if (p) (void)hipFree(p);
     if (stream) (void)hipStreamDestroy(stream);
@@ -426,6 +439,12 @@ struct Engine : h2o4gpu_kmeans_handle {
   }
 
   int update_async() {
+    if (use_buckets && opt_buckets) {
+      PROFILED("accumulate", launch_bucketed_accumulate<T>(stream, X, labels, order, order_label,
+                                                           bucket_offsets, bucket_cursor,
+                                                           bucket_counts, psums, pcounts, n, d, k));
+      return finish_update(1);
+    }
     PROFILED("accumulate", launch_accumulate<T>(stream, plan, X, labels, psums, pcounts, n, d, k));
     return finish_update(plan.row_blocks);
   }
@@ -883,6 +902,11 @@ KM_API int h2o4gpu_kmeans_set_option(h2o4gpu_kmeans_handle *h, const char *name,
   if (strcmp(name, "assign") == 0) {
     if (value < ASSIGN_AUTO || value > ASSIGN_TILED) return H2O4GPU_KMEANS_EARG;
     h->opt_assign = value;
+    return 0;
+  }
+  if (strcmp(name, "buckets") == 0) {
+    if (value != 0 && value != 1) return H2O4GPU_KMEANS_EARG;
+    h->opt_buckets = value;
     return 0;
   }
   if (strcmp(name, "fuse") == 0) {

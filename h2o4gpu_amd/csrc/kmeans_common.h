@@ -103,6 +103,16 @@ template <typename T>
 int launch_accumulate(hipStream_t s, const UpdatePlan &p, const T *X,
                       const int *labels, double *psums, int *pcounts, int64_t n,
                       int d, int k);
+// Pass 1 for shapes whose sums do not fit LDS (plan.k_chunks > 1): rows are bucketed by
+// label (order / order_label: [n] int32 each, offsets / cursor: [k] int32) and every
+// bucket is summed into gsum [k][d] double; counts receives the bucket sizes. The
+// result is consumed by launch_finalize with slots = 1.
+bool bucketed_update_applies(int k_chunks, int k);
+template <typename T>
+int launch_bucketed_accumulate(hipStream_t s, const T *X, const int *labels, int *order,
+                               int *order_label, int *offsets, int *cursor, int *total,
+                               double *gsum, int *counts, int64_t n, int d, int k);
+
 // Pass 2: fixed-order reduction of the partials, empty clusters keep the old
 // centroid, mean = sum * (1/count), per-block partial of sum((old-new)^2).
 template <typename T>

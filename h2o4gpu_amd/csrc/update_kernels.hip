@@ -78,7 +78,7 @@ __global__ __launch_bounds__(WG) void row_norms_coalesced_kernel(
 template <typename T>
 int launch_row_norms(hipStream_t s, const T *X, T *out, int64_t n, int d) {
   if (n <= 0) return 0;
-  if (n >= 65536 && d >= 8) {
+  if (d >= 8 && n * (int64_t)d >= 65536) {
     if (d <= 16) {
       constexpr int LPR = 16;
       hipLaunchKernelGGL((row_norms_coalesced_kernel<T, LPR>),
@@ -308,6 +308,233 @@ int launch_accumulate<double>(hipStream_t s, const UpdatePlan &p, const double *
 }
 
 // ---------------------------------------------------------------------------
+// pass 1, large k*d: bucket rows by label, then sum each bucket.
+//
+// When the per-centroid sums do not fit in LDS the chunked kernel above has to
+// scan all labels once per centroid chunk. Instead the rows are bucketed by
+// label (counting sort: histogram, exclusive scan, scatter) and every wavefront
+// sums 64 consecutive rows of the bucketed order in registers, lanes across
+// features, flushing to the [k][d] double sums with a global atomic add only
+// when the label changes (about once per wavefront). The data set is read once,
+// in whole rows. Sums are double, so for float data the result does not depend
+// on the order inside a bucket (which the scatter does not fix).
+// Replaces the reference's sort_by_key + calculate_centroids
+// (kmeans_centroids.h:40-75, 131).
+// ---------------------------------------------------------------------------
+static constexpr int BUCKET_ROWS = 4096;  // rows per workgroup in count / scatter
+
+__global__ __launch_bounds__(WG) void bucket_count_kernel(const int *__restrict__ labels,
+                                                         int *__restrict__ counts, int64_t n,
+                                                         int k) {
+  extern __shared__ int hist[];  // [k]
+  const int tid = threadIdx.x;
+  for (int c = tid; c < k; c += WG) hist[c] = 0;
+  __syncthreads();
+  const int64_t r0 = (int64_t)blockIdx.x * BUCKET_ROWS;
+  const int64_t r1 = min(n, r0 + BUCKET_ROWS);
+  for (int64_t i = r0 + tid; i < r1; i += WG) {
+    const int l = labels[i];
+    if (l >= 0 && l < k) atomicAdd(&hist[l], 1);
+  }
+  __syncthreads();
+  for (int c = tid; c < k; c += WG)
+    if (hist[c] > 0) atomicAdd(&counts[c], hist[c]);
+}
+
+// offsets[c] = sum of counts[0..c), cursor = copy; single workgroup.
+__global__ __launch_bounds__(WG) void bucket_scan_kernel(const int *__restrict__ counts,
+                                                        int *__restrict__ offsets,
+                                                        int *__restrict__ cursor,
+                                                        int *__restrict__ total, int k) {
+  __shared__ int part[WG];
+  const int tid = threadIdx.x;
+  const int per = (k + WG - 1) / WG;
+  const int lo = tid * per, hi = min(k, lo + per);
+  int s = 0;
+  for (int c = lo; c < hi; c++) s += counts[c];
+  part[tid] = s;
+  __syncthreads();
+  if (tid == 0) {
+    int run = 0;
+    for (int t = 0; t < WG; t++) {
+      const int v = part[t];
+      part[t] = run;
+      run += v;
+    }
+    *total = run;  // rows that carry a label in [0, k)
+  }
+  __syncthreads();
+  int run = part[tid];
+  for (int c = lo; c < hi; c++) {
+    offsets[c] = run;
+    cursor[c] = run;
+    run += counts[c];
+  }
+}
+
+__global__ __launch_bounds__(WG) void bucket_scatter_kernel(const int *__restrict__ labels,
+                                                           int *__restrict__ cursor,
+                                                           int *__restrict__ order,
+                                                           int *__restrict__ order_label,
+                                                           int64_t n, int k) {
+  extern __shared__ int sm[];
+  int *hist = sm;      // [k] rows of this block per label, then running rank
+  int *base = sm + k;  // [k] start of this block's range inside the label's bucket
+  const int tid = threadIdx.x;
+  for (int c = tid; c < k; c += WG) hist[c] = 0;
+  __syncthreads();
+  const int64_t r0 = (int64_t)blockIdx.x * BUCKET_ROWS;
+  const int64_t r1 = min(n, r0 + BUCKET_ROWS);
+  for (int64_t i = r0 + tid; i < r1; i += WG) {
+    const int l = labels[i];
+    if (l >= 0 && l < k) atomicAdd(&hist[l], 1);
+  }
+  __syncthreads();
+  for (int c = tid; c < k; c += WG) {
+    const int h = hist[c];
+    base[c] = h > 0 ? atomicAdd(&cursor[c], h) : 0;
+    hist[c] = 0;
+  }
+  __syncthreads();
+  for (int64_t i = r0 + tid; i < r1; i += WG) {
+    const int l = labels[i];
+    if (l >= 0 && l < k) {
+      const int pos = base[l] + atomicAdd(&hist[l], 1);
+      order[pos] = (int)i;
+      order_label[pos] = l;
+    }
+  }
+}
+
+// One wavefront per 64 bucketed rows; lanes across features (VEC each, NVEC
+// vectors per lane cover up to 64*VEC*NVEC features per pass over the rows).
+template <typename T, int VEC, int NVEC>
+__global__ __launch_bounds__(WG) void segment_sum_kernel(
+    const T *__restrict__ X, const int *__restrict__ order,
+    const int *__restrict__ order_label, double *__restrict__ gsum,
+    const int *__restrict__ total, int d) {
+  const int64_t m = *total;
+  const int lane = threadIdx.x & 63;
+  const int64_t pos0 = ((int64_t)blockIdx.x * (WG / 64) + (threadIdx.x >> 6)) * 64;
+  if (pos0 >= m) return;
+  const int cnt = (int)min<int64_t>(64, m - pos0);
+  const int my_row = lane < cnt ? order[pos0 + lane] : 0;
+  const int my_lab = lane < cnt ? order_label[pos0 + lane] : -1;
+  constexpr int SPAN = 64 * VEC * NVEC;
+  for (int d0 = 0; d0 < d; d0 += SPAN) {
+    double acc[NVEC][VEC];
+#pragma unroll
+    for (int q = 0; q < NVEC; q++)
+#pragma unroll
+      for (int e = 0; e < VEC; e++) acc[q][e] = 0.0;
+    int cur = __shfl(my_lab, 0, 64);
+    auto flush = [&](int label) {
+#pragma unroll
+      for (int q = 0; q < NVEC; q++) {
+        const int j = d0 + (q * 64 + lane) * VEC;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+          if (j + e < d) unsafeAtomicAdd(gsum + (size_t)label * d + j + e, acc[q][e]);
+          acc[q][e] = 0.0;
+        }
+      }
+    };
+    constexpr int U = 4;
+    for (int i0 = 0; i0 < cnt; i0 += U) {
+      typename RowVec<T, VEC>::type v[U][NVEC];
+      int lab[U];
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+        const int i = min(i0 + u, cnt - 1);
+        const int row = __shfl(my_row, i, 64);
+        lab[u] = __shfl(my_lab, i, 64);
+        const T *x = X + (int64_t)row * d;
+#pragma unroll
+        for (int q = 0; q < NVEC; q++) {
+          int j = d0 + (q * 64 + lane) * VEC;
+          if (j + VEC > d) j = 0;  // masked below
+          v[u][q] = load_vec<T, VEC>(x + j);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+        if (i0 + u >= cnt) break;
+        if (lab[u] != cur) {
+          flush(cur);
+          cur = lab[u];
+        }
+#pragma unroll
+        for (int q = 0; q < NVEC; q++) {
+          const int j = d0 + (q * 64 + lane) * VEC;
+          if (j + VEC <= d) {
+            if constexpr (VEC == 1) {
+              acc[q][0] += (double)v[u][q];
+            } else {
+#pragma unroll
+              for (int e = 0; e < VEC; e++) acc[q][e] += (double)v[u][q][e];
+            }
+          }
+        }
+      }
+    }
+    flush(cur);
+  }
+}
+
+size_t bucket_lds_bytes(int k) { return (size_t)2 * k * sizeof(int); }
+bool bucketed_update_applies(int k_chunks, int k) {
+  return k_chunks > 1 && bucket_lds_bytes(k) <= 128 * 1024;
+}
+
+template <typename T>
+int launch_bucketed_accumulate(hipStream_t s, const T *X, const int *labels, int *order,
+                               int *order_label, int *offsets, int *cursor, int *total,
+                               double *gsum, int *counts, int64_t n, int d, int k) {
+  KM_HIP_TRY(hipMemsetAsync(counts, 0, (size_t)k * sizeof(int), s));
+  KM_HIP_TRY(hipMemsetAsync(gsum, 0, (size_t)k * d * sizeof(double), s));
+  const unsigned blocks = (unsigned)((n + BUCKET_ROWS - 1) / BUCKET_ROWS);
+  const size_t lds1 = (size_t)k * sizeof(int), lds2 = bucket_lds_bytes(k);
+  if (lds2 > 64 * 1024) {
+    KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(bucket_scatter_kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds2));
+    KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(bucket_count_kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds2));
+  }
+  hipLaunchKernelGGL(bucket_count_kernel, dim3(blocks), dim3(WG), lds1, s, labels, counts, n, k);
+  hipLaunchKernelGGL(bucket_scan_kernel, dim3(1), dim3(WG), 0, s, counts, offsets, cursor, total, k);
+  hipLaunchKernelGGL(bucket_scatter_kernel, dim3(blocks), dim3(WG), lds2, s, labels, cursor, order,
+                     order_label, n, k);
+  // rows with a label outside [0, k) are not bucketed, so the bucketed order may be
+  // shorter than n: the grid covers n positions and every wavefront bounds itself by
+  // the device-side total
+  const unsigned sblocks = (unsigned)((n + 255) / 256);
+  const bool aligned = (reinterpret_cast<uintptr_t>(X) & 15) == 0;
+#define KM_SEG(VEC, NVEC)                                                                   \
+  hipLaunchKernelGGL((segment_sum_kernel<T, VEC, NVEC>), dim3(sblocks), dim3(WG), 0, s, X, \
+                     order, order_label, gsum, total, d)
+  if constexpr (sizeof(T) == 4) {
+    if (d % 4 == 0 && aligned) {
+      if (d <= 256) KM_SEG(4, 1);
+      else if (d <= 512) KM_SEG(4, 2);
+      else KM_SEG(4, 4);
+    } else {
+      KM_SEG(1, 4);
+    }
+  } else {
+    if (d % 2 == 0 && aligned) {
+      if (d <= 128) KM_SEG(2, 1);
+      else if (d <= 256) KM_SEG(2, 2);
+      else KM_SEG(2, 4);
+    } else {
+      KM_SEG(1, 4);
+    }
+  }
+#undef KM_SEG
+  KM_HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
 // pass 2: finalize. One thread per centroid coordinate.
 // ---------------------------------------------------------------------------
 // A workgroup takes EPW = 32 consecutive coordinates; RS = 8 thread groups each
@@ -424,7 +651,7 @@ __global__ __launch_bounds__(WG) void post_update_kernel(
     return;
   }
   const int c = blockIdx.x * WG + tid;
-  if (c >= k) return;
+  if (c >= k || cnorm == nullptr) return;
   const T *x = c_new + (size_t)c * d;
   T acc = 0;
   for (int j = 0; j < d; j++) {
@@ -438,10 +665,15 @@ template <typename T>
 int launch_post_update(hipStream_t s, const T *c_new, T *cnorm,
                        const T *shift_partials, int n_shift_partials, T *shift2,
                        int d, int k) {
-  const int blocks = (k + WG - 1) / WG + 1;
+  // large centroid sets: norms by the coalesced row-norm kernel (same summation order),
+  // this kernel then only adds up the shift partials
+  const bool separate_norms = (int64_t)k * d >= 65536 && d >= 8;
+  const int blocks = separate_norms ? 1 : (k + WG - 1) / WG + 1;
   hipLaunchKernelGGL((post_update_kernel<T>), dim3(blocks), dim3(WG), 0, s, c_new,
-                     cnorm, shift_partials, n_shift_partials, shift2, d, k);
+                     separate_norms ? (T *)nullptr : cnorm, shift_partials, n_shift_partials,
+                     shift2, d, k);
   KM_HIP_TRY(hipGetLastError());
+  if (separate_norms) return launch_row_norms<T>(s, c_new, cnorm, k, d);
   return 0;
 }
 
@@ -513,6 +745,13 @@ int launch_gather_rows(hipStream_t s, const T *X, const int *idx, T *C, int k, i
   KM_HIP_TRY(hipGetLastError());
   return 0;
 }
+
+template int launch_bucketed_accumulate<float>(hipStream_t, const float *, const int *, int *, int *,
+                                               int *, int *, int *, double *, int *, int64_t, int,
+                                               int);
+template int launch_bucketed_accumulate<double>(hipStream_t, const double *, const int *, int *,
+                                                int *, int *, int *, int *, double *, int *, int64_t,
+                                                int, int);
 
 #define KM_INSTANTIATE(T)                                                            \
   template int launch_row_norms<T>(hipStream_t, const T *, T *, int64_t, int);       \

@@ -59,17 +59,21 @@ def test_assign_matches_oracle(hip, oracle, n, d, k, variant, dtype):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("buckets", [1, 0])
 @pytest.mark.parametrize("n,d,k", [(5000, 32, 256), (3000, 16, 8), (2000, 7, 5), (4000, 256, 300),
-                                   (1000, 784, 130), (70000, 64, 64), (300, 3, 300)])
-def test_update_matches_oracle(hip, oracle, n, d, k, dtype):
+                                   (1000, 784, 130), (70000, 64, 64), (300, 3, 300), (9000, 1100, 70),
+                                   (5000, 130, 90), (6000, 51, 700)])
+def test_update_matches_oracle(hip, oracle, n, d, k, buckets, dtype):
     X = blobs(n, d, k, dtype, seed=7 * n + k)
     C = np.ascontiguousarray(X[RNG.choice(n, size=k, replace=False)])
     labels = RNG.integers(0, k, size=n).astype(np.int32)
     labels[labels == 1] = 0  # cluster 1 empty: must keep its old centroid
+    labels[::97] = -1        # rows without a label (all distances overflowed) are skipped
     with hip.Handle(n, d, k, dtype) as h:
         h.set_data(X)
         h.set_centroids(C)
         h.set_labels(labels)
+        h.set_option("buckets", buckets)
         shift2 = h.update()
         got = h.centroids()
         counts = h.counts()
