@@ -25,6 +25,15 @@ from h2o4gpu_amd.libs import kmeans_hip  # noqa: E402
 PEAK_HBM_GBPS = 8000.0
 PEAK_MFMA_TFLOPS = {"f32": 157.3, "f64": 78.6}
 
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of this script (profiles/assign_accumulate_rowstat_c3.md): raw
+# counter x calibration factor of a plain 1 GiB copy kernel (2.0 for FETCH_SIZE,
+# 1.0 for WRITE_SIZE on this box). Keyed by (workload, dtype, kernel); other
+# combinations report null.
+MEASURED_TRAFFIC_BYTES = {
+    ("C3", "f32", "assign_accumulate"): (644700 * 2.0 + 94765 * 1.0) * 1024.0,
+}
+
 
 def log(msg):
     print("[bench] " + msg, file=sys.stderr, flush=True)
@@ -119,9 +128,12 @@ def main():
     tflops = flops_per_iter / (assign_ms * 1e-3) / 1e12
     peak = PEAK_MFMA_TFLOPS[args.dtype]
     mfma_bound = variant != "valu"
+    traffic = None
+    if args.scale == 1.0:
+        traffic = MEASURED_TRAFFIC_BYTES.get((args.workload, args.dtype, dom))
     if mfma_bound:
         roofline = {"bound": "mfma", "kernel": "%s (%s)" % (dom, variant), "achieved": tflops,
-                    "peak": peak, "unit": "TFLOP/s", "frac": tflops / peak, "traffic": None}
+                    "peak": peak, "unit": "TFLOP/s", "frac": tflops / peak, "traffic": traffic}
     else:
         gbps = (float(n) * d * s + 8.0 * n) / (assign_ms * 1e-3) / 1e9
         roofline = {"bound": "hbm", "kernel": "assign (valu)", "achieved": gbps,

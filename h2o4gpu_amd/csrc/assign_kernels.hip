@@ -142,11 +142,44 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
     for (int c = tid; c < k; c += TPB) cnt[c] = 0;
   }
 
-  for (int e = tid; e < kp * DP; e += TPB) {
-    const int c = e / DP, j = e - c * DP;
-    const T v = (c < k && j < d) ? (T)-2 * C[(size_t)c * d + j] : (T)0;
-    const int t = c / MT, i = c - t * MT, gg = j / DCH, s = j - gg * DCH;
-    Cs[((size_t)(t * NV + s / VW) * 64 + gg * MT + i) * VW + (s % VW)] = v;
+  if (VECLOAD) {
+    // d == DP: 16-byte loads, four in flight per thread, one 16-byte LDS store each
+    constexpr int VPR = DP / VW;  // vectors per centroid row
+    const int nvec = k * VPR;
+    constexpr int U = 4;
+    for (int e0 = tid; e0 < nvec; e0 += U * TPB) {
+      vec_t v[U];
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+        const int e = min(e0 + u * TPB, nvec - 1);
+        v[u] = reinterpret_cast<const vec_t *>(C)[e];
+      }
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+        const int e = e0 + u * TPB;
+        if (e < nvec) {
+          const int c = e / VPR, j = (e - c * VPR) * VW;
+          const int t = c / MT, i = c - t * MT, gg = j / DCH, s = j - gg * DCH;
+          reinterpret_cast<vec_t *>(Cs)[(size_t)(t * NV + s / VW) * 64 + gg * MT + i] = v[u] * (T)-2;
+        }
+      }
+    }
+    // centroid rows k .. kp-1 of the last tile: zeros
+    for (int e = k * VPR + tid; e < kp * VPR; e += TPB) {
+      const int c = e / VPR, j = (e - c * VPR) * VW;
+      const int t = c / MT, i = c - t * MT, gg = j / DCH, s = j - gg * DCH;
+      vec_t z;
+#pragma unroll
+      for (int q = 0; q < VW; q++) z[q] = 0;
+      reinterpret_cast<vec_t *>(Cs)[(size_t)(t * NV + s / VW) * 64 + gg * MT + i] = z;
+    }
+  } else {
+    for (int e = tid; e < kp * DP; e += TPB) {
+      const int c = e / DP, j = e - c * DP;
+      const T v = (c < k && j < d) ? (T)-2 * C[(size_t)c * d + j] : (T)0;
+      const int t = c / MT, i = c - t * MT, gg = j / DCH, s = j - gg * DCH;
+      Cs[((size_t)(t * NV + s / VW) * 64 + gg * MT + i) * VW + (s % VW)] = v;
+    }
   }
   for (int c = tid; c < kp; c += TPB) ccs[c] = c < k ? cnorm[c] : pos_inf<T>();
   __syncthreads();
@@ -712,7 +745,8 @@ static int launch_rowstat_nw(hipStream_t s, const T *X, const T *xnorm, const T 
   if (grid > tiles) grid = tiles;
   if (grid < 1) grid = 1;
   if (slots) *slots = (int)grid;
-  const bool vec = (d == DP) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0);
+  const bool vec = (d == DP) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0) &&
+                   ((reinterpret_cast<uintptr_t>(C) & 15) == 0);
   if (vec) {
     auto kern = assign_rowstat_kernel<T, DP, ROWT, true, FUSE, NW>;
     if (lds > 64 * 1024)
