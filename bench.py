@@ -68,6 +68,8 @@ def main():
     ap.add_argument("--assign", default="auto", choices=sorted(kmeans_hip.ASSIGN_VARIANTS))
     ap.add_argument("--no-fuse", action="store_true",
                     help="keep assignment and accumulation as separate kernels")
+    ap.add_argument("--transform-rows", type=int, default=0,
+                    help="also time transform (full distance matrix) on this many held-out rows (C5)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-iters", type=int, default=0, help="CPU baseline iterations (0 = auto)")
     args = ap.parse_args()
@@ -146,6 +148,20 @@ def main():
     inertia = None
     h.assign()
     inertia = h.inertia()
+    transform = None
+    if args.transform_rows > 0:
+        H = datasets.make_holdout(args.workload, args.transform_rows, dtype)
+        h.transform(H[:1024])  # warm-up
+        h.profile(True)
+        t0 = time.perf_counter()
+        h.transform(H)
+        wall = time.perf_counter() - t0
+        cnt, ms = h.kernel_time("transform")
+        h.profile(False)
+        tf = 2.0 * H.shape[0] * k * d / (ms * 1e-3) / 1e12
+        transform = {"rows": int(H.shape[0]), "kernel_ms": ms, "launches": cnt, "tflops": tf,
+                     "mfma_frac": tf / peak, "end_to_end_seconds": wall,
+                     "output_bytes": float(H.shape[0]) * k * s}
     h.close()
 
     out = {
@@ -166,6 +182,8 @@ def main():
         "h2d_seconds": h2d_s,
         "inertia": inertia,
     }
+    if transform:
+        out["transform"] = transform
     if not args.no_cpu:
         iters = args.cpu_iters
         if iters <= 0:

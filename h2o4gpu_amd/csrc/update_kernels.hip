@@ -639,8 +639,17 @@ __global__ __launch_bounds__(WG) void post_update_kernel(
   const int tid = threadIdx.x;
   if (blockIdx.x == gridDim.x - 1) {
     __shared__ T red[WG];
+    // eight loads in flight per thread, added in index order
     T acc = 0;
-    for (int i = tid; i < n_partials; i += WG) acc = acc + shift_partials[i];
+    int i = tid;
+    for (; i + 7 * WG < n_partials; i += 8 * WG) {
+      T v[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) v[u] = shift_partials[i + u * WG];
+#pragma unroll
+      for (int u = 0; u < 8; u++) acc = acc + v[u];
+    }
+    for (; i < n_partials; i += WG) acc = acc + shift_partials[i];
     red[tid] = acc;
     __syncthreads();
     for (int off = WG / 2; off > 0; off >>= 1) {
