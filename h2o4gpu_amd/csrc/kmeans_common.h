@@ -52,7 +52,7 @@ enum AssignVariant {
 
 // Rows the centroid buffer C (zeros) and entries the norm buffer cnorm (+inf) must
 // be padded to: launch_assign / launch_transform may read that far.
-static const int CENTROID_PAD = 128;
+static const int CENTROID_PAD = 256;
 
 // Fused distance + argmin. labels[i] = argmin_c |(xx_i + cc_c) - 2 x_i.c_c|,
 // strict '<', lowest index wins, -1 when no distance is below FLT_MAX.

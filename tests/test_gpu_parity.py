@@ -21,7 +21,7 @@ ASSIGN_CASES = [
     # (n, d, k) covering padding of rows, features and centroids in every variant
     (1000, 16, 8), (777, 5, 3), (4096, 32, 256), (5000, 32, 100), (3001, 64, 64),
     (2000, 24, 33), (1500, 128, 40), (2500, 100, 70), (1200, 256, 130), (900, 300, 257),
-    (64, 8, 64), (1, 4, 1), (130, 2, 2),
+    (64, 8, 64), (1, 4, 1), (130, 2, 2), (3000, 40, 600), (2100, 66, 1030),
 ]
 
 
