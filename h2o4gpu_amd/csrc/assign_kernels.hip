@@ -76,6 +76,109 @@ __global__ __launch_bounds__(WG) void assign_valu_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// VALU Lloyd step for the small shapes (k <= 16, d <= 64): assignment and
+// per-centroid accumulation in one pass over the data.
+//
+// Persistent workgroups walk over blocks of 256 rows. A block is fetched with
+// coalesced (16-byte where possible) loads into LDS, row stride odd so that
+// thread t reading row t is conflict-free; every thread then runs the same
+// scalar loop as assign_valu_kernel on its row (j ascending, multiply and add
+// rounded separately: bit-identical to a CPU loop), and adds its row into the
+// double-precision per-centroid sums of the workgroup. Sums and counts go to
+// the workgroup's slot psums[blockIdx.x][k][d], pcounts[blockIdx.x][k].
+// This is the HBM-bound regime: 2*k*d flop per row against d*s bytes.
+// ---------------------------------------------------------------------------
+template <typename T, int DREG, int VEC>
+__global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
+    const T *__restrict__ X, const T *__restrict__ xnorm, const T *__restrict__ C,
+    const T *__restrict__ cnorm, int *__restrict__ labels, T *__restrict__ mindist,
+    double *__restrict__ psums, int *__restrict__ pcounts, int64_t n, int d, int k) {
+#pragma clang fp contract(off)
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  const int sx = d | 1;                                          // row stride of the staged block
+  double *sums = reinterpret_cast<double *>(smem_raw);           // [k][sx]
+  T *Cs = reinterpret_cast<T *>(sums + (size_t)k * sx);          // [k][d]
+  T *ccs = Cs + (size_t)k * d;                                   // [k]
+  int *cnt = reinterpret_cast<int *>(ccs + k);                   // [k]
+  T *Xs = reinterpret_cast<T *>(cnt + k + ((k & 1) ? 1 : 0));    // [WG][sx]
+  const int tid = threadIdx.x;
+  for (int e = tid; e < k * sx; e += WG) sums[e] = 0.0;
+  for (int e = tid; e < k * d; e += WG) Cs[e] = C[e];
+  for (int c = tid; c < k; c += WG) {
+    ccs[c] = cnorm[c];
+    cnt[c] = 0;
+  }
+  __syncthreads();
+  for (int64_t base = (int64_t)blockIdx.x * WG; base < n; base += (int64_t)gridDim.x * WG) {
+    const int rows = (int)min<int64_t>(WG, n - base);
+    const int64_t total = (int64_t)rows * d;
+    const T *src = X + base * (int64_t)d;
+    if (VEC > 1) {
+      typedef typename Mfma<T>::vec_t vec_t;  // 16 bytes
+      const int64_t nv = total / VEC;
+      for (int64_t e = tid; e < nv; e += WG) {
+        const vec_t v = reinterpret_cast<const vec_t *>(src)[e];
+        const int el = (int)(e * VEC);
+        const int r = el / d, j = el - r * d;  // d % VEC == 0: a vector never straddles rows
+#pragma unroll
+        for (int q = 0; q < VEC; q++) Xs[r * sx + j + q] = v[q];
+      }
+    } else {
+      for (int64_t e = tid; e < total; e += WG) {
+        const int r = (int)(e / d), j = (int)(e - (int64_t)r * d);
+        Xs[r * sx + j] = src[e];
+      }
+    }
+    __syncthreads();
+    const int64_t row = base + tid;
+    if (tid < rows) {
+      T xr[DREG];
+#pragma unroll
+      for (int j = 0; j < DREG; j++) xr[j] = j < d ? Xs[tid * sx + j] : (T)0;
+      const T xx = xnorm[row];
+      T best = argmin_start<T>();
+      int bidx = -1;
+      for (int c = 0; c < k; c++) {
+        const T *cp = Cs + (size_t)c * d;
+        T dot = 0;
+#pragma unroll
+        for (int j = 0; j < DREG; j++)
+          if (j < d) dot = dot + xr[j] * cp[j];
+        const T t = xx + ccs[c];
+        const T dist = fabs(t - (T)2 * dot);
+        if (dist < best) {
+          best = dist;
+          bidx = c;
+        }
+      }
+      labels[row] = bidx;
+      if (mindist) mindist[row] = best;
+      if (bidx >= 0) {
+        // Lane l starts at feature l mod d: with only a handful of centroids the
+        // lanes of a wavefront would otherwise all add to the same few addresses
+        // at once, and same-address LDS atomics are served one lane at a time.
+        double *srow = sums + (size_t)bidx * sx;
+        const T *xrow = Xs + tid * sx;
+        int j = (tid & 63) % d;
+        for (int q = 0; q < d; q++) {
+          unsafeAtomicAdd(srow + j, (double)xrow[j]);
+          j = (j + 1 == d) ? 0 : j + 1;
+        }
+        atomicAdd(&cnt[bidx], 1);
+      }
+    }
+    __syncthreads();  // the staged block is overwritten next round
+  }
+  double *dst = psums + (size_t)blockIdx.x * k * d;
+  for (int e = tid; e < k * d; e += WG) {
+    const int c = e / d, j = e - c * d;
+    dst[e] = sums[(size_t)c * sx + j];
+  }
+  int *cdst = pcounts + (size_t)blockIdx.x * k;
+  for (int c = tid; c < k; c += WG) cdst[c] = cnt[c];
+}
+
 // Three-input unsigned minimum as ONE instruction. Written as inline assembly
 // because the optimiser otherwise re-associates a chain of them into pairs of
 // two-input minima and spends 12 instead of 8 instructions on 16 keys.
@@ -830,21 +933,81 @@ struct RowstatDispatch<double, FUSE> {
 };
 #undef KM_ROWSTAT_CASE
 
+static bool valu_fused_applies(int d, int k) { return k <= 16 && d <= 64; }
+template <typename T>
+static size_t valu_fused_lds(int d, int k) {
+  const int sx = d | 1;
+  return (size_t)k * sx * sizeof(double) + ((size_t)k * d + k) * sizeof(T) +
+         ((size_t)k + 1) * sizeof(int) + (size_t)WG * sx * sizeof(T) + 16;
+}
+static int valu_fused_grid(int64_t n, size_t lds, int num_cu) {
+  int per_cu = (int)((150 * 1024) / lds);
+  if (per_cu > 8) per_cu = 8;
+  if (per_cu < 1) per_cu = 1;
+  int64_t grid = (int64_t)num_cu * per_cu;
+  const int64_t blocks = (n + WG - 1) / WG;
+  if (grid > blocks) grid = blocks;
+  return (int)(grid < 1 ? 1 : grid);
+}
+
 // Fused assign + accumulate is offered where the row-stationary kernel applies
-// and centroids plus the double-precision sums fit in one CU's LDS.
+// and centroids plus the double-precision sums fit in one CU's LDS, and for the
+// small shapes the VALU kernel serves.
 template <typename T>
 int fused_slots(int requested_variant, int64_t n, int d, int k, int num_cu) {
-  if (pick_assign_variant<T>(requested_variant, n, d, k) != ASSIGN_ROWSTAT) return 0;
+  const int v = pick_assign_variant<T>(requested_variant, n, d, k);
+  if (v == ASSIGN_VALU && valu_fused_applies(d, k)) return 8 * num_cu;
+  if (v != ASSIGN_ROWSTAT) return 0;
   const size_t lds = rowstat_fused_lds<T>(d, k);
   if (lds > 150 * 1024) return 0;
   return 2 * num_cu;  // upper bound of the grid = number of partial slots
 }
 
 template <typename T>
-int launch_assign_accumulate(hipStream_t s, const T *X, const T *xnorm, const T *C,
+static int launch_valu_fused(hipStream_t s, const T *X, const T *xnorm, const T *C,
+                             const T *cnorm, int *labels, T *mindist, int64_t n, int d, int k,
+                             int num_cu, double *psums, int *pcounts, int *slots) {
+  const size_t lds = valu_fused_lds<T>(d, k);
+  const int grid = valu_fused_grid(n, lds, num_cu);
+  if (slots) *slots = grid;
+  const int vw = Mfma<T>::VW;
+  const bool vec = (d % vw == 0) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0);
+#define KM_VF(DREG)                                                                             \
+  do {                                                                                          \
+    if (vec)                                                                                    \
+      hipLaunchKernelGGL((lloyd_valu_fused_kernel<T, DREG, Mfma<T>::VW>), dim3(grid), dim3(WG), \
+                         lds, s, X, xnorm, C, cnorm, labels, mindist, psums, pcounts, n, d, k); \
+    else                                                                                        \
+      hipLaunchKernelGGL((lloyd_valu_fused_kernel<T, DREG, 1>), dim3(grid), dim3(WG), lds, s,   \
+                         X, xnorm, C, cnorm, labels, mindist, psums, pcounts, n, d, k);         \
+  } while (0)
+  if (lds > 64 * 1024) {
+    KM_HIP_TRY(hipFuncSetAttribute(
+        reinterpret_cast<const void *>(lloyd_valu_fused_kernel<T, 64, Mfma<T>::VW>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(lloyd_valu_fused_kernel<T, 64, 1>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  }
+  if (d <= 16) KM_VF(16);
+  else if (d <= 32) KM_VF(32);
+  else KM_VF(64);
+#undef KM_VF
+  KM_HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+template <typename T>
+int launch_assign_accumulate(hipStream_t s, int variant, const T *X, const T *xnorm, const T *C,
                              const T *cnorm, int *labels, T *mindist, int64_t n, int d,
-                             int k, int num_cu, double *psums, int *pcounts, int *slots) {
+                             int k, int num_cu, double *psums, int *pcounts, int *slots,
+                             int *used) {
   if (n <= 0 || d < 1 || k < 1) return H2O4GPU_KMEANS_EARG;
+  const int v = pick_assign_variant<T>(variant, n, d, k);
+  if (used) *used = v;
+  if (v == ASSIGN_VALU && valu_fused_applies(d, k))
+    return launch_valu_fused<T>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu, psums,
+                                pcounts, slots);
+  if (v != ASSIGN_ROWSTAT) return H2O4GPU_KMEANS_EARG;
   return RowstatDispatch<T, true>::run(s, X, xnorm, C, cnorm, labels, mindist, n, d, k,
                                        num_cu, psums, pcounts, slots);
 }
@@ -922,12 +1085,14 @@ int launch_transform(hipStream_t s, const T *X, const T *xnorm, const T *C,
 
 template int fused_slots<float>(int, int64_t, int, int, int);
 template int fused_slots<double>(int, int64_t, int, int, int);
-template int launch_assign_accumulate<float>(hipStream_t, const float *, const float *,
+template int launch_assign_accumulate<float>(hipStream_t, int, const float *, const float *,
                                              const float *, const float *, int *, float *,
-                                             int64_t, int, int, int, double *, int *, int *);
-template int launch_assign_accumulate<double>(hipStream_t, const double *, const double *,
+                                             int64_t, int, int, int, double *, int *, int *,
+                                             int *);
+template int launch_assign_accumulate<double>(hipStream_t, int, const double *, const double *,
                                               const double *, const double *, int *, double *,
-                                              int64_t, int, int, int, double *, int *, int *);
+                                              int64_t, int, int, int, double *, int *, int *,
+                                              int *);
 template int pick_assign_variant<float>(int, int64_t, int, int);
 template int pick_assign_variant<double>(int, int64_t, int, int);
 template int launch_assign<float>(hipStream_t, int, const float *, const float *,

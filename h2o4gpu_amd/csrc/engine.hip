@@ -454,9 +454,9 @@ struct Engine : h2o4gpu_kmeans_handle {
     if (opt_fuse && fused_slots<T>(opt_assign, n, d, k, num_cu) > 0) {
       int slots = 0;
       PROFILED("assign_accumulate",
-               launch_assign_accumulate<T>(stream, X, xnorm, C[cur], cnorm, labels, mindist, n, d,
-                                           k, num_cu, psums, pcounts, &slots));
-      last_variant = ASSIGN_ROWSTAT;
+               launch_assign_accumulate<T>(stream, opt_assign, X, xnorm, C[cur], cnorm, labels,
+                                           mindist, n, d, k, num_cu, psums, pcounts, &slots,
+                                           &last_variant));
       have_mindist = true;
       return finish_update(slots);
     }

@@ -66,7 +66,7 @@ template <typename T>
 int pick_assign_variant(int requested, int64_t n, int d, int k);
 const char *assign_variant_name(int variant);
 
-// Fused assign + accumulate (row-stationary shapes only): labels/mindist as
+// Fused assign + accumulate (row-stationary MFMA shapes and the small VALU shapes): labels/mindist as
 // launch_assign, plus per-workgroup partial sums psums[slot][k][d] and counts
 // pcounts[slot][k]; *slots receives the number of slots written. fused_slots()
 // returns the largest slot count the launch can use, or 0 when the shape (or a
@@ -74,9 +74,10 @@ const char *assign_variant_name(int variant);
 template <typename T>
 int fused_slots(int requested_variant, int64_t n, int d, int k, int num_cu);
 template <typename T>
-int launch_assign_accumulate(hipStream_t s, const T *X, const T *xnorm, const T *C,
+int launch_assign_accumulate(hipStream_t s, int variant, const T *X, const T *xnorm, const T *C,
                              const T *cnorm, int *labels, T *mindist, int64_t n, int d,
-                             int k, int num_cu, double *psums, int *pcounts, int *slots);
+                             int k, int num_cu, double *psums, int *pcounts, int *slots,
+                             int *used);
 
 // Full squared-distance matrix, centroid-major: D[c * ldn + i], i < n.
 template <typename T>

@@ -181,6 +181,34 @@ def test_fused_step_equals_separate_kernels(hip, oracle, n, d, k, dtype):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n,d,k", [(100000, 16, 8), (5001, 3, 2), (777, 64, 16), (3000, 33, 11), (256, 8, 1)])
+def test_small_shape_fused_step_is_bit_exact(hip, oracle, n, d, k, dtype):
+    """k <= 16 and d <= 64: the one-pass VALU step. Labels and minimum distances are
+    bit-identical to the scalar CPU loop; float32 centroids are bit-identical to the
+    oracle update (exact double sums, rounded once)."""
+    X = blobs(n, d, max(k, 2), dtype, seed=n + k)
+    C0 = np.ascontiguousarray(X[RNG.choice(n, size=k, replace=False)])
+    res = {}
+    for fuse in (1, 0):
+        with hip.Handle(n, d, k, dtype) as h:
+            h.set_data(X)
+            h.set_centroids(C0)
+            h.set_option("fuse", fuse)
+            assert h.assign_variant() == "valu"
+            h.iterate(1)
+            res[fuse] = (h.labels(), h.min_distances(), h.counts(), h.centroids())
+    wl, wm = oracle.assign(X, C0, return_mindist=True)
+    wC, wcounts = oracle.update(X, wl, C0)
+    for fuse in (1, 0):
+        L, M, counts, C = res[fuse]
+        assert np.array_equal(L, wl) and np.array_equal(M, wm) and np.array_equal(counts, wcounts)
+        if dtype == np.float32:
+            assert np.array_equal(C, wC)
+        else:
+            assert np.allclose(C, wC, rtol=1e-13, atol=1e-13)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_threshold_stop(hip, oracle, dtype):
     n, d, k = 6000, 8, 5
     # one start per blob (true centre + offset): no blob is split, so no row sits
