@@ -137,8 +137,9 @@ def main():
         roofline = {"bound": "mfma", "kernel": "%s (%s)" % (dom, variant), "achieved": tflops,
                     "peak": peak, "unit": "TFLOP/s", "frac": tflops / peak, "traffic": traffic}
     else:
-        gbps = (float(n) * d * s + 8.0 * n) / (assign_ms * 1e-3) / 1e9
-        roofline = {"bound": "hbm", "kernel": "assign (valu)", "achieved": gbps,
+        # per row: the row and its squared norm read, label and minimum distance written
+        gbps = float(n) * (d * s + s + 4 + s) / (assign_ms * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "kernel": "%s (valu)" % dom, "achieved": gbps,
                     "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": gbps / PEAK_HBM_GBPS,
                     "traffic": None}
     iter_gbps = bytes_per_iter / (ms_step * 1e-3) / 1e9

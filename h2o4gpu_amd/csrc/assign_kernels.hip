@@ -81,71 +81,109 @@ __global__ __launch_bounds__(WG) void assign_valu_kernel(
 // per-centroid accumulation in one pass over the data.
 //
 // Persistent workgroups walk over blocks of 256 rows. A block is fetched with
-// coalesced (16-byte where possible) loads into LDS, row stride odd so that
-// thread t reading row t is conflict-free; every thread then runs the same
-// scalar loop as assign_valu_kernel on its row (j ascending, multiply and add
-// rounded separately: bit-identical to a CPU loop), and adds its row into the
-// double-precision per-centroid sums of the workgroup. Sums and counts go to
-// the workgroup's slot psums[blockIdx.x][k][d], pcounts[blockIdx.x][k].
+// coalesced (16-byte where possible) loads into registers while the previous
+// block is being processed, then written to LDS with an odd row stride so that
+// thread t reading row t is conflict-free. Every thread runs the same scalar
+// loop as assign_valu_kernel on its row (j ascending, multiply and add rounded
+// separately: bit-identical to a CPU loop); the centroid values have a
+// wavefront-uniform address and are read straight from global memory, which
+// lets them travel through the scalar path instead of LDS. The thread then
+// adds its row into the double-precision per-centroid sums of the workgroup.
+// Sums and counts go to the workgroup's slot psums[blockIdx.x][k][d],
+// pcounts[blockIdx.x][k].
 // This is the HBM-bound regime: 2*k*d flop per row against d*s bytes.
+// FULL: d == DREG, no per-feature guards.
 // ---------------------------------------------------------------------------
-template <typename T, int DREG, int VEC>
+template <typename T, int VEC>
+struct BlockLoad {  // VEC is Mfma<T>::VW (one 16-byte load) or 1
+  typedef typename Mfma<T>::vec_t type;
+};
+template <typename T>
+struct BlockLoad<T, 1> {
+  typedef T type;
+};
+template <typename T, int DREG, int VEC, bool FULL>
 __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
     const T *__restrict__ X, const T *__restrict__ xnorm, const T *__restrict__ C,
     const T *__restrict__ cnorm, int *__restrict__ labels, T *__restrict__ mindist,
-    double *__restrict__ psums, int *__restrict__ pcounts, int64_t n, int d, int k) {
+    double *__restrict__ psums, int *__restrict__ pcounts, int64_t n, int dd, int k) {
 #pragma clang fp contract(off)
   extern __shared__ __align__(16) unsigned char smem_raw[];
+  const int d = FULL ? DREG : dd;
   const int sx = d | 1;                                          // row stride of the staged block
   double *sums = reinterpret_cast<double *>(smem_raw);           // [k][sx]
-  T *Cs = reinterpret_cast<T *>(sums + (size_t)k * sx);          // [k][d]
-  T *ccs = Cs + (size_t)k * d;                                   // [k]
-  int *cnt = reinterpret_cast<int *>(ccs + k);                   // [k]
-  T *Xs = reinterpret_cast<T *>(cnt + k + ((k & 1) ? 1 : 0));    // [WG][sx]
+  int *cnt = reinterpret_cast<int *>(sums + (size_t)k * sx);     // [k]
+  T *Xs = reinterpret_cast<T *>(cnt + k + (k & 1));              // [WG][sx]
+  typedef typename BlockLoad<T, VEC>::type ld_t;
+  constexpr int NLD = DREG / VEC;  // loads per thread and block (upper bound)
   const int tid = threadIdx.x;
   for (int e = tid; e < k * sx; e += WG) sums[e] = 0.0;
-  for (int e = tid; e < k * d; e += WG) Cs[e] = C[e];
-  for (int c = tid; c < k; c += WG) {
-    ccs[c] = cnorm[c];
-    cnt[c] = 0;
-  }
-  __syncthreads();
-  for (int64_t base = (int64_t)blockIdx.x * WG; base < n; base += (int64_t)gridDim.x * WG) {
-    const int rows = (int)min<int64_t>(WG, n - base);
-    const int64_t total = (int64_t)rows * d;
-    const T *src = X + base * (int64_t)d;
-    if (VEC > 1) {
-      typedef typename Mfma<T>::vec_t vec_t;  // 16 bytes
-      const int64_t nv = total / VEC;
-      for (int64_t e = tid; e < nv; e += WG) {
-        const vec_t v = reinterpret_cast<const vec_t *>(src)[e];
-        const int el = (int)(e * VEC);
-        const int r = el / d, j = el - r * d;  // d % VEC == 0: a vector never straddles rows
+  for (int c = tid; c < k; c += WG) cnt[c] = 0;
+  // LDS offset of the i-th load of this thread: element (tid + i*WG)*VEC of the block
+  int off[NLD];
 #pragma unroll
-        for (int q = 0; q < VEC; q++) Xs[r * sx + j + q] = v[q];
-      }
-    } else {
-      for (int64_t e = tid; e < total; e += WG) {
-        const int r = (int)(e / d), j = (int)(e - (int64_t)r * d);
-        Xs[r * sx + j] = src[e];
+  for (int i = 0; i < NLD; i++) {
+    const int el = (tid + i * WG) * VEC;
+    const int r = el / d;
+    off[i] = r * sx + (el - r * d);
+  }
+  const int nld = d / VEC;  // loads per thread for a full block (d % VEC == 0)
+  ld_t pre[NLD];
+  T pre_xx = 0;  // squared norm of this thread's row in the fetched block
+  // Loads are never predicated: indices past the end of the data set are
+  // clamped instead, which keeps the loop free of divergent branches and lets
+  // the fetched block stay in flight across the processing of the current one.
+  auto fetch = [&](int64_t base) {
+    const int64_t last = (n - base) * d / VEC - 1;  // last load of the data set
+    const ld_t *src = reinterpret_cast<const ld_t *>(X + base * (int64_t)d);
+#pragma unroll
+    for (int i = 0; i < NLD; i++) {
+      const int64_t e = tid + i * WG;
+      if (FULL || i < nld) pre[i] = src[e < last ? e : last];
+    }
+    const int64_t r = base + tid;
+    pre_xx = xnorm[r < n ? r : n - 1];
+  };
+  const int64_t stride = (int64_t)gridDim.x * WG;
+  int64_t base = (int64_t)blockIdx.x * WG;
+  if (base >= n) return;  // the grid never exceeds the number of blocks
+  fetch(base);
+  const int jrot = (tid & 63) % d;
+  for (; base < n; base += stride) {
+    const int rows = (int)min<int64_t>(WG, n - base);
+    __syncthreads();  // the previous block has been consumed
+#pragma unroll
+    for (int i = 0; i < NLD; i++) {
+      if (FULL || i < nld) {  // rows past the end of a last, partial block hold clamped copies
+        if constexpr (VEC == 1) {
+          Xs[off[i]] = pre[i];
+        } else {
+#pragma unroll
+          for (int q = 0; q < VEC; q++) Xs[off[i] + q] = pre[i][q];
+        }
       }
     }
+    const T xx = pre_xx;
     __syncthreads();
+    // the next block travels while this one is processed: no other vector
+    // load is issued below, so nothing waits for these until the next round
+    fetch(base + stride < n ? base + stride : base);
     const int64_t row = base + tid;
     if (tid < rows) {
+      const T *xrow = Xs + tid * sx;
       T xr[DREG];
 #pragma unroll
-      for (int j = 0; j < DREG; j++) xr[j] = j < d ? Xs[tid * sx + j] : (T)0;
-      const T xx = xnorm[row];
+      for (int j = 0; j < DREG; j++) xr[j] = (FULL || j < d) ? xrow[j] : (T)0;
       T best = argmin_start<T>();
       int bidx = -1;
+#pragma unroll 2
       for (int c = 0; c < k; c++) {
-        const T *cp = Cs + (size_t)c * d;
+        const T *cp = C + (size_t)c * d;
         T dot = 0;
 #pragma unroll
         for (int j = 0; j < DREG; j++)
-          if (j < d) dot = dot + xr[j] * cp[j];
-        const T t = xx + ccs[c];
+          if (FULL || j < d) dot = dot + xr[j] * cp[j];
+        const T t = xx + cnorm[c];
         const T dist = fabs(t - (T)2 * dot);
         if (dist < best) {
           best = dist;
@@ -159,8 +197,7 @@ __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
         // lanes of a wavefront would otherwise all add to the same few addresses
         // at once, and same-address LDS atomics are served one lane at a time.
         double *srow = sums + (size_t)bidx * sx;
-        const T *xrow = Xs + tid * sx;
-        int j = (tid & 63) % d;
+        int j = jrot;
         for (int q = 0; q < d; q++) {
           unsafeAtomicAdd(srow + j, (double)xrow[j]);
           j = (j + 1 == d) ? 0 : j + 1;
@@ -168,8 +205,8 @@ __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
         atomicAdd(&cnt[bidx], 1);
       }
     }
-    __syncthreads();  // the staged block is overwritten next round
   }
+  __syncthreads();
   double *dst = psums + (size_t)blockIdx.x * k * d;
   for (int e = tid; e < k * d; e += WG) {
     const int c = e / d, j = e - c * d;
@@ -937,8 +974,8 @@ static bool valu_fused_applies(int d, int k) { return k <= 16 && d <= 64; }
 template <typename T>
 static size_t valu_fused_lds(int d, int k) {
   const int sx = d | 1;
-  return (size_t)k * sx * sizeof(double) + ((size_t)k * d + k) * sizeof(T) +
-         ((size_t)k + 1) * sizeof(int) + (size_t)WG * sx * sizeof(T) + 16;
+  return (size_t)k * sx * sizeof(double) + ((size_t)k + 1) * sizeof(int) +
+         (size_t)WG * sx * sizeof(T) + 16;
 }
 static int valu_fused_grid(int64_t n, size_t lds, int num_cu) {
   int per_cu = (int)((150 * 1024) / lds);
@@ -972,25 +1009,25 @@ static int launch_valu_fused(hipStream_t s, const T *X, const T *xnorm, const T 
   if (slots) *slots = grid;
   const int vw = Mfma<T>::VW;
   const bool vec = (d % vw == 0) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0);
-#define KM_VF(DREG)                                                                             \
-  do {                                                                                          \
-    if (vec)                                                                                    \
-      hipLaunchKernelGGL((lloyd_valu_fused_kernel<T, DREG, Mfma<T>::VW>), dim3(grid), dim3(WG), \
-                         lds, s, X, xnorm, C, cnorm, labels, mindist, psums, pcounts, n, d, k); \
-    else                                                                                        \
-      hipLaunchKernelGGL((lloyd_valu_fused_kernel<T, DREG, 1>), dim3(grid), dim3(WG), lds, s,   \
-                         X, xnorm, C, cnorm, labels, mindist, psums, pcounts, n, d, k);         \
+#define KM_VF_LAUNCH(DREG, VEC, FULL)                                                       \
+  do {                                                                                      \
+    auto kern = lloyd_valu_fused_kernel<T, DREG, VEC, FULL>;                                \
+    if (lds > 64 * 1024)                                                                    \
+      KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                  \
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(WG), lds, s, X, xnorm, C, cnorm, labels,      \
+                       mindist, psums, pcounts, n, d, k);                                   \
   } while (0)
-  if (lds > 64 * 1024) {
-    KM_HIP_TRY(hipFuncSetAttribute(
-        reinterpret_cast<const void *>(lloyd_valu_fused_kernel<T, 64, Mfma<T>::VW>),
-        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(lloyd_valu_fused_kernel<T, 64, 1>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-  }
+#define KM_VF(DREG)                                            \
+  do {                                                         \
+    if (vec && d == DREG) KM_VF_LAUNCH(DREG, Mfma<T>::VW, true); \
+    else if (vec) KM_VF_LAUNCH(DREG, Mfma<T>::VW, false);      \
+    else KM_VF_LAUNCH(DREG, 1, false);                         \
+  } while (0)
   if (d <= 16) KM_VF(16);
   else if (d <= 32) KM_VF(32);
   else KM_VF(64);
+#undef KM_VF_LAUNCH
 #undef KM_VF
   KM_HIP_TRY(hipGetLastError());
   return 0;

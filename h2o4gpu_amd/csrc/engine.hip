@@ -265,7 +265,7 @@ struct Engine : h2o4gpu_kmeans_handle {
       KM_TRY(dalloc(&bucket_cursor, k));
       KM_TRY(dalloc(&bucket_counts, k));
     }
-    KM_TRY(dalloc(&shift_partials, (kd + 31) / 32 + 1));
+    KM_TRY(dalloc(&shift_partials, (size_t)max_shift_partials(d, k) + 1));
     KM_TRY(dalloc(&shift2, 1));
     KM_TRY(dalloc(&sum_partials, sum_partials_needed() + 1));
     KM_TRY(dalloc(&kpp_bsums, (n + KPP_BLOCK - 1) / KPP_BLOCK + 1));

@@ -116,6 +116,12 @@ int launch_bucketed_accumulate(hipStream_t s, const T *X, const int *labels, int
 
 // Pass 2: fixed-order reduction of the partials, empty clusters keep the old
 // centroid, mean = sum * (1/count), per-block partial of sum((old-new)^2).
+// shift_partials must hold max_shift_partials(d, k) entries.
+static const int64_t FINALIZE_NARROW_KD = 4096;
+static inline int max_shift_partials(int d, int k) {
+  const int64_t kd = (int64_t)k * d;
+  return (int)(kd <= FINALIZE_NARROW_KD ? (kd + 3) / 4 : (kd + 31) / 32);
+}
 template <typename T>
 int launch_finalize(hipStream_t s, int slots, const double *psums,
                     const int *pcounts, const T *c_old, T *c_new, int *counts,

@@ -537,16 +537,18 @@ int launch_bucketed_accumulate(hipStream_t s, const T *X, const int *labels, int
 // ---------------------------------------------------------------------------
 // pass 2: finalize. One thread per centroid coordinate.
 // ---------------------------------------------------------------------------
-// A workgroup takes EPW = 32 consecutive coordinates; RS = 8 thread groups each
-// sum a contiguous range of the row-block slots for those coordinates (slot
-// order), then group 0 adds the 8 range sums in range order.
-template <typename T>
+// A workgroup takes EPW consecutive coordinates; RS = 256 / EPW thread groups
+// each sum a contiguous range of the row-block slots for those coordinates (slot
+// order), then group 0 adds the RS range sums in range order. EPW is 32, or 4
+// for a small model with many slots, where 32 would leave a handful of
+// workgroups walking thousands of slots one after the other.
+template <typename T, int EPW>
 __global__ __launch_bounds__(WG) void finalize_kernel(
     const double *__restrict__ psums, const int *__restrict__ pcounts, int row_blocks,
     const T *__restrict__ c_old, T *__restrict__ c_new, int *__restrict__ counts,
     T *__restrict__ shift_partials, int d, int k) {
 #pragma clang fp contract(off)
-  constexpr int EPW = 32, RS = WG / EPW;
+  constexpr int RS = WG / EPW;
   __shared__ double part[RS][EPW];
   __shared__ int cpart[RS][EPW];
   __shared__ T red[EPW];
@@ -617,9 +619,14 @@ int launch_finalize(hipStream_t s, int slots, const double *psums,
                     const int *pcounts, const T *c_old, T *c_new, int *counts,
                     T *shift_partials, int *n_shift_partials, int d, int k) {
   const int64_t kd = (int64_t)k * d;
-  const int blocks = (int)((kd + 31) / 32);
-  hipLaunchKernelGGL((finalize_kernel<T>), dim3(blocks), dim3(WG), 0, s, psums,
-                     pcounts, slots, c_old, c_new, counts, shift_partials, d, k);
+  const bool narrow = kd <= FINALIZE_NARROW_KD && slots >= 256;
+  const int blocks = narrow ? (int)((kd + 3) / 4) : (int)((kd + 31) / 32);
+  if (narrow)
+    hipLaunchKernelGGL((finalize_kernel<T, 4>), dim3(blocks), dim3(WG), 0, s, psums, pcounts,
+                       slots, c_old, c_new, counts, shift_partials, d, k);
+  else
+    hipLaunchKernelGGL((finalize_kernel<T, 32>), dim3(blocks), dim3(WG), 0, s, psums, pcounts,
+                       slots, c_old, c_new, counts, shift_partials, d, k);
   KM_HIP_TRY(hipGetLastError());
   *n_shift_partials = blocks;
   return 0;
