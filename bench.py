@@ -39,22 +39,81 @@ def log(msg):
     print("[bench] " + msg, file=sys.stderr, flush=True)
 
 
-def cpu_baseline(X, C0, iters):
-    """The CPU restatement (oracle port) timed on this host's cores: `iters` full
-    Lloyd iterations (assign + update) over all rows, all hardware threads."""
+def cpu_baseline(X, C0, iters, budget_s=12.0):
+    """The CPU restatement (oracle port) timed on this host's cores: full Lloyd
+    iterations (assign + update) over all rows, all hardware threads. With iters == 0
+    it runs whole iterations until `budget_s` seconds have passed (at least 3)."""
     from oracle import load_oracle
     orc = load_oracle()
     threads = min(os.cpu_count() or 1, orc.max_threads)
     C = C0.copy()
+    done = 0
     t0 = time.perf_counter()
-    for _ in range(iters):
+    while True:
         labels = orc.assign(X, C, threads=threads)
         C, _ = orc.update(X, labels, C, threads=threads)
-    dt = time.perf_counter() - t0
-    return {"value": iters / dt, "unit": "iter/s", "cores": threads, "kind": "port",
+        done += 1
+        dt = time.perf_counter() - t0
+        if iters > 0 and done >= iters:
+            break
+        if iters <= 0 and done >= 3 and (dt >= budget_s or done >= 200):
+            break
+    return {"value": done / dt, "unit": "iter/s", "cores": threads, "kind": "port",
             "sample": "%d full Lloyd iterations (assign+update) over all %d rows, "
-                      "C++/OpenMP restatement of the reference semantics" % (iters, X.shape[0]),
+                      "C++/OpenMP restatement of the reference semantics" % (done, X.shape[0]),
             "seconds": dt}
+
+
+def sklearn_baseline(X, C0, sample_rows, iters=5):
+    """The reference's CPU fallback (kmeans.py:713-750 hands the fit to scikit-learn's
+    KMeans): Lloyd from the same initial centroids on the first `sample_rows` rows, timed
+    around fit(); per-iteration time = wall / n_iter_ (validation, centring and the final
+    relabel included), scaled to the full row count."""
+    try:
+        import sklearn
+        from sklearn.cluster import KMeans as SkKMeans
+    except Exception as exc:  # not installed on this box
+        return {"available": False, "reason": repr(exc)}
+    import warnings
+    n = X.shape[0]
+    m = min(n, sample_rows)
+
+    def timed(rows, max_iter):
+        est = SkKMeans(n_clusters=C0.shape[0], init=C0.copy(), n_init=1, max_iter=max_iter, tol=0.0,
+                       algorithm="lloyd")
+        t0 = time.perf_counter()
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            est.fit(X[:rows])
+        return time.perf_counter() - t0, int(est.n_iter_)
+
+    timed(min(m, 50_000), 1)  # thread-pool start-up and lazy imports
+    dt, n_iter = timed(m, iters)
+    per_iter = dt / max(n_iter, 1) * (float(n) / m)
+    return {"available": True, "version": sklearn.__version__, "value": 1.0 / per_iter,
+            "unit": "iter/s", "cores": os.cpu_count() or 1,
+            "kind": "reference CPU fallback (scikit-learn)",
+            "sample": "KMeans(init=<same centroids>, n_init=1, max_iter=%d, tol=0, algorithm='lloyd')"
+                      ".fit on the first %d rows: wall / n_iter_ (%d), scaled by %d/%d rows"
+                      % (iters, m, n_iter, n, m),
+            "seconds": dt}
+
+
+def c_abi_fit(X, C0, iters):
+    """One whole fit through the reference's C entry point (host pointers in, host
+    results out): upload, row norms, `iters` Lloyd iterations, final relabel, download."""
+    from h2o4gpu_amd.libs import ch2o4gpu_gpu as shim
+    n, d = X.shape
+    k = C0.shape[0]
+    fn = shim.make_ptr_float_kmeans if X.dtype == np.float32 else shim.make_ptr_double_kmeans
+    cent = np.empty(k * d, X.dtype)
+    lab = np.empty(n, np.int32)
+    t0 = time.perf_counter()
+    rc = fn(0, 0, 0, 0, 1, n, d, k, iters, 2, 0.0, X.reshape(-1), C0.reshape(-1), cent, lab)
+    dt = time.perf_counter() - t0
+    return {"status": int(rc), "iterations": iters, "seconds": dt,
+            "note": "make_ptr_*_kmeans with init_from_data=2: pageable host memory in, "
+                    "malloc'ed results out"}
 
 
 def main():
@@ -71,7 +130,11 @@ def main():
     ap.add_argument("--transform-rows", type=int, default=0,
                     help="also time transform (full distance matrix) on this many held-out rows (C5)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-iters", type=int, default=0, help="CPU baseline iterations (0 = auto)")
+    ap.add_argument("--cpu-iters", type=int, default=0, help="CPU baseline iterations (0 = about 12 s worth)")
+    ap.add_argument("--sklearn-rows", type=int, default=10_000_000,
+                    help="rows of the workload the scikit-learn leg runs on")
+    ap.add_argument("--end-to-end", action="store_true",
+                    help="also time one whole fit through make_ptr_*_kmeans (upload included)")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -186,12 +249,10 @@ def main():
     if transform:
         out["transform"] = transform
     if not args.no_cpu:
-        iters = args.cpu_iters
-        if iters <= 0:
-            # ~10-30 s of CPU work: assume ~5 GFLOP/s per core for the estimate
-            est = flops_per_iter / (5e9 * (os.cpu_count() or 1))
-            iters = int(max(1, min(5, round(20.0 / max(est, 1e-3)))))
-        out["cpu_baseline"] = cpu_baseline(X, C0, iters)
+        out["cpu_baseline"] = cpu_baseline(X, C0, args.cpu_iters)
+        out["cpu_reference_path"] = sklearn_baseline(X, C0, args.sklearn_rows)
+    if args.end_to_end:
+        out["c_abi_fit"] = c_abi_fit(X, C0, datasets.SHAPES[args.workload][4])
     print(json.dumps(out), flush=True)
     return 0
 
