@@ -678,6 +678,15 @@ __global__ void copy_probe_kernel(const float4 *__restrict__ src, float4 *__rest
 // ---------------------------------------------------------------------------
 // C ABI, part 1: the reference's entry points
 // ---------------------------------------------------------------------------
+// Inertia and iteration count of the calling thread's most recent successful fit
+// through make_ptr_*_kmeans: the reference's signature has no slot for either.
+struct LastFitInfo {
+  bool valid = false;
+  double inertia = 0.0;
+  int iterations = 0;
+};
+static thread_local LastFitInfo g_last_fit;
+
 template <typename T>
 static int fit_entry(int verbose, int seed, int gpu_id, size_t rows, size_t cols, int k,
                      int max_iterations, int init_from_data, double threshold,
@@ -708,7 +717,12 @@ static int fit_entry(int verbose, int seed, int gpu_id, size_t rows, size_t cols
     }
   }
   int iters = 0;
+  double inertia = 0.0;
+  g_last_fit.valid = false;
   if (rc == 0) rc = h->fit(max_iterations, threshold, &iters);
+  // minimum distances of the final relabel; a run of zero iterations has none
+  bool have_inertia = false;
+  if (rc == 0) have_inertia = h->inertia(&inertia) == 0;
   T *oc = nullptr;
   int *ol = nullptr;
   if (rc == 0) {
@@ -727,7 +741,10 @@ static int fit_entry(int verbose, int seed, int gpu_id, size_t rows, size_t cols
   }
   *pred_centroids = oc;
   *pred_labels = ol;
-  log_msg(verbose, LOG_INFO, "fit: %d iterations", iters);
+  g_last_fit.valid = have_inertia;
+  g_last_fit.inertia = inertia;
+  g_last_fit.iterations = iters;
+  log_msg(verbose, LOG_INFO, "fit: %d iterations, inertia %.9g", iters, inertia);
   return 0;
 }
 
@@ -874,6 +891,13 @@ KM_API int h2o4gpu_kmeans_get_min_distances(h2o4gpu_kmeans_handle *h, void *m) {
   KM_CHECK_HANDLE(h);
   return m ? h->get_min_distances(m) : H2O4GPU_KMEANS_EARG;
 }
+KM_API int h2o4gpu_kmeans_last_fit_info(double *inertia, int *iterations) {
+  if (!g_last_fit.valid) return H2O4GPU_KMEANS_ESTATE;
+  if (inertia) *inertia = g_last_fit.inertia;
+  if (iterations) *iterations = g_last_fit.iterations;
+  return 0;
+}
+
 KM_API int h2o4gpu_kmeans_inertia(h2o4gpu_kmeans_handle *h, double *inertia) {
   KM_CHECK_HANDLE(h);
   return inertia ? h->inertia(inertia) : H2O4GPU_KMEANS_EARG;

@@ -147,3 +147,9 @@ def cudaresetdevice(wDev, nDev):
 
 def cudaresetdevice_bare():
     return _k.lib().cudaresetdevice_bare()
+
+
+def last_fit_info():
+    """(inertia, iterations) of this thread's last successful make_ptr_*_kmeans fit, or
+    None. Not part of the reference's module: its entry points cannot return either."""
+    return _k.last_fit_info()

@@ -39,6 +39,7 @@ PROTOTYPES = {
     "cudaresetdevice": (c_int, [c_int, c_int]),
     "cudaresetdevice_bare": (c_int, []),
     "h2o4gpu_kmeans_device_count": (c_int, []),
+    "h2o4gpu_kmeans_last_fit_info": (c_int, [P(c_double), P(c_int)]),
     "h2o4gpu_kmeans_create": (c_int, [P(c_void_p), c_int, c_size_t, c_size_t, c_int, c_int, c_int]),
     "h2o4gpu_kmeans_destroy": (c_int, [c_void_p]),
     "h2o4gpu_kmeans_set_data_host": (c_int, [c_void_p, c_void_p]),
@@ -277,6 +278,15 @@ def copy_probe(nbytes, reps=10, gpu_id=0):
     ms = c_float(0.0)
     _check("copy_probe", lib().h2o4gpu_kmeans_copy_probe(gpu_id, nbytes, reps, ctypes.byref(ms)))
     return ms.value
+
+
+def last_fit_info():
+    """(inertia, iterations) of this thread's last successful fit through the
+    make_ptr_*_kmeans entry points, or None when there is none."""
+    inertia, iters = c_double(0.0), c_int(0)
+    if lib().h2o4gpu_kmeans_last_fit_info(ctypes.byref(inertia), ctypes.byref(iters)) != 0:
+        return None
+    return float(inertia.value), int(iters.value)
 
 
 def device_count():

@@ -76,6 +76,7 @@ class KMeansH2O:
         self.cluster_centers_ = None
         self.labels_ = None
         self.inertia_ = None
+        self.n_iter_ = None
         self.sklearn_model = None
         self.double_precision = 0
 
@@ -181,23 +182,46 @@ class KMeansH2O:
             c_init = 1
         else:
             c_init = 0
-        pred_centers = np.zeros(cols * self._n_clusters, data.dtype)
-        pred_labels = np.zeros(rows, dtype=np.int32)
         fn = lib.make_ptr_float_kmeans if self.double_precision == 0 else lib.make_ptr_double_kmeans
-        status = fn(0, self.verbose, self.random_state, self._gpu_id, self.n_gpus, rows, cols,
-                    self._n_clusters, self._max_iter, c_init, self.tol, c_data, centroids,
-                    pred_centers, pred_labels)
-        if status != 0:
-            raise RuntimeError("KMeans fit failed in the native library (status %d)" % status)
+        # n_init restarts (seed, seed+1, ...) keep the lowest inertia; the reference runs one
+        # (kmeans.py:722-725). Restarts are pointless when the start is given.
+        restarts = 1 if c_init == 2 else max(1, int(self.n_init or 1))
+        best = None
+        for r in range(restarts):
+            pred_centers = np.zeros(cols * self._n_clusters, data.dtype)
+            pred_labels = np.zeros(rows, dtype=np.int32)
+            status = fn(0, self.verbose, self.random_state + r, self._gpu_id, self.n_gpus, rows,
+                        cols, self._n_clusters, self._max_iter, c_init, self.tol, c_data, centroids,
+                        pred_centers, pred_labels)
+            if status != 0:
+                raise RuntimeError("KMeans fit failed in the native library (status %d)" % status)
+            # a module that offers only the reference's entry points has no such getter
+            getter = getattr(lib, "last_fit_info", None)
+            info = getter() if getter is not None else None
+            inertia, n_iter = info if info is not None else (None, None)
+            if best is None or (inertia is not None and inertia < best[2]):
+                best = (pred_centers, pred_labels, inertia, n_iter)
+        pred_centers, pred_labels, self.inertia_, self.n_iter_ = best
         self.cluster_centers_ = np.reshape(pred_centers, (self._n_clusters, cols))
         self.labels_ = np.reshape(pred_labels, rows)
-        self.inertia_ = self._inertia(data)
         return self.cluster_centers_, self.labels_
 
-    def _inertia(self, data):
-        """Sum of squared distances of the rows to their centre, from the fitted result."""
-        diff = data.astype(np.float64) - self.cluster_centers_.astype(np.float64)[self.labels_]
-        return float(np.einsum("ij,ij->", diff, diff))
+    def score(self, X, y=None):
+        """Opposite of the k-means objective of X under the fitted centres: the rows go to
+        the device once, one assignment pass, and the minimum distances are summed there."""
+        self._validate_centroids(X)
+        if self._load_lib() is None:
+            raise RuntimeError("score needs a usable GPU")
+        from ..libs import kmeans_hip
+        X_np = _to_np(X)
+        dtype = np.float64 if X_np.dtype == np.float64 else np.float32
+        X_np = np.ascontiguousarray(X_np, dtype=dtype)
+        with kmeans_hip.Handle(X_np.shape[0], X_np.shape[1], self._n_clusters, dtype,
+                               gpu_id=self._gpu_id, verbose=self.verbose) as h:
+            h.set_data(X_np)
+            h.set_centroids(np.ascontiguousarray(self.cluster_centers_, dtype=dtype))
+            h.assign()
+            return -h.inertia()
 
     def _toc(self, data, convert=True):
         if convert and data.dtype != np.float64 and data.dtype != np.float32:
@@ -277,8 +301,6 @@ class KMeans:
         if _backend is not None:
             backend = _backend
         self.do_sklearn = backend == 'sklearn'
-        if backend == 'auto' and n_init != 1:
-            KMeans._print_verbose(verbose, 0, "'n_init' not supported. Running h2o4gpu with n_init = 1.")
         self.model_h2o4gpu = KMeansH2O(n_clusters=n_clusters, init=init, n_init=n_init, max_iter=max_iter,
                                        tol=tol, precompute_distances=precompute_distances,
                                        verbose=verbose, random_state=random_state, copy_x=copy_x,
@@ -343,8 +365,7 @@ class KMeans:
         """Opposite of the k-means objective on X (scikit-learn's definition)."""
         if self.backend == 'sklearn':
             return self.model.score(X, y)
-        D = self.model.transform(X)
-        return -float(np.min(D, axis=1).astype(np.float64).sum())
+        return self.model.score(X, y)
 
     def set_params(self, **params):
         res = self.model.set_params(**params)
@@ -357,7 +378,7 @@ class KMeans:
         return res
 
     def set_attributes(self):
-        for name in ("cluster_centers_", "labels_", "inertia_"):
+        for name in ("cluster_centers_", "labels_", "inertia_", "n_iter_"):
             setattr(self, name, getattr(self.model, name, None))
 
     @staticmethod

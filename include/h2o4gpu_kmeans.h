@@ -63,6 +63,16 @@ int make_ptr_double_kmeans(int dopredict, int verbose, int seed, int gpu_id,
                            const double *centroids, double **pred_centroids,
                            int **pred_labels);
 
+/* Inertia (sum over rows of the squared distance to the assigned centroid,
+ * accumulated in double in a fixed order) and number of Lloyd iterations of
+ * the calling thread's most recent successful fit through make_ptr_*_kmeans.
+ * Either pointer may be NULL. Returns H2O4GPU_KMEANS_ESTATE when the thread
+ * has no successful fit yet.
+ * No counterpart in the reference: its estimator leaves inertia_ at None
+ * (src/interface_py/h2o4gpu/solvers/kmeans.py:187) because the entry point
+ * has no slot to return it. */
+int h2o4gpu_kmeans_last_fit_info(double *inertia, int *iterations);
+
 /* Squared distances |xx + cc - 2 x.c| of every row to every centroid, no
  * sqrt, centroid-major: (*preds)[c * m + i]. malloc()ed, caller owns.
  * Replaces: kmeans_transform<T>, src/gpu/kmeans/kmeans_h2o4gpu.cu:891-975. */

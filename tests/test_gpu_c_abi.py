@@ -184,3 +184,50 @@ def test_estimator_round_trip(oracle, dtype):
     m3 = KMeans(n_clusters=2, init="random", max_iter=3, tol=0, random_state=1)
     m3.fit(np.array([[0, 0], [0, 1], [9, 9], [9, 8]]))
     assert m3.cluster_centers_.dtype == np.float32 and sorted(m3.labels_.tolist()) == [0, 0, 1, 1]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_last_fit_info_reports_inertia_and_iterations(shim, oracle, dtype):
+    """The side channel of the fit entry point: inertia equals the exact (float64, brute
+    force) objective of the returned labels and centroids, the iteration count follows the
+    reference's stop rule, and a thread that never fitted has nothing to report."""
+    import threading
+    X, centers = blobs(4000, 7, 5, dtype, 11)
+    C0 = (centers + 0.2).astype(dtype)
+    rc, C, L = fit(shim, X, 5, 6, 2, C0=C0)          # tol = 0: all 6 iterations run
+    assert rc == 0
+    inertia, iters = shim.last_fit_info()
+    assert iters == 6
+    want = ((X.astype(np.float64) - C.astype(np.float64)[L]) ** 2).sum()
+    assert abs(inertia - want) <= (1e-5 if dtype == np.float32 else 1e-11) * want
+    wC, wL, w_it, _ = oracle.lloyd(X, C0, 50, 1e-3)   # stops early on the shift threshold
+    rc, C, L = fit(shim, X, 5, 50, 2, tol=1e-3, C0=C0)
+    # the oracle returns the loop index at the break as the reference does
+    # (kmeans_impl.h:246); the entry point reports the number of updates made, one more
+    assert rc == 0 and shim.last_fit_info()[1] == w_it + 1 < 50
+    seen = []
+    t = threading.Thread(target=lambda: seen.append(shim.last_fit_info()))
+    t.start()
+    t.join()
+    assert seen == [None]
+
+
+def test_estimator_restarts_and_score(oracle):
+    """n_init restarts keep the best of the seeds seed, seed+1, ...; n_iter_ and inertia_
+    come from the native fit; score is the negated objective on new rows."""
+    from h2o4gpu_amd import KMeans
+    Xb, _ = blobs(6000, 6, 8, np.float32, 21)
+    singles = []
+    for seed in (40, 41, 42, 43):
+        m = KMeans(n_clusters=8, init="random", max_iter=30, tol=1e-6, random_state=seed)
+        m.fit(Xb)
+        assert 1 <= m.n_iter_ <= 30
+        singles.append(m.inertia_)
+    multi = KMeans(n_clusters=8, init="random", n_init=4, max_iter=30, tol=1e-6, random_state=40)
+    multi.fit(Xb)
+    assert multi.inertia_ == min(singles)
+    want = ((Xb.astype(np.float64) - multi.cluster_centers_.astype(np.float64)[multi.labels_]) ** 2).sum()
+    assert abs(multi.inertia_ - want) <= 1e-5 * want
+    Xn, _ = blobs(1500, 6, 8, np.float32, 22)
+    d2 = ((Xn[:, None, :].astype(np.float64) - multi.cluster_centers_[None].astype(np.float64)) ** 2).sum(-1)
+    assert abs(multi.score(Xn) + d2.min(1).sum()) <= 1e-5 * d2.min(1).sum()
