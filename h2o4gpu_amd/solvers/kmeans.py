@@ -9,7 +9,12 @@ on top of the gfx950 engine. Differences, all additive:
     scikit-learn backend;
   * `inertia_` is filled after fit (the reference leaves it None, :187);
   * when scikit-learn is chosen as backend it is the installed scikit-learn (the
-    reference uses its own renamed copy).
+    reference uses its own renamed copy);
+  * `n_init` restarts, `n_iter_` and a native `score`;
+  * fit / predict / score / transform accept rows that already live on the GPU (any
+    object with `__cuda_array_interface__`, e.g. a PyTorch-ROCm tensor): the engine adopts
+    the pointer, nothing crosses PCIe (the reference re-uploads the rows on every call,
+    kmeans_h2o4gpu.cu:679,857,930).
 """
 import sys
 
@@ -19,14 +24,46 @@ import numpy as np
 def _to_np(data):
     """Reference solvers/utils.py:_get_data/_to_np for the dense-matrix case: numpy
     array, 2-D, float32 unless the data already is float64/float32."""
-    if hasattr(data, "values") and not isinstance(data, np.ndarray):  # pandas
-        data = data.values
+    if not isinstance(data, np.ndarray) and not callable(getattr(data, "values", data.__class__)):
+        data = data.values  # pandas (a tensor's `values` is a method and stays as it is)
     arr = np.asarray(data)
     if arr.ndim == 1:
         arr = arr.reshape(-1, 1)
     if arr.dtype not in (np.float32, np.float64):
         arr = arr.astype(np.float32)
     return arr
+
+
+class _DeviceRows:
+    """A C-contiguous (rows, cols) float32/float64 array in device memory."""
+
+    def __init__(self, owner, ptr, rows, cols, dtype):
+        self.owner, self.ptr, self.rows, self.cols, self.dtype = owner, ptr, rows, cols, dtype
+
+
+def _device_rows(X):
+    """_DeviceRows for an object exposing `__cuda_array_interface__`, else None. Work
+    queued on the array by its owner must have finished; for PyTorch tensors the current
+    stream is synchronised here."""
+    try:
+        cai = getattr(X, "__cuda_array_interface__", None)
+    except Exception:  # PyTorch raises for CPU tensors and tensors that require grad
+        return None
+    if not isinstance(cai, dict):
+        return None
+    shape = tuple(cai["shape"])
+    dtype = np.dtype(cai["typestr"])
+    if dtype not in (np.dtype(np.float32), np.dtype(np.float64)):
+        raise TypeError("device input must be float32 or float64, got %s" % dtype)
+    if len(shape) != 2:
+        raise ValueError("device input must be 2-D (rows, cols), got shape %s" % (shape,))
+    strides = cai.get("strides")
+    if strides is not None and tuple(strides) != (shape[1] * dtype.itemsize, dtype.itemsize):
+        raise ValueError("device input must be C-contiguous")
+    torch = sys.modules.get("torch")
+    if torch is not None and isinstance(X, torch.Tensor):
+        torch.cuda.current_stream(X.device).synchronize()
+    return _DeviceRows(X, int(cai["data"][0]), int(shape[0]), int(shape[1]), dtype)
 
 
 def _check_data_content(do_check, name, data):
@@ -101,11 +138,51 @@ class KMeansH2O:
         return self
 
     def fit(self, X, y=None):
-        X_np = _to_np(X)
-        _check_data_content(self.do_checks, "X", X_np)
-        self._fit(X_np)
+        dev = _device_rows(X)
+        if dev is not None:
+            self._fit_device(dev)
+        else:
+            X_np = _to_np(X)
+            _check_data_content(self.do_checks, "X", X_np)
+            self._fit(X_np)
         self._did_sklearn_fit = 0
         return self
+
+    def _device_handle(self, dev, k):
+        """A handle that adopts the device rows (no copy)."""
+        if self._load_lib() is None:
+            raise RuntimeError("device input needs a usable GPU")
+        from ..libs import kmeans_hip
+        h = kmeans_hip.Handle(dev.rows, dev.cols, k, dev.dtype, gpu_id=self._gpu_id, verbose=self.verbose)
+        h.set_data_device(dev.ptr, keepalive=dev.owner)
+        return h
+
+    def _fit_device(self, dev):
+        """fit on rows resident in device memory, through the handle entry points: same
+        start rules, loop and outputs as the host-pointer entry point."""
+        self.double_precision = 1 if dev.dtype == np.float64 else 0
+        k = min(self._n_clusters, dev.rows)  # clamp as kmeans_h2o4gpu.cu:630-635
+        start = None
+        if isinstance(self.init, np.ndarray):
+            assert self.init.shape == (self._n_clusters, dev.cols), \
+                "init must have shape (n_clusters, n_features)"
+            start = np.ascontiguousarray(self.init[:k], dtype=dev.dtype)
+        restarts = 1 if start is not None else max(1, int(self.n_init or 1))
+        best = None
+        with self._device_handle(dev, k) as h:
+            for r in range(restarts):
+                if start is not None:
+                    h.set_centroids(start)
+                elif self.init == "k-means++":
+                    h.init_plusplus(self.random_state + r)
+                else:
+                    h.init_random_rows(self.random_state + r)
+                n_iter = h.fit(self._max_iter, self.tol)
+                inertia = h.inertia() if self._max_iter > 0 else None
+                if best is None or (inertia is not None and inertia < best[2]):
+                    best = (h.centroids(), h.labels(), inertia, n_iter)
+        self.cluster_centers_, self.labels_, self.inertia_, self.n_iter_ = best
+        return self.cluster_centers_, self.labels_
 
     def sklearn_fit(self, X, y=None):
         assert self.cluster_centers_ is not None, "Centroids are None. Run fit() first."
@@ -122,6 +199,12 @@ class KMeansH2O:
     def predict(self, X):
         lib = self._load_lib()
         cols, rows = self._validate_centroids(X)
+        dev = _device_rows(X)
+        if dev is not None:
+            with self._device_handle(dev, self.cluster_centers_.shape[0]) as h:
+                h.set_centroids(self.cluster_centers_)
+                h.assign()
+                return h.labels()
         X_np = _to_np(X)
         _check_data_content(self.do_checks, "X", X_np)
         c_X_np = self._toc(X_np)
@@ -143,6 +226,9 @@ class KMeansH2O:
         the squared values, kmeans.py:389-422 with kmeans_h2o4gpu.cu:937-950)."""
         lib = self._load_lib()
         cols, rows = self._validate_centroids(X)
+        dev = _device_rows(X)
+        if dev is not None:
+            return self._transform_device(X, dev)
         X_np = _to_np(X)
         c_X_np = self._toc(X_np)
         cluster_centers_ = self._toc(self.cluster_centers_, convert=False)
@@ -154,6 +240,22 @@ class KMeansH2O:
             lib.kmeans_transform_double(self.verbose, self._gpu_id, self.n_gpus, rows, cols,
                                         self._n_clusters, c_X_np, cluster_centers_, c_res)
         return np.reshape(c_res, (rows, self._n_clusters), order='F')
+
+    def _transform_device(self, X, dev):
+        """Distances of device rows, left on the device: a (rows, k) view of the engine's
+        centroid-major [k][rows] result, i.e. the same Fortran-ordered layout the host path
+        returns. The output buffer comes from the array's own library."""
+        torch = sys.modules.get("torch")
+        if torch is None or not isinstance(X, torch.Tensor):
+            raise TypeError("transform of device rows returns a device array and is available "
+                            "for PyTorch tensors; pass host rows otherwise")
+        k = self.cluster_centers_.shape[0]
+        out = torch.empty((k, dev.rows), dtype=X.dtype, device=X.device)
+        torch.cuda.current_stream(X.device).synchronize()
+        with self._device_handle(dev, k) as h:
+            h.set_centroids(self.cluster_centers_)
+            h.transform_resident(out.data_ptr())
+        return out.t()
 
     def sklearn_transform(self, X, y=None):
         _check_data_content(self.do_checks, "X", X)
@@ -213,6 +315,12 @@ class KMeansH2O:
         if self._load_lib() is None:
             raise RuntimeError("score needs a usable GPU")
         from ..libs import kmeans_hip
+        dev = _device_rows(X)
+        if dev is not None:
+            with self._device_handle(dev, self.cluster_centers_.shape[0]) as h:
+                h.set_centroids(self.cluster_centers_)
+                h.assign()
+                return -h.inertia()
         X_np = _to_np(X)
         dtype = np.float64 if X_np.dtype == np.float64 else np.float32
         X_np = np.ascontiguousarray(X_np, dtype=dtype)
