@@ -274,3 +274,87 @@ def test_kmeanspp_seeding(hip, oracle, n, d, k, seed, dtype):
         pot_o = want_mind.astype(np.float64).sum()
         assert abs(pot_g - pot_o) <= 0.2 * pot_o
         print("k-means++ picks diverged at pick %d of %d" % (i, k))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("variant", ["valu", "mfma_rowstat", "mfma_tiled"])
+def test_non_finite_rows_and_centroids(hip, oracle, variant, dtype):
+    """NaN / infinity follow the reference's relabel rule (kmeans_labels.h:360-377): a
+    distance that is not below FLT_MAX never wins, a row with no such distance gets
+    label -1 and is left out of the sums; a centroid holding a NaN is never chosen;
+    rows and centroids next to them are unaffected."""
+    n, d, k = 2048, 32, 40
+    X = blobs(n, d, k, dtype, seed=99)
+    C = np.ascontiguousarray(X[RNG.choice(n, size=k, replace=False)])
+    X[5, 3] = np.nan
+    X[70, :] = np.nan
+    X[130, 0] = np.inf
+    X[131, 7] = -np.inf
+    X[1999, d - 1] = np.nan
+    C[4, 2] = np.nan
+    C[17, :] = np.inf
+    bad_rows = [5, 70, 130, 131, 1999]
+    with hip.Handle(n, d, k, dtype) as h:
+        h.set_data(X)
+        h.set_centroids(C)
+        h.set_option("assign", variant)
+        if h.assign_variant() == "unsupported":
+            pytest.skip("shape outside %s" % variant)
+        h.assign()
+        got = h.labels()
+        h.update()
+        counts = h.counts()
+        newC = h.centroids()
+    want = oracle.assign(X, C)
+    assert np.all(want[bad_rows] == -1) and np.all(got[bad_rows] == -1)
+    assert not np.any(np.isin(got, [4, 17])) and not np.any(np.isin(want, [4, 17]))
+    good = np.ones(n, bool)
+    good[bad_rows] = False
+    Cf = np.delete(C, [4, 17], axis=0)   # near-tie analysis on the finite part only
+    remap = np.delete(np.arange(k), [4, 17])
+    inv = {int(c): i for i, c in enumerate(remap)}
+    g2 = np.array([inv[int(c)] for c in got[good]], np.int32)
+    w2 = np.array([inv[int(c)] for c in want[good]], np.int32)
+    if variant == "valu":
+        assert np.array_equal(g2, w2)
+    else:
+        label_report(oracle, np.ascontiguousarray(X[good]), np.ascontiguousarray(Cf), g2, w2)
+    wC, wcounts = oracle.update(X, got, C)
+    assert np.array_equal(counts, wcounts) and counts.sum() == n - len(bad_rows)
+    keep = counts > 0
+    tol = 1e-5 if dtype == np.float32 else 1e-12
+    assert np.allclose(newC[keep], wC[keep], rtol=tol, atol=tol * np.abs(wC[keep]).max())
+    # empty clusters (the two poisoned ones among them) keep their old coordinates, NaN included
+    assert np.array_equal(newC[~keep], C[~keep], equal_nan=True)
+
+
+def test_more_than_two_to_the_31_elements(hip, oracle):
+    """Row offsets are 64-bit: 70,000,000 x 32 float32 (2.24e9 elements, 8.96 GB) through
+    the fused step, checked on the first, middle and last rows against the oracle and by
+    mass conservation."""
+    n, d, k = 70_000_000, 32, 64
+    rng = np.random.default_rng(31)
+    centers = rng.uniform(-40, 40, size=(k, d)).astype(np.float32)
+    block = 1_000_000
+    base = (centers[rng.integers(0, k, size=block)] + rng.standard_normal((block, d), dtype=np.float32))
+    X = np.empty((n, d), np.float32)
+    for b in range(n // block):
+        np.add(base, np.float32(1e-3 * b), out=X[b * block:(b + 1) * block])
+    C0 = np.ascontiguousarray(centers + np.float32(0.3))
+    with hip.Handle(n, d, k, np.float32) as h:
+        h.set_data(X)
+        h.set_centroids(C0)
+        h.iterate(1)             # fused assign + sums, finalize
+        C1 = h.centroids()
+        counts = h.counts()
+        labels = h.labels()
+    assert counts.sum() == n
+    for lo in (0, 34_999_000, n - 3000):
+        rows = slice(lo, lo + 3000)
+        want = oracle.assign(np.ascontiguousarray(X[rows]), C0)
+        label_report(oracle, np.ascontiguousarray(X[rows]), C0, labels[rows], want)
+    assert np.array_equal(np.bincount(labels, minlength=k), counts)
+    # centroid of cluster c = mean of its rows: check two clusters in float64 on the host
+    for c in (0, k - 1):
+        m = X[labels == c].astype(np.float64).mean(0)
+        assert np.allclose(C1[c], m, rtol=1e-5, atol=1e-4)
