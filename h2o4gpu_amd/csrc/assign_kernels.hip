@@ -878,7 +878,10 @@ static size_t rowstat_fused_lds(int d, int k) {
 // Persistent grid of the row-stationary kernels: as many workgroups as stay
 // resident (two 4-wave workgroups per CU while two LDS images fit, otherwise
 // one 8-wave workgroup per CU), never more than there are row tiles.
-static bool rowstat_two_per_cu(size_t lds) { return lds <= 80 * 1024; }
+#ifndef KM_TWO_PER_CU_LIMIT
+#define KM_TWO_PER_CU_LIMIT (80 * 1024)
+#endif
+static bool rowstat_two_per_cu(size_t lds) { return lds <= (size_t)KM_TWO_PER_CU_LIMIT; }
 
 template <typename T, int DP, int ROWT, bool FUSE, int NW>
 static int launch_rowstat_nw(hipStream_t s, const T *X, const T *xnorm, const T *C,
