@@ -7,6 +7,8 @@
 // Kept from the reference: dist = |(xx + cc) - 2 x.c| with xx + cc rounded
 // first, strict '<' argmin, lowest index on ties, start value FLT_MAX, label -1
 // when nothing is below it.
+#include <type_traits>
+
 #include "kmeans_common.h"
 #include "mfma_traits.h"
 
@@ -622,10 +624,13 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 2 ? 2 : 1) void assign_tiled_k
   }
 
   vec_t areg[A_VECS], breg[B_VECS];
-  auto gload = [&](int c0, int st) {
+  // Only the last d-step can reach past the feature count: the guards live in a second
+  // instance of the loader (tail_tag true) used for that step alone.
+  auto gload = [&](int c0, int st, auto tail_tag) {
+    constexpr bool TAILSTEP = DTAIL && decltype(tail_tag)::value;
     int j = st * BK + jj;
     bool jok = true;
-    if (DTAIL) {
+    if (TAILSTEP) {
       jok = j < d;
       j = VECLOAD ? min(j, d - VW) : j;
     }
@@ -636,7 +641,7 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 2 ? 2 : 1) void assign_tiled_k
       vec_t v;
       if (VECLOAD) {
         v = *reinterpret_cast<const vec_t *>(src + j);
-        if (DTAIL && !jok)
+        if (TAILSTEP && !jok)
 #pragma unroll
           for (int e = 0; e < VW; e++) v[e] = 0;
       } else {
@@ -677,13 +682,15 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 2 ? 2 : 1) void assign_tiled_k
         for (int rt = 0; rt < RT; rt++) acc[ct][rt][v] = xx[rt] + cc;
       }
     }
-    gload(c0, 0);
+    if (DTAIL && nstage == 1) gload(c0, 0, std::true_type{});
+    else gload(c0, 0, std::false_type{});
     __syncthreads();  // previous block's readers are done with buffer 0
     lstore(0);
     __syncthreads();
     for (int st = 0; st < nstage; st++) {
       const int buf = st & 1;
-      if (st + 1 < nstage) gload(c0, st + 1);
+      if (st + 2 < nstage || (!DTAIL && st + 1 < nstage)) gload(c0, st + 1, std::false_type{});
+      else if (st + 1 < nstage) gload(c0, st + 1, std::true_type{});
       const vec_t *ap = reinterpret_cast<const vec_t *>(As + buf * A_ELEMS);
       const vec_t *bp = reinterpret_cast<const vec_t *>(Bs + buf * B_ELEMS);
 #pragma unroll
