@@ -149,8 +149,8 @@ __device__ __forceinline__ void add_row_slice(double *srow, const T *xrow, int c
 
 // sd = LDS row stride of the sums (>= d): chosen odd-ish by the host so that
 // rows of different centroids do not all start on the same bank.
-template <typename T, int VEC>
-__global__ __launch_bounds__(WG) void accumulate_kernel(
+template <typename T, int VEC, int TPB>
+__global__ __launch_bounds__(TPB) void accumulate_kernel(
     const T *__restrict__ X, const int *__restrict__ labels,
     double *__restrict__ psums, int *__restrict__ pcounts, int64_t n, int d, int k,
     int kc, int64_t rows_per_block, int lpr, int sd) {
@@ -161,8 +161,8 @@ __global__ __launch_bounds__(WG) void accumulate_kernel(
   const int lane = tid & 63, wave = tid >> 6;
   const int k0 = blockIdx.y * kc;
   const int nk = min(kc, k - k0);
-  for (int e = tid; e < nk * sd; e += WG) sums[e] = 0.0;
-  for (int c = tid; c < nk; c += WG) cnt[c] = 0;
+  for (int e = tid; e < nk * sd; e += TPB) sums[e] = 0.0;
+  for (int c = tid; c < nk; c += TPB) cnt[c] = 0;
   __syncthreads();
 
   const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
@@ -173,7 +173,7 @@ __global__ __launch_bounds__(WG) void accumulate_kernel(
   const bool narrow = d <= lpr * VEC;  // one vector per lane covers a row
   constexpr int U = 8;
 
-  for (int64_t g0 = r0 + (int64_t)wave * 64; g0 < r1; g0 += (WG / 64) * 64) {
+  for (int64_t g0 = r0 + (int64_t)wave * 64; g0 < r1; g0 += (TPB / 64) * 64) {
     const int64_t myrow = g0 + lane;
     int lab = -1;
     if (myrow < r1) lab = labels[myrow] - k0;
@@ -228,24 +228,28 @@ __global__ __launch_bounds__(WG) void accumulate_kernel(
   }
   __syncthreads();
   double *dst = psums + ((size_t)blockIdx.x * k + k0) * d;
-  for (int e = tid; e < nk * d; e += WG) {
+  for (int e = tid; e < nk * d; e += TPB) {
     const int c = e / d, j = e - c * d;
     dst[e] = sums[(size_t)c * sd + j];
   }
   int *cdst = pcounts + (size_t)blockIdx.x * k + k0;
-  for (int c = tid; c < nk; c += WG) cdst[c] = cnt[c];
+  for (int c = tid; c < nk; c += TPB) cdst[c] = cnt[c];
 }
 
 // LDS row stride of the sums (in doubles): odd, so that the rows of different
 // centroids start on different banks.
 static int update_lds_stride(int d) { return d | 1; }
+static constexpr size_t UPDATE_LDS_MAX = 150 * 1024;
 
 template <typename T>
 UpdatePlan plan_update(int64_t n, int d, int k, int num_cu) {
   UpdatePlan p;
   p.sd = update_lds_stride(d);
   const size_t per_centroid = (size_t)p.sd * sizeof(double) + sizeof(int);
-  const size_t budget = 64 * 1024;
+  // One chunk whenever all sums fit a CU's LDS (the kernel then runs one 1024-thread
+  // workgroup per CU); otherwise chunks of 64 KB.
+  const size_t whole = (size_t)k * per_centroid;
+  const size_t budget = whole <= UPDATE_LDS_MAX ? whole : 64 * 1024;
   int kc = (int)(budget / per_centroid);
   if (kc < 1) kc = 1;
   if (kc > k) kc = k;
@@ -257,7 +261,9 @@ UpdatePlan plan_update(int64_t n, int d, int k, int num_cu) {
   else if (d % 2 == 0) p.vec = 2;
   // enough workgroups to cover the machine a few times, but bounded so the
   // partials buffer (row_blocks * k * d) stays small next to the data
-  int64_t want = (int64_t)num_cu * 4 / p.k_chunks;
+  // (fewer when a workgroup's LDS image leaves room for only one or two per CU)
+  const int per_cu = p.lds_bytes > 80 * 1024 ? 1 : (p.lds_bytes > 40 * 1024 ? 2 : 4);
+  int64_t want = (int64_t)num_cu * per_cu / p.k_chunks;
   if (want < 1) want = 1;
   int64_t max_by_rows = (n + 1023) / 1024;  // at least 1024 rows per block
   if (max_by_rows < 1) max_by_rows = 1;
@@ -278,13 +284,19 @@ static int launch_accumulate_vec(hipStream_t s, const UpdatePlan &p, const T *X,
   int groups = (d + VEC - 1) / VEC;  // lanes wanted per row
   int lpr = 1;
   while (lpr < groups && lpr < 64) lpr <<= 1;
-  auto kern = accumulate_kernel<T, VEC>;
-  if (p.lds_bytes > 64 * 1024)
+  // a large LDS image means one workgroup per CU: make it 16 wavefronts
+  if (p.lds_bytes > 64 * 1024) {
+    auto kern = accumulate_kernel<T, VEC, 1024>;
     KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                    hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)p.lds_bytes));
-  hipLaunchKernelGGL(kern, dim3(p.row_blocks, p.k_chunks), dim3(WG), p.lds_bytes, s,
-                     X, labels, psums, pcounts, n, d, k, p.kc, rows_per_block, lpr, p.sd);
+    hipLaunchKernelGGL(kern, dim3(p.row_blocks, p.k_chunks), dim3(1024), p.lds_bytes, s, X, labels,
+                       psums, pcounts, n, d, k, p.kc, rows_per_block, lpr, p.sd);
+  } else {
+    auto kern = accumulate_kernel<T, VEC, WG>;
+    hipLaunchKernelGGL(kern, dim3(p.row_blocks, p.k_chunks), dim3(WG), p.lds_bytes, s, X, labels,
+                       psums, pcounts, n, d, k, p.kc, rows_per_block, lpr, p.sd);
+  }
   KM_HIP_TRY(hipGetLastError());
   return 0;
 }
