@@ -249,7 +249,12 @@ __device__ __forceinline__ int key_row(unsigned v, int g) {
 // different banks) and writes them to its own slot psums[blockIdx.x][k][d],
 // pcounts[blockIdx.x][k] when it has walked all its row tiles: the centroid
 // update then needs no second pass over the data.
-template <typename T, int DP, int ROWT, bool VECLOAD, bool FUSE, int NW>
+// LOAD: how a lane fetches its feature slice of a data row. 1: d == DP, 16-byte loads of
+// the slice as it lies in memory. 2: d < DP but d a multiple of the vector width: 16-byte
+// loads, a vector that would start at or past feature d re-reads the row's last valid
+// vector instead (finite x * 0 from the zero-padded centroid side adds nothing, and the
+// padded columns of the fused sums are never written back). 0: scalar loads, zero padded.
+template <typename T, int DP, int ROWT, int LOAD, bool FUSE, int NW>
 __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
     const T *__restrict__ X, const T *__restrict__ xnorm,
     const T *__restrict__ C, const T *__restrict__ cnorm,
@@ -263,6 +268,7 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
   static_assert(DCH % VW == 0, "DP must be a multiple of KL*VW");
   typedef typename M::acc_t acc_t;
   typedef typename M::vec_t vec_t;
+  constexpr bool VECLOAD = LOAD == 1;
 
   extern __shared__ __align__(16) unsigned char smem_raw[];
   T *Cs = reinterpret_cast<T *>(smem_raw);  // [KT][NV][64][VW]
@@ -342,6 +348,14 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
 #pragma unroll
         for (int q = 0; q < NV; q++) {
           vec_t v = src[q];
+#pragma unroll
+          for (int e = 0; e < VW; e++) xn[rt][q * VW + e] = v[e];
+        }
+      } else if (LOAD == 2) {
+        const T *src = X + row * (int64_t)d;
+#pragma unroll
+        for (int q = 0; q < NV; q++) {
+          const vec_t v = *reinterpret_cast<const vec_t *>(src + min(g * DCH + q * VW, d - VW));
 #pragma unroll
           for (int e = 0; e < VW; e++) xn[rt][q * VW + e] = v[e];
         }
@@ -831,7 +845,7 @@ static const size_t LDS_LIMIT = 160 * 1024;
 template <typename T>
 static int rowstat_dp(int d) {
   const int maxdp = sizeof(T) == 4 ? 128 : 64;
-  for (int dp = 16; dp <= maxdp; dp *= 2)
+  for (int dp = 8; dp <= maxdp; dp *= 2)
     if (d <= dp) return dp;
   return 0;
 }
@@ -867,7 +881,9 @@ static int launch_valu(hipStream_t s, const T *X, const T *xnorm, const T *C,
 #define KM_VALU(DREG)                                                          \
   hipLaunchKernelGGL((assign_valu_kernel<T, DREG, MODE>), grid, dim3(WG), lds, \
                      s, X, xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k, kc)
-  if (d <= 16) KM_VALU(16);
+  if (d <= 4) KM_VALU(4);
+  else if (d <= 8) KM_VALU(8);
+  else if (d <= 16) KM_VALU(16);
   else if (d <= 32) KM_VALU(32);
   else if (d <= 64) KM_VALU(64);
   else KM_VALU(0);
@@ -903,23 +919,23 @@ static int launch_rowstat_nw(hipStream_t s, const T *X, const T *xnorm, const T 
   if (grid > tiles) grid = tiles;
   if (grid < 1) grid = 1;
   if (slots) *slots = (int)grid;
-  const bool vec = (d == DP) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0) &&
-                   ((reinterpret_cast<uintptr_t>(C) & 15) == 0);
-  if (vec) {
-    auto kern = assign_rowstat_kernel<T, DP, ROWT, true, FUSE, NW>;
-    if (lds > 64 * 1024)
-      KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), lds, s, X, xnorm, C,
-                       cnorm, labels, mindist, n, d, k, kp, psums, pcounts);
-  } else {
-    auto kern = assign_rowstat_kernel<T, DP, ROWT, false, FUSE, NW>;
-    if (lds > 64 * 1024)
-      KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), lds, s, X, xnorm, C,
-                       cnorm, labels, mindist, n, d, k, kp, psums, pcounts);
-  }
+  const bool xal = (reinterpret_cast<uintptr_t>(X) & 15) == 0;
+  const bool vec = (d == DP) && xal && ((reinterpret_cast<uintptr_t>(C) & 15) == 0);
+  const int vw = Mfma<T>::VW;
+  const bool padvec = !vec && xal && d >= vw && d % vw == 0;
+#define KM_RS_LAUNCH(LOAD)                                                                    \
+  do {                                                                                        \
+    auto kern = assign_rowstat_kernel<T, DP, ROWT, LOAD, FUSE, NW>;                           \
+    if (lds > 64 * 1024)                                                                      \
+      KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                    \
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));  \
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), lds, s, X, xnorm, C, cnorm, \
+                       labels, mindist, n, d, k, kp, psums, pcounts);                         \
+  } while (0)
+  if (vec) KM_RS_LAUNCH(1);
+  else if (padvec) KM_RS_LAUNCH(2);
+  else KM_RS_LAUNCH(0);
+#undef KM_RS_LAUNCH
   KM_HIP_TRY(hipGetLastError());
   return 0;
 }
@@ -954,6 +970,7 @@ struct RowstatDispatch<float, FUSE> {
                  const float *cnorm, int *labels, float *mindist, int64_t n, int d,
                  int k, int num_cu, double *psums, int *pcounts, int *slots) {
     switch (rowstat_dp<float>(d)) {
+      KM_ROWSTAT_CASE(float, 8, 2);
       KM_ROWSTAT_CASE(float, 16, 2);
 #ifndef KM_ROWT_F32_32
 #define KM_ROWT_F32_32 2
@@ -971,6 +988,7 @@ struct RowstatDispatch<double, FUSE> {
                  const double *cnorm, int *labels, double *mindist, int64_t n, int d,
                  int k, int num_cu, double *psums, int *pcounts, int *slots) {
     switch (rowstat_dp<double>(d)) {
+      KM_ROWSTAT_CASE(double, 8, 4);
       KM_ROWSTAT_CASE(double, 16, 4);
       KM_ROWSTAT_CASE(double, 32, 4);
       KM_ROWSTAT_CASE(double, 64, 2);
@@ -1034,7 +1052,9 @@ static int launch_valu_fused(hipStream_t s, const T *X, const T *xnorm, const T 
     else if (vec) KM_VF_LAUNCH(DREG, Mfma<T>::VW, false);      \
     else KM_VF_LAUNCH(DREG, 1, false);                         \
   } while (0)
-  if (d <= 16) KM_VF(16);
+  if (d <= 4) KM_VF(4);
+  else if (d <= 8) KM_VF(8);
+  else if (d <= 16) KM_VF(16);
   else if (d <= 32) KM_VF(32);
   else KM_VF(64);
 #undef KM_VF_LAUNCH

@@ -181,7 +181,8 @@ def test_fused_step_equals_separate_kernels(hip, oracle, n, d, k, dtype):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
-@pytest.mark.parametrize("n,d,k", [(100000, 16, 8), (5001, 3, 2), (777, 64, 16), (3000, 33, 11), (256, 8, 1)])
+@pytest.mark.parametrize("n,d,k", [(100000, 16, 8), (5001, 3, 2), (777, 64, 16), (3000, 33, 11), (256, 8, 1),
+                                   (40000, 4, 16), (30001, 8, 7), (9000, 2, 4), (5000, 6, 3), (4000, 1, 2)])
 def test_small_shape_fused_step_is_bit_exact(hip, oracle, n, d, k, dtype):
     """k <= 16 and d <= 64: the one-pass VALU step. Labels and minimum distances are
     bit-identical to the scalar CPU loop; float32 centroids are bit-identical to the
