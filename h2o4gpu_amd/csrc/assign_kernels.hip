@@ -557,7 +557,7 @@ struct TiledCfg {
 };
 
 template <typename T, int MODE, bool VECLOAD, bool DTAIL, int BCW>
-__global__ __launch_bounds__(2 * BCW * 64, BCW == 2 ? 2 : 1) void assign_tiled_kernel(
+__global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_kernel(
     const T *__restrict__ X, const T *__restrict__ xnorm,
     const T *__restrict__ C, const T *__restrict__ cnorm,
     int *__restrict__ labels, T *__restrict__ mindist, T *__restrict__ D,
@@ -1113,7 +1113,10 @@ static int launch_tiled(hipStream_t s, const T *X, const T *xnorm, const T *C,
                         int64_t ldn, int d, int k) {
   // Measured at 2M x 256, k = 1024 and 500k x 784, k = 4096: two 4-wave workgroups per CU
   // (BCW = 2) beat one 8-wave workgroup with the wider centroid block (BCW = 4) by 5-10 %,
-  // so the narrow form is used throughout.
+  // so the 128-centroid form is used for large models. Up to 64 centroids a 64-wide block
+  // (two wavefronts) halves the matrix work spent on padding; such shapes are bandwidth-bound.
+  if (k <= 64)
+    return launch_tiled_bcw<T, MODE, 1>(s, X, xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k);
   return launch_tiled_bcw<T, MODE, 2>(s, X, xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k);
 }
 

@@ -257,7 +257,7 @@ struct Engine : h2o4gpu_kmeans_handle {
     if (fs > slots) slots = fs;
     KM_TRY(dalloc(&psums, (size_t)slots * kd));
     KM_TRY(dalloc(&pcounts, (size_t)slots * k));
-    use_buckets = bucketed_update_applies(plan.k_chunks, k);
+    use_buckets = bucketed_update_applies(plan.k_chunks, k, d);
     if (use_buckets) {
       KM_TRY(dalloc(&order, n));
       KM_TRY(dalloc(&order_label, n));

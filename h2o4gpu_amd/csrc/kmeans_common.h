@@ -108,7 +108,7 @@ int launch_accumulate(hipStream_t s, const UpdatePlan &p, const T *X,
 // label (order / order_label: [n] int32 each, offsets / cursor: [k] int32) and every
 // bucket is summed into gsum [k][d] double; counts receives the bucket sizes. The
 // result is consumed by launch_finalize with slots = 1.
-bool bucketed_update_applies(int k_chunks, int k);
+bool bucketed_update_applies(int k_chunks, int k, int d);
 template <typename T>
 int launch_bucketed_accumulate(hipStream_t s, const T *X, const int *labels, int *order,
                                int *order_label, int *offsets, int *cursor, int *total,

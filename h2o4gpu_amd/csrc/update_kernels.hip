@@ -78,7 +78,9 @@ __global__ __launch_bounds__(WG) void row_norms_coalesced_kernel(
 template <typename T>
 int launch_row_norms(hipStream_t s, const T *X, T *out, int64_t n, int d) {
   if (n <= 0) return 0;
-  if (d >= 8 && n * (int64_t)d >= 65536) {
+  // (a thread per row is enough for a handful of short rows; long rows always go
+  // through the cooperative kernel, a single thread would walk them serially)
+  if (d >= 8 && (n * (int64_t)d >= 65536 || d >= 64)) {
     if (d <= 16) {
       constexpr int LPR = 16;
       hipLaunchKernelGGL((row_norms_coalesced_kernel<T, LPR>),
@@ -494,7 +496,10 @@ __global__ __launch_bounds__(WG) void segment_sum_kernel(
 }
 
 size_t bucket_lds_bytes(int k) { return (size_t)2 * k * sizeof(int); }
-bool bucketed_update_applies(int k_chunks, int k) {
+bool bucketed_update_applies(int k_chunks, int k, int d) {
+  // (measured: with a handful of centroids the scatter's few cursors serialise and the
+  // LDS kernel stays ahead, so bucketing is not used while the sums fit LDS)
+  (void)d;
   return k_chunks > 1 && bucket_lds_bytes(k) <= 128 * 1024;
 }
 
@@ -695,7 +700,7 @@ int launch_post_update(hipStream_t s, const T *c_new, T *cnorm,
                        int d, int k) {
   // large centroid sets: norms by the coalesced row-norm kernel (same summation order),
   // this kernel then only adds up the shift partials
-  const bool separate_norms = (int64_t)k * d >= 65536 && d >= 8;
+  const bool separate_norms = d >= 8 && ((int64_t)k * d >= 65536 || d >= 64);
   const int blocks = separate_norms ? 1 : (k + WG - 1) / WG + 1;
   hipLaunchKernelGGL((post_update_kernel<T>), dim3(blocks), dim3(WG), 0, s, c_new,
                      separate_norms ? (T *)nullptr : cnorm, shift_partials, n_shift_partials,
