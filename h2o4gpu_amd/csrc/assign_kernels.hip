@@ -259,7 +259,7 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
     const T *__restrict__ X, const T *__restrict__ xnorm,
     const T *__restrict__ C, const T *__restrict__ cnorm,
     int *__restrict__ labels, T *__restrict__ mindist, int64_t n, int d, int k,
-    int kp, double *__restrict__ psums, int *__restrict__ pcounts) {
+    int kp, double *__restrict__ psums, int *__restrict__ pcounts, int c_off, int merge) {
   constexpr int TPB = NW * 64;
   typedef Mfma<T> M;
   constexpr int MT = M::MT, KL = M::KL, NACC = M::NACC, VW = M::VW;
@@ -504,8 +504,15 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
       }
       const int64_t row = wrow0 + rt * MT + r;
       if (g == 0 && row < n) {
-        labels[row] = bidx[rt];
-        if (mindist) mindist[row] = best[rt];
+        // A model too large for LDS is swept in chunks of centroids, one launch each:
+        // C and cnorm then point at the chunk, c_off is its first centroid, and from the
+        // second chunk on (merge) the row's result so far is read back and kept unless
+        // this chunk is strictly closer (earlier chunks hold the lower indices).
+        T bv = best[rt];
+        int bi = bidx[rt] < 0 ? -1 : bidx[rt] + c_off;
+        if (merge) argmin_merge(bv, bi, mindist[row], labels[row]);
+        labels[row] = bi;
+        if (mindist) mindist[row] = bv;
       }
       if (FUSE && row < n && bidx[rt] >= 0) {
         double *srow = sums + (size_t)bidx[rt] * SD + g * DCH;
@@ -856,15 +863,34 @@ static size_t rowstat_lds(int d, int k) {
   return ((size_t)kp * rowstat_dp<T>(d) + kp) * sizeof(T);
 }
 
+static const size_t ROWSTAT_LDS_MAX = 96 * 1024;
+// centroids per chunk of a chunked row-stationary sweep (a multiple of the MFMA tile)
+template <typename T>
+static int rowstat_chunk(int d, int k) {
+  if (rowstat_lds<T>(d, k) <= ROWSTAT_LDS_MAX) return k;
+  const int MT = Mfma<T>::MT;
+  const size_t per = ((size_t)rowstat_dp<T>(d) + 1) * sizeof(T);
+  const int kc_max = (int)(ROWSTAT_LDS_MAX / per) / MT * MT;
+  const int chunks = (k + kc_max - 1) / kc_max;
+  const int kc = ((k + chunks - 1) / chunks + MT - 1) / MT * MT;  // balanced
+  return kc;
+}
+
 template <typename T>
 int pick_assign_variant(int requested, int64_t n, int d, int k) {
-  const bool rowstat_ok = rowstat_dp<T>(d) != 0 && rowstat_lds<T>(d, k) <= 96 * 1024;
-  if (requested == ASSIGN_ROWSTAT) return rowstat_ok ? ASSIGN_ROWSTAT : -1;
+  const int dp = rowstat_dp<T>(d);
+  const bool rowstat_ok = dp != 0 && rowstat_lds<T>(d, k) <= ROWSTAT_LDS_MAX;
+  // any model can be swept in LDS-sized chunks of centroids (one launch per chunk)
+  if (requested == ASSIGN_ROWSTAT) return dp != 0 ? ASSIGN_ROWSTAT : -1;
   if (requested == ASSIGN_VALU || requested == ASSIGN_TILED) return requested;
   // the reference switches to its hand-written small kernel at k<=16 && d<=64
   // (kmeans_labels.cu:140,207); same boundary here
   if (k <= 16 && d <= 64) return ASSIGN_VALU;
   if (rowstat_ok) return ASSIGN_ROWSTAT;
+  // Short rows with a large model: the tiled kernel's d-loop has one or two stages and
+  // cannot hide its loads; chunked row-stationary sweeps re-read X once per chunk, which
+  // is cheap next to the matrix work of 700+ centroids.
+  if (dp != 0 && dp * (int)sizeof(T) <= 256) return ASSIGN_ROWSTAT;
   return ASSIGN_TILED;
 }
 
@@ -910,7 +936,7 @@ template <typename T, int DP, int ROWT, bool FUSE, int NW>
 static int launch_rowstat_nw(hipStream_t s, const T *X, const T *xnorm, const T *C,
                              const T *cnorm, int *labels, T *mindist, int64_t n, int d,
                              int k, int num_cu, double *psums, int *pcounts, int *slots,
-                             size_t lds) {
+                             size_t lds, int c_off, int merge) {
   const int MT = Mfma<T>::MT;
   const int kp = (k + MT - 1) / MT * MT;
   const int rows_per_wg = NW * ROWT * MT;
@@ -930,7 +956,7 @@ static int launch_rowstat_nw(hipStream_t s, const T *X, const T *xnorm, const T 
       KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                    \
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));  \
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), lds, s, X, xnorm, C, cnorm, \
-                       labels, mindist, n, d, k, kp, psums, pcounts);                         \
+                       labels, mindist, n, d, k, kp, psums, pcounts, c_off, merge);           \
   } while (0)
   if (vec) KM_RS_LAUNCH(1);
   else if (padvec) KM_RS_LAUNCH(2);
@@ -944,18 +970,18 @@ template <typename T, int DP, int ROWT, bool FUSE>
 static int launch_rowstat_dp(hipStream_t s, const T *X, const T *xnorm,
                              const T *C, const T *cnorm, int *labels,
                              T *mindist, int64_t n, int d, int k, int num_cu,
-                             double *psums, int *pcounts, int *slots) {
+                             double *psums, int *pcounts, int *slots, int c_off, int merge) {
   const size_t lds = FUSE ? rowstat_fused_lds<T>(d, k) : rowstat_lds<T>(d, k);
   if (rowstat_two_per_cu(lds))
     return launch_rowstat_nw<T, DP, ROWT, FUSE, 4>(s, X, xnorm, C, cnorm, labels, mindist, n, d,
-                                                   k, num_cu, psums, pcounts, slots, lds);
+                                                   k, num_cu, psums, pcounts, slots, lds, c_off, merge);
   // one workgroup per CU: as many wavefronts as the register budget allows
   if constexpr (sizeof(T) == 4 && DP <= 32)
     return launch_rowstat_nw<T, DP, ROWT, FUSE, 16>(s, X, xnorm, C, cnorm, labels, mindist, n, d,
-                                                    k, num_cu, psums, pcounts, slots, lds);
+                                                    k, num_cu, psums, pcounts, slots, lds, c_off, merge);
   else
     return launch_rowstat_nw<T, DP, ROWT, FUSE, 8>(s, X, xnorm, C, cnorm, labels, mindist, n, d,
-                                                   k, num_cu, psums, pcounts, slots, lds);
+                                                   k, num_cu, psums, pcounts, slots, lds, c_off, merge);
 }
 
 template <typename T, bool FUSE>
@@ -963,12 +989,13 @@ struct RowstatDispatch;
 #define KM_ROWSTAT_CASE(T, DP, ROWT)                                                  \
   case DP:                                                                            \
     return launch_rowstat_dp<T, DP, ROWT, FUSE>(s, X, xnorm, C, cnorm, labels, mindist, \
-                                                n, d, k, num_cu, psums, pcounts, slots)
+                                                n, d, k, num_cu, psums, pcounts, slots, c_off, merge)
 template <bool FUSE>
 struct RowstatDispatch<float, FUSE> {
   static int run(hipStream_t s, const float *X, const float *xnorm, const float *C,
                  const float *cnorm, int *labels, float *mindist, int64_t n, int d,
-                 int k, int num_cu, double *psums, int *pcounts, int *slots) {
+                 int k, int num_cu, double *psums, int *pcounts, int *slots, int c_off = 0,
+                 int merge = 0) {
     switch (rowstat_dp<float>(d)) {
       KM_ROWSTAT_CASE(float, 8, 2);
       KM_ROWSTAT_CASE(float, 16, 2);
@@ -986,7 +1013,8 @@ template <bool FUSE>
 struct RowstatDispatch<double, FUSE> {
   static int run(hipStream_t s, const double *X, const double *xnorm, const double *C,
                  const double *cnorm, int *labels, double *mindist, int64_t n, int d,
-                 int k, int num_cu, double *psums, int *pcounts, int *slots) {
+                 int k, int num_cu, double *psums, int *pcounts, int *slots, int c_off = 0,
+                 int merge = 0) {
     switch (rowstat_dp<double>(d)) {
       KM_ROWSTAT_CASE(double, 8, 4);
       KM_ROWSTAT_CASE(double, 16, 4);
@@ -1132,9 +1160,18 @@ int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
   switch (v) {
     case ASSIGN_VALU:
       return launch_valu<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k);
-    case ASSIGN_ROWSTAT:
-      return RowstatDispatch<T, false>::run(s, X, xnorm, C, cnorm, labels, mindist, n, d, k,
-                                            num_cu, nullptr, nullptr, nullptr);
+    case ASSIGN_ROWSTAT: {
+      const int kc = rowstat_chunk<T>(d, k);
+      if (kc < k && !mindist) {  // merging chunks needs the running minimum in memory
+        if (used) *used = ASSIGN_TILED;
+        return launch_tiled<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k);
+      }
+      for (int c0 = 0; c0 < k; c0 += kc)
+        KM_TRY((RowstatDispatch<T, false>::run(s, X, xnorm, C + (size_t)c0 * d, cnorm + c0, labels,
+                                               mindist, n, d, min(kc, k - c0), num_cu, nullptr,
+                                               nullptr, nullptr, c0, c0 > 0)));
+      return 0;
+    }
     case ASSIGN_TILED:
       return launch_tiled<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k);
   }
