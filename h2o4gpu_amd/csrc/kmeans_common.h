@@ -104,7 +104,7 @@ template <typename T>
 int launch_accumulate(hipStream_t s, const UpdatePlan &p, const T *X,
                       const int *labels, double *psums, int *pcounts, int64_t n,
                       int d, int k);
-// Pass 1 for shapes whose sums do not fit LDS (plan.k_chunks > 1): rows are bucketed by
+// Pass 1 for shapes whose sums need many LDS chunks: rows are bucketed by
 // label (order / order_label: [n] int32 each, offsets / cursor: [k] int32) and every
 // bucket is summed into gsum [k][d] double; counts receives the bucket sizes. The
 // result is consumed by launch_finalize with slots = 1.
