@@ -62,7 +62,7 @@ def test_assign_matches_oracle(hip, oracle, n, d, k, variant, dtype):
 @pytest.mark.parametrize("buckets", [1, 0])
 @pytest.mark.parametrize("n,d,k", [(5000, 32, 256), (3000, 16, 8), (2000, 7, 5), (4000, 256, 300),
                                    (1000, 784, 130), (70000, 64, 64), (300, 3, 300), (9000, 1100, 70),
-                                   (5000, 130, 90), (6000, 51, 700)])
+                                   (5000, 130, 90), (6000, 51, 700), (3000, 256, 700), (9000, 40, 5000)])
 def test_update_matches_oracle(hip, oracle, n, d, k, buckets, dtype):
     X = blobs(n, d, k, dtype, seed=7 * n + k)
     C = np.ascontiguousarray(X[RNG.choice(n, size=k, replace=False)])
