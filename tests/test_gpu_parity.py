@@ -359,3 +359,46 @@ def test_more_than_two_to_the_31_elements(hip, oracle):
     for c in (0, k - 1):
         m = X[labels == c].astype(np.float64).mean(0)
         assert np.allclose(C1[c], m, rtol=1e-5, atol=1e-4)
+
+
+def _random_shapes(count, seed):
+    """Seeded shapes spread over every dispatch rule: feature counts around the vector
+    and MFMA-slice boundaries, models from one centroid to several LDS chunks."""
+    rng = np.random.default_rng(seed)
+    d_pool = [1, 2, 3, 4, 5, 7, 8, 9, 12, 15, 16, 17, 20, 24, 31, 32, 33, 40, 48, 63, 64, 65, 72, 96,
+              100, 127, 128, 129, 160, 200, 256, 257, 300, 384, 520]
+    shapes = []
+    for _ in range(count):
+        d = int(rng.choice(d_pool))
+        k = int(rng.choice([1, 2, 3, 8, 16, 17, 31, 32, 33, 50, 64, 65, 100, 128, 129, 200, 256, 300,
+                            500, 700, 1000, 1500, 2500]))
+        n = int(rng.integers(max(k, 2), 12000))
+        shapes.append((n, d, k))
+    return shapes
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_one_step_on_random_shapes(hip, oracle, dtype):
+    """One Lloyd step (the kernels the dispatcher picks by itself) on 60 seeded shapes:
+    labels against the oracle up to excused near-ties, counts and new centroids against
+    the oracle update of the engine's own labels."""
+    tol = 1e-5 if dtype == np.float32 else 1e-12
+    seen = {}
+    for (n, d, k) in _random_shapes(60, 2024):
+        X = blobs(n, d, max(k, 2), dtype, seed=n + 3 * d + 7 * k)
+        C0 = np.ascontiguousarray(X[np.random.default_rng(n).choice(n, size=k, replace=False)])
+        with hip.Handle(n, d, k, dtype) as h:
+            h.set_data(X)
+            h.set_centroids(C0)
+            variant = h.assign_variant()
+            h.iterate(1)
+            labels, counts, C1 = h.labels(), h.counts(), h.centroids()
+        where = "n=%d d=%d k=%d %s %s" % (n, d, k, variant, np.dtype(dtype).name)
+        rep = label_report(oracle, X, C0, labels, oracle.assign(X, C0, threads=4))
+        wC, wcounts = oracle.update(X, labels, C0)
+        assert np.array_equal(counts, wcounts), where
+        assert np.allclose(C1, wC, rtol=tol, atol=tol * np.abs(wC).max()), where
+        seen[variant] = seen.get(variant, 0) + 1
+        if rep["mismatch"]:
+            print("random shape %s: %s" % (where, rep))
+    assert set(seen) == {"valu", "mfma_rowstat", "mfma_tiled"}, seen
