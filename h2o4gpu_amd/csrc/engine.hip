@@ -209,6 +209,8 @@ struct Engine : h2o4gpu_kmeans_handle {
   bool use_buckets = false;
   double *sum_partials = nullptr;  // [sum_partials_needed() + 1]
   double *kpp_bsums = nullptr;
+  int *kpp_rows = nullptr;  // [k] rows chosen so far by k-means++
+  T *kpp_dcc = nullptr;     // [k] distances newest centre -> earlier centres
   bool have_data = false, have_centroids = false, have_mindist = false;
 
   template <typename U>
@@ -269,6 +271,8 @@ struct Engine : h2o4gpu_kmeans_handle {
     KM_TRY(dalloc(&shift2, 1));
     KM_TRY(dalloc(&sum_partials, sum_partials_needed() + 1));
     KM_TRY(dalloc(&kpp_bsums, (n + KPP_BLOCK - 1) / KPP_BLOCK + 1));
+    KM_TRY(dalloc(&kpp_rows, (size_t)k + 1));
+    KM_TRY(dalloc(&kpp_dcc, (size_t)k + 1));
     // the reference's label vector starts zeroed (thrust::device_vector<int>)
     KM_HIP_TRY(hipMemsetAsync(labels, 0, (size_t)n * sizeof(int), stream));
     KM_HIP_TRY(hipMemsetAsync(counts, 0, (size_t)k * sizeof(int), stream));
@@ -288,7 +292,7 @@ struct Engine : h2o4gpu_kmeans_handle {
     if (own_X && X) (void)hipFree(X);
     void *ptrs[] = {xnorm,  C[0],    C[1],           cnorm,  labels,       mindist,
                     counts, psums,   pcounts,        shift_partials, shift2,
-                    sum_partials, kpp_bsums, order, order_label, bucket_offsets,
+                    sum_partials, kpp_bsums, kpp_rows, kpp_dcc, order, order_label, bucket_offsets,
                     bucket_cursor, bucket_counts};
     for (void *p : ptrs)
       if (p) (void)hipFree(p);
@@ -387,8 +391,8 @@ struct Engine : h2o4gpu_kmeans_handle {
     idx[0] = first(gen);
     for (int c = 1; c <= k; c++) {
       PROFILED("min_dist_update",
-               launch_min_dist_update<T>(stream, X, xnorm, idx[c - 1], mindist,
-                                         kpp_bsums, n, d, c == 1));
+               launch_min_dist_update<T>(stream, X, xnorm, idx[c - 1], mindist, labels,
+                                         kpp_rows, kpp_dcc, c - 1, kpp_bsums, n, d));
       if (c == k) break;
       KM_HIP_TRY(hipMemcpyAsync(bs.data(), kpp_bsums, (size_t)nb * sizeof(double),
                                 hipMemcpyDeviceToHost, stream));

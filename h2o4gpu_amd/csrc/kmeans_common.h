@@ -139,15 +139,17 @@ int launch_sum(hipStream_t s, const T *v, int64_t n, double *partials,
                int n_partials, double *out);
 int sum_partials_needed();
 
-// k-means++ seeding: mind[i] = min(mind[i], |xx_i + cc - 2 x_i.c|) against one
-// centre (row `centre_row` of X; init != 0 overwrites instead of taking the
-// min), then bsums[b] = sum of mind over rows [b*KPP_BLOCK, (b+1)*KPP_BLOCK) in
-// double with a fixed tree.
+// k-means++ seeding, round t (t = 0 first): mind[i] = min(mind[i], |xx_i + cc - 2 x_i.c|)
+// against the t-th chosen centre (row `centre_row` of X; t == 0 overwrites), then
+// bsums[b] = sum of mind over rows [b*KPP_BLOCK, (b+1)*KPP_BLOCK) in double with a fixed
+// tree. nearest [n] keeps the index of the closest chosen centre so far, rows [k] the
+// chosen rows and dcc [k] the distances from the newest centre to the earlier ones: rows
+// that the triangle inequality rules out are not read.
 static const int KPP_BLOCK = 1024;
 template <typename T>
-int launch_min_dist_update(hipStream_t s, const T *X, const T *xnorm,
-                           int64_t centre_row, T *mind, double *bsums, int64_t n,
-                           int d, int init);
+int launch_min_dist_update(hipStream_t s, const T *X, const T *xnorm, int64_t centre_row,
+                           T *mind, int *nearest, int *rows, T *dcc, int t, double *bsums,
+                           int64_t n, int d);
 
 // Copy rows idx[0..k-1] of X into C ([k][d]).
 template <typename T>
