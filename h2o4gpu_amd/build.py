@@ -11,7 +11,7 @@ SOURCES = ["engine.hip", "assign_kernels.hip", "update_kernels.hip", "seed_kerne
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
-    "-munsafe-fp-atomics",
+    "-munsafe-fp-atomics", "-pthread",
     # packed-FP32 VALU forms stay off for every kernel of this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-result",
@@ -45,7 +45,7 @@ def build(verbose=False, jobs=4):
             print("\n".join(lines))
     if failed:
         raise RuntimeError("hipcc failed")
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-pthread", "-o", LIB_PATH] + objs
     subprocess.check_call(cmd)
     return LIB_PATH
 

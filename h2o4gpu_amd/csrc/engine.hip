@@ -15,9 +15,11 @@
 #include <ctime>
 #include <limits>
 #include <map>
+#include <mutex>
 #include <numeric>
 #include <random>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "kmeans_common.h"
@@ -180,6 +182,85 @@ struct h2o4gpu_kmeans_handle {
 
 namespace kmhip {
 
+// ---------------------------------------------------------------------------
+// Host-to-device upload of a large pageable buffer through two pinned staging
+// buffers: a few host threads copy chunk i+1 into one buffer while the DMA engine
+// drains chunk i from the other. The entry points receive ordinary malloc'ed /
+// numpy memory (src/gpu/kmeans/kmeans_h2o4gpu.h:24-42 copies it on the host first
+// and then uploads it from pageable memory in one call).
+// The buffers are allocated once per process and device and kept; uploads of
+// different handles take turns.
+// ---------------------------------------------------------------------------
+struct StagingPool {
+  static constexpr size_t CHUNK = 32u << 20;
+  static constexpr int MAX_DEV = 64;
+  std::mutex mu;
+  void *buf[MAX_DEV][2] = {};
+  hipEvent_t done[MAX_DEV][2] = {};
+  bool broken[MAX_DEV] = {};
+
+  static void parallel_copy(char *dst, const char *src, size_t bytes, int threads) {
+    if (threads <= 1 || bytes < (4u << 20)) {
+      memcpy(dst, src, bytes);
+      return;
+    }
+    std::vector<std::thread> pool;
+    const size_t per = ((bytes + threads - 1) / threads + 4095) & ~(size_t)4095;
+    for (int t = 1; t < threads; t++) {
+      const size_t lo = per * t;
+      if (lo >= bytes) break;
+      const size_t len = std::min(per, bytes - lo);
+      pool.emplace_back([=] { memcpy(dst + lo, src + lo, len); });
+    }
+    memcpy(dst, src, std::min(per, bytes));
+    for (auto &th : pool) th.join();
+  }
+
+  // Returns 0 on success; a positive value means "staging unavailable, use a plain copy".
+  int upload(int dev, hipStream_t stream, void *dst, const void *src, size_t bytes) {
+    if (dev < 0 || dev >= MAX_DEV || bytes < 4 * CHUNK) return 1;
+    std::lock_guard<std::mutex> lock(mu);
+    if (broken[dev]) return 1;
+    if (!buf[dev][0]) {
+      for (int i = 0; i < 2; i++) {
+        if (hipHostMalloc(&buf[dev][i], CHUNK, hipHostMallocDefault) != hipSuccess ||
+            hipEventCreateWithFlags(&done[dev][i], hipEventDisableTiming) != hipSuccess) {
+          (void)hipGetLastError();
+          broken[dev] = true;
+          return 1;
+        }
+      }
+    }
+    unsigned hw = std::thread::hardware_concurrency();
+    const char *env = getenv("H2O4GPU_KMEANS_UPLOAD_THREADS");
+    int threads = env ? atoi(env) : (int)std::min(8u, hw ? hw : 1u);
+    if (threads < 1) threads = 1;
+    size_t off = 0;
+    for (int i = 0; off < bytes; i ^= 1) {
+      const size_t len = std::min(CHUNK, bytes - off);
+      KM_HIP_TRY(hipEventSynchronize(done[dev][i]));  // the DMA that last read this buffer
+      parallel_copy(static_cast<char *>(buf[dev][i]), static_cast<const char *>(src) + off, len,
+                    threads);
+      KM_HIP_TRY(hipMemcpyAsync(static_cast<char *>(dst) + off, buf[dev][i], len,
+                                hipMemcpyHostToDevice, stream));
+      KM_HIP_TRY(hipEventRecord(done[dev][i], stream));
+      off += len;
+    }
+    // both buffers must be drained before the next caller (or this one) refills them
+    KM_HIP_TRY(hipEventSynchronize(done[dev][0]));
+    KM_HIP_TRY(hipEventSynchronize(done[dev][1]));
+    return 0;
+  }
+};
+static StagingPool g_staging;
+
+static int upload_rows(int dev, hipStream_t stream, void *dst, const void *src, size_t bytes) {
+  const int rc = g_staging.upload(dev, stream, dst, src, bytes);
+  if (rc <= 0) return rc;
+  KM_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, stream));
+  return 0;
+}
+
 #define PROFILED(name, call)   \
   do {                         \
     prof_begin(name);          \
@@ -309,7 +390,7 @@ struct Engine : h2o4gpu_kmeans_handle {
       KM_TRY(dalloc(&X, (size_t)n * d));
       own_X = true;
     }
-    KM_HIP_TRY(hipMemcpyAsync(X, hX, (size_t)n * d * sizeof(T), hipMemcpyHostToDevice, stream));
+    KM_TRY(upload_rows(dev, stream, X, hX, (size_t)n * d * sizeof(T)));
     PROFILED("row_norms", launch_row_norms<T>(stream, X, xnorm, n, d));
     KM_HIP_TRY(hipStreamSynchronize(stream));
     have_data = true;
@@ -581,7 +662,7 @@ struct Engine : h2o4gpu_kmeans_handle {
     return rc;
   }
   int run_predict(size_t rows, const void *hX, int *out, T *dX, T *dxn, int *dl) {
-    KM_HIP_TRY(hipMemcpyAsync(dX, hX, rows * d * sizeof(T), hipMemcpyHostToDevice, stream));
+    KM_TRY(upload_rows(dev, stream, dX, hX, rows * d * sizeof(T)));
     PROFILED("row_norms", launch_row_norms<T>(stream, dX, dxn, (int64_t)rows, d));
     PROFILED("assign", launch_assign<T>(stream, opt_assign, dX, dxn, C[cur], cnorm, dl,
                                         (T *)nullptr, (int64_t)rows, d, k, num_cu, &last_variant));
