@@ -216,21 +216,26 @@ struct StagingPool {
     for (auto &th : pool) th.join();
   }
 
+  // Pinned buffers and events of a device, created on first use (caller holds mu).
+  bool ensure(int dev) {
+    if (broken[dev]) return false;
+    if (buf[dev][1] && done[dev][1]) return true;
+    for (int i = 0; i < 2; i++) {
+      if (hipHostMalloc(&buf[dev][i], CHUNK, hipHostMallocDefault) != hipSuccess ||
+          hipEventCreateWithFlags(&done[dev][i], hipEventDisableTiming) != hipSuccess) {
+        (void)hipGetLastError();
+        broken[dev] = true;
+        return false;
+      }
+    }
+    return true;
+  }
+
   // Returns 0 on success; a positive value means "staging unavailable, use a plain copy".
   int upload(int dev, hipStream_t stream, void *dst, const void *src, size_t bytes) {
     if (dev < 0 || dev >= MAX_DEV || bytes < 4 * CHUNK) return 1;
     std::lock_guard<std::mutex> lock(mu);
-    if (broken[dev]) return 1;
-    if (!buf[dev][0]) {
-      for (int i = 0; i < 2; i++) {
-        if (hipHostMalloc(&buf[dev][i], CHUNK, hipHostMallocDefault) != hipSuccess ||
-            hipEventCreateWithFlags(&done[dev][i], hipEventDisableTiming) != hipSuccess) {
-          (void)hipGetLastError();
-          broken[dev] = true;
-          return 1;
-        }
-      }
-    }
+    if (!ensure(dev)) return 1;
     unsigned hw = std::thread::hardware_concurrency();
     const char *env = getenv("H2O4GPU_KMEANS_UPLOAD_THREADS");
     int threads = env ? atoi(env) : (int)std::min(8u, hw ? hw : 1u);
@@ -251,8 +256,43 @@ struct StagingPool {
     KM_HIP_TRY(hipEventSynchronize(done[dev][1]));
     return 0;
   }
+
+  // The way back: the DMA engine fills one buffer while host threads copy the other out.
+  int download(int dev, hipStream_t stream, void *dst, const void *src, size_t bytes) {
+    if (dev < 0 || dev >= MAX_DEV || bytes < 4 * CHUNK) return 1;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ensure(dev)) return 1;
+    unsigned hw = std::thread::hardware_concurrency();
+    const char *env = getenv("H2O4GPU_KMEANS_UPLOAD_THREADS");
+    int threads = env ? atoi(env) : (int)std::min(8u, hw ? hw : 1u);
+    if (threads < 1) threads = 1;
+    const size_t chunks = (bytes + CHUNK - 1) / CHUNK;
+    for (size_t c = 0; c <= chunks; c++) {
+      const int b = (int)(c & 1);
+      if (c < chunks) {
+        const size_t off = c * CHUNK, len = std::min(CHUNK, bytes - off);
+        KM_HIP_TRY(hipMemcpyAsync(buf[dev][b], static_cast<const char *>(src) + off, len,
+                                  hipMemcpyDeviceToHost, stream));
+        KM_HIP_TRY(hipEventRecord(done[dev][b], stream));
+      }
+      if (c >= 1) {  // chunk c-1 sits in the other buffer
+        const size_t off = (c - 1) * CHUNK, len = std::min(CHUNK, bytes - off);
+        KM_HIP_TRY(hipEventSynchronize(done[dev][b ^ 1]));
+        parallel_copy(static_cast<char *>(dst) + off, static_cast<const char *>(buf[dev][b ^ 1]), len,
+                      threads);
+      }
+    }
+    return 0;
+  }
 };
 static StagingPool g_staging;
+
+static int download_rows(int dev, hipStream_t stream, void *dst, const void *src, size_t bytes) {
+  const int rc = g_staging.download(dev, stream, dst, src, bytes);
+  if (rc <= 0) return rc;
+  KM_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, stream));
+  return 0;
+}
 
 static int upload_rows(int dev, hipStream_t stream, void *dst, const void *src, size_t bytes) {
   const int rc = g_staging.upload(dev, stream, dst, src, bytes);
@@ -699,13 +739,16 @@ struct Engine : h2o4gpu_kmeans_handle {
   int run_transform_batch(size_t lo, size_t cur_rows, size_t rows, const void *hX, void *hD,
                           T *dX, T *dxn, T *dD) {
     const T *src = static_cast<const T *>(hX) + lo * d;
-    KM_HIP_TRY(hipMemcpyAsync(dX, src, cur_rows * d * sizeof(T), hipMemcpyHostToDevice, stream));
+    KM_TRY(upload_rows(dev, stream, dX, src, cur_rows * d * sizeof(T)));
     PROFILED("row_norms", launch_row_norms<T>(stream, dX, dxn, (int64_t)cur_rows, d));
     PROFILED("transform", launch_transform<T>(stream, dX, dxn, C[cur], cnorm, dD,
                                               (int64_t)cur_rows, (int64_t)cur_rows, d, k, num_cu));
     T *dst = static_cast<T *>(hD) + lo;
-    KM_HIP_TRY(hipMemcpy2DAsync(dst, rows * sizeof(T), dD, cur_rows * sizeof(T),
-                                cur_rows * sizeof(T), (size_t)k, hipMemcpyDeviceToHost, stream));
+    if (cur_rows == rows)  // a single batch is one contiguous [k][rows] block
+      KM_TRY(download_rows(dev, stream, dst, dD, (size_t)k * rows * sizeof(T)));
+    else
+      KM_HIP_TRY(hipMemcpy2DAsync(dst, rows * sizeof(T), dD, cur_rows * sizeof(T),
+                                  cur_rows * sizeof(T), (size_t)k, hipMemcpyDeviceToHost, stream));
     KM_HIP_TRY(hipStreamSynchronize(stream));
     return 0;
   }
