@@ -231,3 +231,37 @@ def test_estimator_restarts_and_score(oracle):
     Xn, _ = blobs(1500, 6, 8, np.float32, 22)
     d2 = ((Xn[:, None, :].astype(np.float64) - multi.cluster_centers_[None].astype(np.float64)) ** 2).sum(-1)
     assert abs(multi.score(Xn) + d2.min(1).sum()) <= 1e-5 * d2.min(1).sum()
+
+
+def test_concurrent_fits_from_two_threads(shim):
+    """The entry points are re-entrant (the reference keeps per-device globals and is not,
+    kmeans_labels.cu:11-49): two threads fitting different data at the same time get the
+    results, and the last-fit record, of their own call."""
+    import threading
+    jobs = []
+    for seed, (n, d, k) in enumerate([(40000, 24, 9), (25000, 40, 14)]):
+        X, centers = blobs(n, d, k, np.float32, 50 + seed)
+        C0 = (centers + 0.3).astype(np.float32)
+        rc, C, L = fit(shim, X, k, 6, 2, C0=C0)
+        assert rc == 0
+        jobs.append((X, C0, k, C, L, shim.last_fit_info()))
+    out = [None, None]
+
+    def work(i):
+        X, C0, k = jobs[i][:3]
+        res = []
+        for _ in range(5):
+            rc, C, L = fit(shim, X, k, 6, 2, C0=C0)
+            res.append((rc, C, L, shim.last_fit_info()))
+        out[i] = res
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for i in range(2):
+        _, _, _, wantC, wantL, want_info = jobs[i]
+        for rc, C, L, info in out[i]:
+            assert rc == 0 and np.array_equal(C, wantC) and np.array_equal(L, wantL)
+            assert info == want_info
