@@ -410,6 +410,12 @@ struct Engine : h2o4gpu_kmeans_handle {
     (void)hipSetDevice(dev);
     if (stream) (void)hipStreamSynchronize(stream);
     prof_free();
+    if (host_shift) (void)hipHostFree(host_shift);
+    host_shift = nullptr;
+    for (auto &e : shift_ready) {
+      if (e) (void)hipEventDestroy(e);
+      e = nullptr;
+    }
     if (own_X && X) (void)hipFree(X);
     void *ptrs[] = {xnorm,  C[0],    C[1],           cnorm,  labels,       mindist,
                     counts, psums,   pcounts,        shift_partials, shift2,
@@ -623,31 +629,77 @@ struct Engine : h2o4gpu_kmeans_handle {
     if (!have_data || !have_centroids) return H2O4GPU_KMEANS_ESTATE;
     maybe_install_signal_handlers();
     int updates = 0;
-    for (int i = 0; i < max_iterations; i++) {
-      log_msg(verbose, LOG_VERBOSE, "KMeans - Iteration %d/%d", i, max_iterations);
-      KM_TRY(step_async());
-      updates++;
-      bool done = false;
-      if (threshold > 0) {
-        double s2 = 0;
-        KM_TRY(read_shift2(&s2));
-        if (s2 < threshold) {
-          log_msg(verbose, LOG_INFO, "Threshold triggered. Terminating early.");
+    if (threshold > 0 && max_iterations > 0) {
+      KM_TRY(fit_with_threshold(max_iterations, threshold, &updates));
+    } else {
+      for (int i = 0; i < max_iterations; i++) {
+        log_msg(verbose, LOG_VERBOSE, "KMeans - Iteration %d/%d", i, max_iterations);
+        KM_TRY(step_async());
+        updates++;
+        bool done = false;
+        if (g_stop_flag) {
+          fprintf(stderr, "Signal caught. Terminated early.\n");
+          g_stop_flag = 0;
           done = true;
         }
+        if (done || i == max_iterations - 1) {
+          KM_TRY(assign());  // final relabel with the final centroids
+          break;
+        }
       }
+    }
+    KM_HIP_TRY(hipStreamSynchronize(stream));
+    if (iters) *iters = updates;
+    return 0;
+  }
+
+  // The loop with a convergence test (kmeans_impl.h:189-232: stop after the update whose
+  // squared shift is below the threshold, then relabel with the final centroids). The
+  // scalar of iteration i travels to pinned host memory while iteration i+1 is already
+  // queued, so the device never waits for the host. When iteration i turns out to be the
+  // last one, the queued iteration's assignment pass IS the final relabel (it ran with the
+  // centroids of update i); only its centroid update is dropped: the buffers are flipped
+  // back and the centroid norms recomputed.
+  T *host_shift = nullptr;            // [2] pinned
+  hipEvent_t shift_ready[2] = {nullptr, nullptr};
+  int fit_with_threshold(int max_iterations, double threshold, int *updates_out) {
+    if (!host_shift) {
+      KM_HIP_TRY(hipHostMalloc(reinterpret_cast<void **>(&host_shift), 2 * sizeof(T), hipHostMallocDefault));
+      for (int i = 0; i < 2; i++)
+        KM_HIP_TRY(hipEventCreateWithFlags(&shift_ready[i], hipEventDisableTiming));
+    }
+    auto queue_iteration = [&](int i) -> int {
+      log_msg(verbose, LOG_VERBOSE, "KMeans - Iteration %d/%d", i, max_iterations);
+      KM_TRY(step_async());
+      KM_HIP_TRY(hipMemcpyAsync(host_shift + (i & 1), shift2, sizeof(T), hipMemcpyDeviceToHost, stream));
+      KM_HIP_TRY(hipEventRecord(shift_ready[i & 1], stream));
+      return 0;
+    };
+    KM_TRY(queue_iteration(0));
+    int updates = 0;
+    for (int i = 0; i < max_iterations; i++) {
+      const bool queued_next = i + 1 < max_iterations;
+      if (queued_next) KM_TRY(queue_iteration(i + 1));
+      KM_HIP_TRY(hipEventSynchronize(shift_ready[i & 1]));
+      updates = i + 1;
+      bool done = (double)host_shift[i & 1] < threshold;
+      if (done) log_msg(verbose, LOG_INFO, "Threshold triggered. Terminating early.");
       if (g_stop_flag) {
         fprintf(stderr, "Signal caught. Terminated early.\n");
         g_stop_flag = 0;
         done = true;
       }
-      if (done || i == max_iterations - 1) {
-        KM_TRY(assign());  // final relabel with the final centroids
-        break;
+      if (!done && queued_next) continue;
+      if (queued_next) {
+        // labels and minimum distances of the queued iteration are the final relabel
+        cur ^= 1;
+        PROFILED("row_norms", launch_row_norms<T>(stream, C[cur], cnorm, k, d));
+      } else {
+        KM_TRY(assign());
       }
+      break;
     }
-    KM_HIP_TRY(hipStreamSynchronize(stream));
-    if (iters) *iters = updates;
+    *updates_out = updates;
     return 0;
   }
 

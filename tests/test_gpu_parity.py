@@ -224,9 +224,29 @@ def test_threshold_stop(hip, oracle, dtype):
         h.set_centroids(C0)
         done = h.fit(200, thr)
         C = h.centroids()
-    wC, _, it, hist = oracle.lloyd(X, C0, 200, thr, threads=2)
+        L = h.labels()
+        inertia = h.inertia()
+        # The convergence scalar is read one iteration behind the queue: at the stop the
+        # queued iteration's update is dropped. The handle must be left exactly at the
+        # stopping point: same centroids and labels from a fresh assignment pass, and
+        # the next step continues from them.
+        h.assign()
+        assert np.array_equal(h.labels(), L) and h.inertia() == inertia
+        h.iterate(1)
+        C_next = h.centroids()
+        # max_iterations reached while the threshold never triggers: no queued iteration
+        h.set_centroids(C0)
+        assert h.fit(2, 1e-30) == 2
+        C2, L2 = h.centroids(), h.labels()
+    wC, wL, it, hist = oracle.lloyd(X, C0, 200, thr, threads=2)
     assert done == it + 1 and done < 200
     assert_centroids_close(C, wC, dtype)
+    assert np.array_equal(L, wL)
+    wnext, _ = oracle.update(X, L, C)
+    assert_centroids_close(C_next, wnext, dtype)
+    w2C, w2L, _, _ = oracle.lloyd(X, C0, 2, 0.0, threads=2)
+    assert_centroids_close(C2, w2C, dtype)
+    assert np.array_equal(L2, w2L)
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
