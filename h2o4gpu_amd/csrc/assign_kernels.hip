@@ -889,8 +889,10 @@ int pick_assign_variant(int requested, int64_t n, int d, int k) {
   if (rowstat_ok) return ASSIGN_ROWSTAT;
   // Short rows with a large model: the tiled kernel's d-loop has one or two stages and
   // cannot hide its loads; chunked row-stationary sweeps re-read X once per chunk, which
-  // is cheap next to the matrix work of 700+ centroids.
-  if (dp != 0 && dp * (int)sizeof(T) <= 256) return ASSIGN_ROWSTAT;
+  // is cheap next to the matrix work of 700+ centroids. Longer rows only when they fill the
+  // register slice exactly (measured, chunked vs tiled: 2M x 128 f32 k=2048 0.83 vs 0.78 of
+  // peak, 4M x 64 f64 k=2048 0.78 vs 0.68; with d = 96 padded to 128 it is 0.58 vs 0.71).
+  if (dp != 0 && (dp * (int)sizeof(T) <= 256 || d == dp)) return ASSIGN_ROWSTAT;
   return ASSIGN_TILED;
 }
 
