@@ -741,23 +741,26 @@ struct Engine : h2o4gpu_kmeans_handle {
     KM_HIP_TRY(hipSetDevice(dev));
     if (!have_centroids) return H2O4GPU_KMEANS_ESTATE;
     if (rows == 0) return 0;
-    T *dX = nullptr, *dxn = nullptr;
+    T *dX = nullptr, *dxn = nullptr, *dmin = nullptr;
     int *dl = nullptr;
     int rc = dalloc(&dX, rows * d);
     if (rc == 0) rc = dalloc(&dxn, rows);
     if (rc == 0) rc = dalloc(&dl, rows);
-    if (rc == 0) rc = run_predict(rows, hX, out, dX, dxn, dl);
+    // running minimum per row: a model swept in chunks of centroids merges through it
+    if (rc == 0) rc = dalloc(&dmin, rows);
+    if (rc == 0) rc = run_predict(rows, hX, out, dX, dxn, dl, dmin);
     (void)hipStreamSynchronize(stream);
     if (dX) (void)hipFree(dX);
     if (dxn) (void)hipFree(dxn);
     if (dl) (void)hipFree(dl);
+    if (dmin) (void)hipFree(dmin);
     return rc;
   }
-  int run_predict(size_t rows, const void *hX, int *out, T *dX, T *dxn, int *dl) {
+  int run_predict(size_t rows, const void *hX, int *out, T *dX, T *dxn, int *dl, T *dmin) {
     KM_TRY(upload_rows(dev, stream, dX, hX, rows * d * sizeof(T)));
     PROFILED("row_norms", launch_row_norms<T>(stream, dX, dxn, (int64_t)rows, d));
-    PROFILED("assign", launch_assign<T>(stream, opt_assign, dX, dxn, C[cur], cnorm, dl,
-                                        (T *)nullptr, (int64_t)rows, d, k, num_cu, &last_variant));
+    PROFILED("assign", launch_assign<T>(stream, opt_assign, dX, dxn, C[cur], cnorm, dl, dmin,
+                                        (int64_t)rows, d, k, num_cu, &last_variant));
     KM_HIP_TRY(hipMemcpyAsync(out, dl, rows * sizeof(int), hipMemcpyDeviceToHost, stream));
     KM_HIP_TRY(hipStreamSynchronize(stream));
     return 0;
