@@ -695,7 +695,12 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
       *reinterpret_cast<vec_t *>(Bs + buf * B_ELEMS + lds_off[q]) = breg[q];
   };
 
-  for (int c0 = 0; c0 < k; c0 += BC) {
+  // MODE 1 has no dependency between centroid blocks: each workgroup takes the single
+  // block blockIdx.y, which keeps a short batch of rows (a transform of 100,000 rows is
+  // 782 row tiles on 512 workgroup slots) from ending in a half-empty last round.
+  const int c_begin = MODE == 1 ? (int)blockIdx.y * BC : 0;
+  const int c_end = MODE == 1 ? min(k, c_begin + BC) : k;
+  for (int c0 = c_begin; c0 < c_end; c0 += BC) {
     acc_t acc[CT][RT];
 #pragma unroll
     for (int ct = 0; ct < CT; ct++) {
@@ -1121,7 +1126,8 @@ static int launch_tiled_bcw(hipStream_t s, const T *X, const T *xnorm, const T *
                             int64_t ldn, int d, int k) {
   typedef TiledCfg<T, BCW> Cfg;
   const size_t lds = (size_t)2 * (Cfg::BC + Cfg::BR) * Cfg::BK * sizeof(T);
-  const dim3 grid((unsigned)((n + Cfg::BR - 1) / Cfg::BR));
+  const dim3 grid((unsigned)((n + Cfg::BR - 1) / Cfg::BR),
+                  MODE == 1 ? (unsigned)((k + Cfg::BC - 1) / Cfg::BC) : 1u);
   const int vw = Mfma<T>::VW;
   const bool vec = (d % vw == 0) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0) &&
                    ((reinterpret_cast<uintptr_t>(C) & 15) == 0);
