@@ -475,6 +475,7 @@ struct Engine : h2o4gpu_kmeans_handle {
   int init_random_rows(int seed) override {
     KM_HIP_TRY(hipSetDevice(dev));
     if (!have_data) return H2O4GPU_KMEANS_ESTATE;
+    if ((int64_t)k > n) return H2O4GPU_KMEANS_EARG;
     std::vector<int> v((size_t)n);
     std::iota(v.begin(), v.end(), 0);
     if (seed >= 0) {
@@ -508,6 +509,7 @@ struct Engine : h2o4gpu_kmeans_handle {
   int init_plusplus(int seed) override {
     KM_HIP_TRY(hipSetDevice(dev));
     if (!have_data) return H2O4GPU_KMEANS_ESTATE;
+    if ((int64_t)k > n) return H2O4GPU_KMEANS_EARG;
     std::mt19937 gen(seed >= 0 ? (unsigned)seed : std::random_device{}());
     std::uniform_int_distribution<> first(0, (int)(n - 1));
     std::uniform_real_distribution<double> uni(0.0, 1.0);
@@ -993,8 +995,9 @@ KM_API int h2o4gpu_kmeans_create(h2o4gpu_kmeans_handle **out, int elem_size, siz
   *out = nullptr;
   // rows must fit int32 (labels and row indices are int32, as in kmeans_init
   // kmeans_h2o4gpu.cu:574-579, which exits instead)
-  if (rows < 1 || cols < 1 || k < 1 || rows > 2147483647ull || cols > 1000000ull ||
-      (size_t)k > rows)
+  // k may exceed rows (a shard can hold fewer rows than the model has centroids); only
+  // the row-based starts need k <= rows
+  if (rows < 1 || cols < 1 || k < 1 || rows > 2147483647ull || cols > 1000000ull)
     return H2O4GPU_KMEANS_EARG;
   if (elem_size == 4) return create_engine<float>(out, rows, cols, k, gpu_id, verbose);
   if (elem_size == 8) return create_engine<double>(out, rows, cols, k, gpu_id, verbose);

@@ -118,7 +118,9 @@ int h2o4gpu_kmeans_device_count(void);
  * ------------------------------------------------------------------------- */
 typedef struct h2o4gpu_kmeans_handle h2o4gpu_kmeans_handle;
 
-/* elem_size: 4 = float, 8 = double. */
+/* elem_size: 4 = float, 8 = double. rows <= INT32_MAX (labels are int32). k may
+ * exceed rows; only the row-based starts (init_random_rows, init_plusplus) then
+ * return H2O4GPU_KMEANS_EARG. */
 int h2o4gpu_kmeans_create(h2o4gpu_kmeans_handle **out, int elem_size,
                           size_t rows, size_t cols, int k, int gpu_id,
                           int verbose);

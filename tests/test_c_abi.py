@@ -45,7 +45,7 @@ def test_bad_arguments_are_rejected_without_a_device(hip):
     h = ctypes.c_void_p()
     assert lib.h2o4gpu_kmeans_create(ctypes.byref(h), 3, 10, 2, 2, 0, 0) == -2     # elem size
     assert lib.h2o4gpu_kmeans_create(ctypes.byref(h), 4, 0, 2, 2, 0, 0) == -2      # no rows
-    assert lib.h2o4gpu_kmeans_create(ctypes.byref(h), 4, 10, 2, 11, 0, 0) == -2    # k > rows
+    assert lib.h2o4gpu_kmeans_create(ctypes.byref(h), 4, 10, 2, 0, 0, 0) == -2     # no centroids
     assert lib.h2o4gpu_kmeans_create(None, 4, 10, 2, 2, 0, 0) == -2
     assert lib.h2o4gpu_kmeans_assign(None) == -2
     slot_c, slot_l = ctypes.c_void_p(), ctypes.c_void_p()
