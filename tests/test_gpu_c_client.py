@@ -20,6 +20,29 @@ def client_data():
     return np.ascontiguousarray(X), np.ascontiguousarray(C0.astype(np.float32))
 
 
+CXX_CLIENT = os.path.join(HERE, "cxx_abi_client")
+
+
+def test_cxx_client_builds_from_the_template_header():
+    """include/h2o4gpu_kmeans.hpp mirrors the reference's C++ templates
+    (src/include/solver/kmeans.h:16-54); a caller written against them compiles with g++
+    and resolves the library (no GPU needed to check that)."""
+    if not os.path.exists(CXX_CLIENT):
+        subprocess.check_call(["g++", "-O1", "-Wall", "-Wextra", "-std=c++17", "-o", CXX_CLIENT,
+                               CXX_CLIENT + ".cpp", "-L" + os.path.join(HERE, "..", "h2o4gpu_amd"),
+                               "-lh2o4gpu_kmeans_hip", "-Wl,-rpath,$ORIGIN/../h2o4gpu_amd"])
+    out = subprocess.run(["ldd", CXX_CLIENT], capture_output=True, text=True).stdout
+    line = [l for l in out.splitlines() if "libh2o4gpu_kmeans_hip.so" in l]
+    assert line and "not found" not in line[0], out
+
+
+@pytest.mark.gpu
+def test_cxx_client_runs():
+    proc = subprocess.run([CXX_CLIENT], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    assert proc.stdout.split() == ["float", "ok", "double", "ok"]
+
+
 def test_client_is_built_against_the_public_header():
     """build() compiles the client with gcc from the header alone; it must resolve the
     library next to the package (no GPU needed to check the link)."""
