@@ -338,6 +338,13 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
   // the only exposed memory latency is that of the first tile.
   T xn[ROWT][DCH];
   T xxn[ROWT];
+  T pmn[ROWT];
+  int pln[ROWT];
+#pragma unroll
+  for (int rt = 0; rt < ROWT; rt++) {
+    pmn[rt] = 0;
+    pln[rt] = -1;
+  }
   auto fetch_rows = [&](int64_t wrow0) {
 #pragma unroll
     for (int rt = 0; rt < ROWT; rt++) {
@@ -368,6 +375,10 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
         }
       }
       xxn[rt] = xnorm[row];
+      if (merge) {  // the row's result from the earlier chunks travels with the prefetch
+        pmn[rt] = mindist[row];
+        pln[rt] = labels[row];
+      }
     }
   };
   const int64_t base0 = (int64_t)blockIdx.x * ROWS_PER_WG;
@@ -376,11 +387,15 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
     const int64_t wrow0 = base + (int64_t)wave * ROWS_PER_WAVE;
     T x[ROWT][DCH];
     T xx[ROWT];
+    T pm[ROWT];
+    int pl[ROWT];
 #pragma unroll
     for (int rt = 0; rt < ROWT; rt++) {
 #pragma unroll
       for (int s = 0; s < DCH; s++) x[rt][s] = xn[rt][s];
       xx[rt] = xxn[rt];
+      pm[rt] = pmn[rt];
+      pl[rt] = pln[rt];
     }
     {
       const int64_t nbase = base + (int64_t)gridDim.x * ROWS_PER_WG;
@@ -510,7 +525,7 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
         // this chunk is strictly closer (earlier chunks hold the lower indices).
         T bv = best[rt];
         int bi = bidx[rt] < 0 ? -1 : bidx[rt] + c_off;
-        if (merge) argmin_merge(bv, bi, mindist[row], labels[row]);
+        if (merge) argmin_merge(bv, bi, pm[rt], pl[rt]);
         labels[row] = bi;
         if (mindist) mindist[row] = bv;
       }
@@ -1016,7 +1031,10 @@ struct RowstatDispatch<float, FUSE> {
 #define KM_ROWT_F32_32 2
 #endif
       KM_ROWSTAT_CASE(float, 32, KM_ROWT_F32_32);
-      KM_ROWSTAT_CASE(float, 64, 2);
+#ifndef KM_ROWT_F32_64
+#define KM_ROWT_F32_64 2
+#endif
+      KM_ROWSTAT_CASE(float, 64, KM_ROWT_F32_64);
       KM_ROWSTAT_CASE(float, 128, 1);
     }
     return H2O4GPU_KMEANS_EARG;
