@@ -265,3 +265,19 @@ def test_concurrent_fits_from_two_threads(shim):
         for rc, C, L, info in out[i]:
             assert rc == 0 and np.array_equal(C, wantC) and np.array_equal(L, wantL)
             assert info == want_info
+
+
+def test_sigint_stops_the_loop_when_handlers_are_enabled(hip):
+    """Runs in a child process: the handler is process-wide and must not replace pytest's."""
+    import json
+    import os
+    import subprocess
+    import sys
+    here = os.path.dirname(os.path.abspath(__file__))
+    proc = subprocess.run([sys.executable, os.path.join(here, "signal_stop_check.py")],
+                          capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    r = json.loads(proc.stdout.strip().splitlines()[-1])
+    assert r["rc"] == 0 and r["labels_in_range"]
+    assert 1 <= r["iterations"] < 2_000_000       # stopped early ...
+    assert "Signal caught" in proc.stderr         # ... for the stated reason
