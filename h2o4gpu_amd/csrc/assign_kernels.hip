@@ -997,14 +997,16 @@ static int launch_rowstat_dp(hipStream_t s, const T *X, const T *xnorm,
                              T *mindist, int64_t n, int d, int k, int num_cu,
                              double *psums, int *pcounts, int *slots, int c_off, int merge) {
   const size_t lds = FUSE ? rowstat_fused_lds<T>(d, k) : rowstat_lds<T>(d, k);
-  // float32 rows of up to 32 features leave registers for 16 wavefronts: one such
-  // workgroup per CU measured 5-12 % ahead of two 4-wave workgroups (10M x 32 and 8M x 16)
-  constexpr bool wide = sizeof(T) == 4 && DP <= 32;
+  // Shapes whose register use fits 128 VGPRs run one 16-wavefront workgroup per CU, which
+  // measured ahead of two 4-wave workgroups everywhere it applies (float32 10M x 32 and
+  // 8M x 16: 5-12 %; 1M x 64, k = 64: 12 %; float64 8M x 16: 8 %).
+  constexpr bool wide = (sizeof(T) == 4 && (DP <= 32 || (DP == 64 && ROWT == 1))) ||
+                        (sizeof(T) == 8 && DP <= 32 && ROWT <= 2);
   if (!wide && rowstat_two_per_cu(lds))
     return launch_rowstat_nw<T, DP, ROWT, FUSE, 4>(s, X, xnorm, C, cnorm, labels, mindist, n, d,
                                                    k, num_cu, psums, pcounts, slots, lds, c_off, merge);
   // one workgroup per CU: as many wavefronts as the register budget allows
-  if constexpr (sizeof(T) == 4 && DP <= 32)
+  if constexpr (wide)
     return launch_rowstat_nw<T, DP, ROWT, FUSE, 16>(s, X, xnorm, C, cnorm, labels, mindist, n, d,
                                                     k, num_cu, psums, pcounts, slots, lds, c_off, merge);
   else
@@ -1031,10 +1033,7 @@ struct RowstatDispatch<float, FUSE> {
 #define KM_ROWT_F32_32 2
 #endif
       KM_ROWSTAT_CASE(float, 32, KM_ROWT_F32_32);
-#ifndef KM_ROWT_F32_64
-#define KM_ROWT_F32_64 2
-#endif
-      KM_ROWSTAT_CASE(float, 64, KM_ROWT_F32_64);
+      KM_ROWSTAT_CASE(float, 64, 1);  // one row tile: fits 16 wavefronts per CU
       KM_ROWSTAT_CASE(float, 128, 1);
     }
     return H2O4GPU_KMEANS_EARG;
@@ -1047,9 +1046,10 @@ struct RowstatDispatch<double, FUSE> {
                  int k, int num_cu, double *psums, int *pcounts, int *slots, int c_off = 0,
                  int merge = 0) {
     switch (rowstat_dp<double>(d)) {
-      KM_ROWSTAT_CASE(double, 8, 4);
-      KM_ROWSTAT_CASE(double, 16, 4);
-      KM_ROWSTAT_CASE(double, 32, 4);
+      // two row tiles keep these within 128 registers, i.e. 16 wavefronts per CU
+      KM_ROWSTAT_CASE(double, 8, 2);
+      KM_ROWSTAT_CASE(double, 16, 2);
+      KM_ROWSTAT_CASE(double, 32, 2);
       KM_ROWSTAT_CASE(double, 64, 2);
     }
     return H2O4GPU_KMEANS_EARG;
