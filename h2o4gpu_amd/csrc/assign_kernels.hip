@@ -1001,7 +1001,7 @@ static int launch_rowstat_dp(hipStream_t s, const T *X, const T *xnorm,
   // measured ahead of two 4-wave workgroups everywhere it applies (float32 10M x 32 and
   // 8M x 16: 5-12 %; 1M x 64, k = 64: 12 %; float64 8M x 16: 8 %).
   constexpr bool wide = (sizeof(T) == 4 && (DP <= 32 || (DP == 64 && ROWT == 1))) ||
-                        (sizeof(T) == 8 && DP <= 32 && ROWT <= 2);
+                        (sizeof(T) == 8 && ((DP <= 32 && ROWT <= 2) || (DP == 64 && ROWT == 1)));
   if (!wide && rowstat_two_per_cu(lds))
     return launch_rowstat_nw<T, DP, ROWT, FUSE, 4>(s, X, xnorm, C, cnorm, labels, mindist, n, d,
                                                    k, num_cu, psums, pcounts, slots, lds, c_off, merge);
@@ -1050,7 +1050,7 @@ struct RowstatDispatch<double, FUSE> {
       KM_ROWSTAT_CASE(double, 8, 2);
       KM_ROWSTAT_CASE(double, 16, 2);
       KM_ROWSTAT_CASE(double, 32, 2);
-      KM_ROWSTAT_CASE(double, 64, 2);
+      KM_ROWSTAT_CASE(double, 64, 1);
     }
     return H2O4GPU_KMEANS_EARG;
   }
