@@ -64,6 +64,63 @@ static void maybe_install_signal_handlers() {
   }
 }
 
+// The first k entries of
+//     std::vector<int> v(n); std::iota(...); std::shuffle(v.begin(), v.end(),
+//                                                        std::default_random_engine(seed));
+// (the reference's random-row start, kmeans_h2o4gpu.cu:662-669) without shuffling n entries.
+// libstdc++'s shuffle walks i = 1 .. n-1 and swaps v[i] with v[j_i], j_i uniform in [0, i];
+// when step i runs, v[i] still holds i, so an entry below k changes only at steps with
+// j_i < k, where it receives i. Only those steps touch memory; what remains per step is
+// the generator (minstd_rand0: x <- 16807 x mod 2^31-1) and the acceptance test of
+// uniform_int_distribution's two-division fallback, with the quotient urngrange / (i+1)
+// carried along instead of recomputed. Below 46341 rows libstdc++ takes a different path
+// (two swaps per draw) and the plain call is used; it is cheap there.
+// 10M rows: 25 ms instead of 190 ms (the plain shuffle is bound by its random swaps).
+static void first_rows_of_shuffle(int64_t n, int k, unsigned seed, int *out) {
+  const uint64_t M = 2147483647ull;    // minstd_rand0 modulus
+  const uint64_t R = M - 2;            // max() - min() of the engine
+  if ((uint64_t)n <= R / (uint64_t)n || n < 2 * (int64_t)k + 2) {
+    std::vector<int> v((size_t)n);
+    std::iota(v.begin(), v.end(), 0);
+    std::shuffle(v.begin(), v.end(), std::default_random_engine(seed));
+    std::copy(v.begin(), v.begin() + k, out);
+    return;
+  }
+  uint64_t x = seed % M;
+  if (x == 0) x = 1;
+  auto next = [&]() -> uint64_t {  // one step of the generator, value in [1, M-1]
+    const uint64_t p = x * 16807ull;
+    uint64_t r = (p & M) + (p >> 31);
+    if (r >= M) r -= M;
+    x = r;
+    return r;
+  };
+  std::vector<int> a((size_t)k);
+  std::iota(a.begin(), a.end(), 0);
+  // steps inside the first k entries: ordinary swaps
+  for (int64_t i = 1; i < k; i++) {
+    const uint64_t ue = (uint64_t)i + 1, scaling = R / ue, past = ue * scaling;
+    uint64_t ret;
+    do ret = next() - 1; while (ret >= past);
+    std::swap(a[(size_t)i], a[(size_t)(ret / scaling)]);
+  }
+  // steps i >= k: v[i] == i arrives at entry j when j < k
+  uint64_t scaling = R / ((uint64_t)k + 1);
+  uint64_t hold_until = R / scaling;  // largest i+1 with this quotient
+  for (int64_t i = k; i < n; i++) {
+    const uint64_t ue = (uint64_t)i + 1;
+    if (ue > hold_until) {
+      scaling = R / ue;
+      hold_until = R / scaling;
+    }
+    const uint64_t past = ue * scaling;
+    uint64_t ret;
+    do ret = next() - 1; while (ret >= past);
+    if (ret < (uint64_t)k * scaling) a[(size_t)(ret / scaling)] = (int)i;
+  }
+  std::copy(a.begin(), a.end(), out);
+}
+
 static int visible_devices() {
   int n = 0;
   if (hipGetDeviceCount(&n) != hipSuccess) {
@@ -110,6 +167,7 @@ struct h2o4gpu_kmeans_handle {
   virtual int set_data_device(const void *dX) = 0;
   virtual int set_centroids_host(const void *C) = 0;
   virtual int init_random_rows(int seed) = 0;
+  virtual int start_from_rows(const int *rows) = 0;  // centroids = the given k rows of the data
   virtual int init_plusplus(int seed) = 0;
   std::vector<int> last_seed_rows;
   virtual int fit(int max_iterations, double threshold, int *iters) = 0;
@@ -476,16 +534,22 @@ struct Engine : h2o4gpu_kmeans_handle {
     KM_HIP_TRY(hipSetDevice(dev));
     if (!have_data) return H2O4GPU_KMEANS_ESTATE;
     if ((int64_t)k > n) return H2O4GPU_KMEANS_EARG;
-    std::vector<int> v((size_t)n);
-    std::iota(v.begin(), v.end(), 0);
-    if (seed >= 0) {
-      std::shuffle(v.begin(), v.end(), std::default_random_engine(seed));
-    } else {
+    unsigned useed = (unsigned)seed;
+    if (seed < 0) {
       std::random_device rd;
-      std::shuffle(v.begin(), v.end(), std::default_random_engine(rd()));
+      useed = rd();
     }
-    last_seed_rows.assign(v.begin(), v.begin() + k);
+    std::vector<int> v((size_t)k);
+    first_rows_of_shuffle(n, k, useed, v.data());
+    last_seed_rows = v;
     return init_from_rows(v.data());
+  }
+
+  int start_from_rows(const int *rows) override {
+    KM_HIP_TRY(hipSetDevice(dev));
+    if (!have_data || !rows) return H2O4GPU_KMEANS_ESTATE;
+    last_seed_rows.assign(rows, rows + k);
+    return init_from_rows(rows);
   }
 
   int init_from_rows(const int *idx_host) {
@@ -886,10 +950,20 @@ static int fit_entry(int verbose, int seed, int gpu_id, size_t rows, size_t cols
   }
   h2o4gpu_kmeans_handle *h = nullptr;
   KM_TRY(h2o4gpu_kmeans_create(&h, sizeof(T), rows, cols, k, gpu_id, verbose));
+  // the seeded permutation behind the random-row start is host work that needs only the
+  // row count: it runs beside the upload
+  std::vector<int> start_rows;
+  std::thread row_picker;
+  if (init_from_data == 0 && seed >= 0) {
+    start_rows.resize((size_t)k);
+    row_picker = std::thread(first_rows_of_shuffle, (int64_t)rows, k, (unsigned)seed,
+                             start_rows.data());
+  }
   int rc = h->set_data_host(srcdata);
+  if (row_picker.joinable()) row_picker.join();
   if (rc == 0) {
     if (init_from_data == 0) {
-      rc = h->init_random_rows(seed);
+      rc = start_rows.empty() ? h->init_random_rows(seed) : h->start_from_rows(start_rows.data());
     } else if (init_from_data == 1) {
       rc = h->init_plusplus(seed);
     } else if (init_from_data == 2) {
@@ -1077,6 +1151,13 @@ KM_API int h2o4gpu_kmeans_get_min_distances(h2o4gpu_kmeans_handle *h, void *m) {
   KM_CHECK_HANDLE(h);
   return m ? h->get_min_distances(m) : H2O4GPU_KMEANS_EARG;
 }
+KM_API int h2o4gpu_kmeans_random_start_rows(int seed, size_t rows, int k, int *out) {
+  if (!out || k < 1 || rows < (size_t)k || rows > 2147483647ull || seed < 0)
+    return H2O4GPU_KMEANS_EARG;
+  first_rows_of_shuffle((int64_t)rows, k, (unsigned)seed, out);
+  return 0;
+}
+
 KM_API int h2o4gpu_kmeans_last_fit_info(double *inertia, int *iterations) {
   if (!g_last_fit.valid) return H2O4GPU_KMEANS_ESTATE;
   if (inertia) *inertia = g_last_fit.inertia;

@@ -40,6 +40,7 @@ PROTOTYPES = {
     "cudaresetdevice_bare": (c_int, []),
     "h2o4gpu_kmeans_device_count": (c_int, []),
     "h2o4gpu_kmeans_last_fit_info": (c_int, [P(c_double), P(c_int)]),
+    "h2o4gpu_kmeans_random_start_rows": (c_int, [c_int, c_size_t, c_int, c_void_p]),
     "h2o4gpu_kmeans_create": (c_int, [P(c_void_p), c_int, c_size_t, c_size_t, c_int, c_int, c_int]),
     "h2o4gpu_kmeans_destroy": (c_int, [c_void_p]),
     "h2o4gpu_kmeans_set_data_host": (c_int, [c_void_p, c_void_p]),
@@ -278,6 +279,13 @@ def copy_probe(nbytes, reps=10, gpu_id=0):
     ms = c_float(0.0)
     _check("copy_probe", lib().h2o4gpu_kmeans_copy_probe(gpu_id, nbytes, reps, ctypes.byref(ms)))
     return ms.value
+
+
+def random_start_rows(seed, rows, k):
+    """Rows a fit with init_from_data = 0 starts from (host-only computation)."""
+    out = np.empty(k, np.int32)
+    _check("random_start_rows", lib().h2o4gpu_kmeans_random_start_rows(int(seed), int(rows), int(k), _vp(out)))
+    return out
 
 
 def last_fit_info():

@@ -63,6 +63,13 @@ int make_ptr_double_kmeans(int dopredict, int verbose, int seed, int gpu_id,
                            const double *centroids, double **pred_centroids,
                            int **pred_labels);
 
+/* The rows a fit with init_from_data == 0 starts from: entries 0..k-1 of
+ * std::shuffle(iota(rows), std::default_random_engine(seed)) as libstdc++ computes
+ * them (the reference's rule, src/gpu/kmeans/kmeans_h2o4gpu.cu:662-669), seed >= 0.
+ * Host-only, needs no device. out: [k]. No counterpart in the reference, which does
+ * not report the rows it picked. */
+int h2o4gpu_kmeans_random_start_rows(int seed, size_t rows, int k, int *out);
+
 /* Inertia (sum over rows of the squared distance to the assigned centroid,
  * accumulated in double in a fixed order) and number of Lloyd iterations of
  * the calling thread's most recent successful fit through make_ptr_*_kmeans.

@@ -67,3 +67,19 @@ def test_no_device_is_an_error_not_a_fallback(hip):
     out_c, out_l = np.zeros(4, np.float32), np.zeros(4, np.int32)
     assert ch2o4gpu_gpu.make_ptr_float_kmeans(0, 0, 1, 0, 1, 4, 2, 2, 3, 0, 0.0, X.flatten(),
                                               np.empty([]), out_c, out_l) != 0
+
+
+def test_random_start_rows_equal_the_standard_library_shuffle(hip, oracle):
+    """The engine computes the first k entries of std::shuffle(iota(n),
+    default_random_engine(seed)) without shuffling n entries; the oracle makes the two
+    standard-library calls as the reference writes them (kmeans_h2o4gpu.cu:662-669).
+    Both sides of libstdc++'s 46340-row switch, generator edge seeds, k from 1 to n."""
+    for n in (1, 2, 3, 10, 257, 1000, 46339, 46340, 46341, 46342, 50000, 100003, 1_000_000):
+        for k in (1, 2, 7, 64, 256, 1000, n):
+            if k > n:
+                continue
+            for seed in (0, 1, 7, 1234, 2147483646, 2147483647):
+                want = oracle.random_rows(seed, n, k)
+                got = hip.random_start_rows(seed, n, k)
+                assert np.array_equal(got, want), (n, k, seed)
+    assert hip.lib().h2o4gpu_kmeans_random_start_rows(1, 5, 6, None) == -2
