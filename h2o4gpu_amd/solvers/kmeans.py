@@ -68,9 +68,13 @@ def _device_rows(X):
 
 def _check_data_content(do_check, name, data):
     """Reference solvers/utils.py:144-158."""
-    if do_check == 1:
-        assert np.isfinite(data).all(), "%s contains Inf" % name
-        assert not np.isnan(data).any(), "%s contains NA" % name
+    if do_check == 1 and np.size(data):
+        # same two assertions as the reference, from the extremes (a NaN propagates into
+        # both, an infinity into one of them): two passes and no boolean temporary the
+        # size of the data
+        lo, hi = np.min(data), np.max(data)
+        assert np.isfinite(lo) and np.isfinite(hi), "%s contains Inf" % name
+        assert not (np.isnan(lo) or np.isnan(hi)), "%s contains NA" % name
 
 
 def assert_satisfies(value, cond, message):
@@ -342,7 +346,8 @@ class KMeansH2O:
         elif data.dtype == np.float32:
             self._print_verbose(1, "Detected np.float32 data")
             self.double_precision = 0
-        return data.flatten()
+        # row-major and contiguous, without the copy flatten() always makes
+        return np.ascontiguousarray(data).reshape(-1)
 
     def _print_verbose(self, level, msg):
         if self.verbose > level:
