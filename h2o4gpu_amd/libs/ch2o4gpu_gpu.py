@@ -48,6 +48,37 @@ def _take(slot, dest, count):
         _k.libc_free(slot)
 
 
+def _adopt(slot, count, dtype):
+    """A numpy array over the library's malloc()ed buffer (no copy); the buffer is freed
+    when the last view of it goes away. This is what SWIG's INPLACE_ARRAY1(T**) typemap
+    does by re-pointing the caller's array, minus the stranded original storage."""
+    import weakref
+    if not slot.value or count <= 0:
+        _k.libc_free(slot)
+        return np.empty(0, dtype)
+    ctype = {np.dtype(np.float32): ctypes.c_float, np.dtype(np.float64): ctypes.c_double,
+             np.dtype(np.int32): ctypes.c_int32}[np.dtype(dtype)]
+    buf = (ctype * int(count)).from_address(slot.value)
+    weakref.finalize(buf, _k.libc_free, ctypes.c_void_p(slot.value))
+    return np.frombuffer(buf, dtype=dtype)
+
+
+def kmeans_transform_owned(verbose, gpu_id, n_gpu, m, n, k, srcdata, centroids, dtype):
+    """kmeans_transform_float/double without the preallocated output array: returns
+    (status, preds) where preds ([k*m], centroid-major) owns the library's buffer. Not part
+    of the reference's module; the estimator uses it to skip zero-filling and copying an
+    m x k array."""
+    dtype = np.dtype(dtype)
+    fn_name = "kmeans_transform_float" if dtype == np.float32 else "kmeans_transform_double"
+    lib = _k.lib()
+    src_p, _src_keep = _in_array(srcdata, dtype)
+    cen_p, _cen_keep = _in_array(centroids, dtype)
+    slot = ctypes.c_void_p()
+    rc = getattr(lib, fn_name)(int(verbose), int(gpu_id), int(n_gpu), int(m), int(n), int(k), src_p, cen_p,
+                               ctypes.byref(slot))
+    return rc, _adopt(slot, int(m) * int(k) if rc == 0 else 0, dtype)
+
+
 def _make_ptr(fn_name, dtype, dopredict, verbose, seed, gpu_id, n_gpu, mTrain, n, k, max_iterations,
               init_from_data, threshold, srcdata, centroids, pred_centroids, pred_labels):
     lib = _k.lib()

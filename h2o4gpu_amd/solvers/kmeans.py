@@ -236,6 +236,13 @@ class KMeansH2O:
         X_np = _to_np(X)
         c_X_np = self._toc(X_np)
         cluster_centers_ = self._toc(self.cluster_centers_, convert=False)
+        owned = getattr(lib, "kmeans_transform_owned", None)
+        if owned is not None:  # adopt the library's buffer instead of zero-filling and copying
+            status, c_res = owned(self.verbose, self._gpu_id, self.n_gpus, rows, cols, self._n_clusters,
+                                  c_X_np, cluster_centers_, X_np.dtype)
+            if status != 0:
+                raise RuntimeError("KMeans transform failed in the native library (status %d)" % status)
+            return np.reshape(c_res, (rows, self._n_clusters), order='F')
         c_res = np.zeros(rows * self._n_clusters, X_np.dtype)
         if self.double_precision == 0:
             lib.kmeans_transform_float(self.verbose, self._gpu_id, self.n_gpus, rows, cols,
