@@ -399,12 +399,17 @@ def _random_shapes(count, seed):
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_one_step_on_random_shapes(hip, oracle, dtype):
-    """One Lloyd step (the kernels the dispatcher picks by itself) on 60 seeded shapes:
+    """One Lloyd step (the kernels the dispatcher picks by itself) on 60 seeded shapes and a
+    dozen extreme ones (thousands of features, more centroids than fit any LDS chunking, one
+    feature, one centroid):
     labels against the oracle up to excused near-ties, counts and new centroids against
     the oracle update of the engine's own labels."""
     tol = 1e-5 if dtype == np.float32 else 1e-12
     seen = {}
-    for (n, d, k) in _random_shapes(60, 2024):
+    extremes = [(3000, 5000, 3), (2000, 2049, 17), (30000, 3, 20000), (25000, 16, 12000), (6000, 1, 300),
+                (4000, 700, 600), (5000, 1023, 129), (70000, 2, 2), (12000, 130, 4097), (9000, 64, 9000),
+                (300, 4000, 300), (100000, 7, 1)]
+    for (n, d, k) in _random_shapes(60, 2024) + extremes:
         X = blobs(n, d, max(k, 2), dtype, seed=n + 3 * d + 7 * k)
         C0 = np.ascontiguousarray(X[np.random.default_rng(n).choice(n, size=k, replace=False)])
         with hip.Handle(n, d, k, dtype) as h:
