@@ -16,6 +16,20 @@ namespace kmhip {
 
 static constexpr int WG = 256;  // threads per workgroup (4 wavefronts)
 
+// Squared norm of one centroid row, j ascending, multiply and add rounded separately:
+// the value row_norms / post_update would store (kmeans_labels.h:187-199). The fused
+// kernels call it when they are given no norm buffer, which spares the Lloyd loop a launch.
+template <typename T>
+__device__ __forceinline__ T row_sqnorm(const T *__restrict__ x, int d) {
+#pragma clang fp contract(off)
+  T acc = 0;
+  for (int j = 0; j < d; j++) {
+    const T v = x[j];
+    acc = acc + v * v;
+  }
+  return acc;
+}
+
 // ---------------------------------------------------------------------------
 // VALU variant: one thread per row, a chunk of centroids broadcast from LDS.
 // Arithmetic order is j ascending with separate multiply and add, so this
@@ -115,12 +129,16 @@ __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
   const int sx = d | 1;                                          // row stride of the staged block
   double *sums = reinterpret_cast<double *>(smem_raw);           // [k][sx]
   int *cnt = reinterpret_cast<int *>(sums + (size_t)k * sx);     // [k]
-  T *Xs = reinterpret_cast<T *>(cnt + k + (k & 1));              // [WG][sx]
+  T *ccs = reinterpret_cast<T *>(cnt + k + (k & 1));             // [k] centroid norms
+  T *Xs = ccs + k + (k & 1);                                     // [WG][sx]
   typedef typename BlockLoad<T, VEC>::type ld_t;
   constexpr int NLD = DREG / VEC;  // loads per thread and block (upper bound)
   const int tid = threadIdx.x;
   for (int e = tid; e < k * sx; e += WG) sums[e] = 0.0;
-  for (int c = tid; c < k; c += WG) cnt[c] = 0;
+  for (int c = tid; c < k; c += WG) {
+    cnt[c] = 0;
+    ccs[c] = cnorm ? cnorm[c] : row_sqnorm<T>(C + (size_t)c * d, d);
+  }
   // LDS offset of the i-th load of this thread: element (tid + i*WG)*VEC of the block
   int off[NLD];
 #pragma unroll
@@ -185,7 +203,7 @@ __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
 #pragma unroll
         for (int j = 0; j < DREG; j++)
           if (FULL || j < d) dot = dot + xr[j] * cp[j];
-        const T t = xx + cnorm[c];
+        const T t = xx + ccs[c];
         const T dist = fabs(t - (T)2 * dot);
         if (dist < best) {
           best = dist;
@@ -329,8 +347,25 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
       Cs[((size_t)(t * NV + s / VW) * 64 + gg * MT + i) * VW + (s % VW)] = v;
     }
   }
-  for (int c = tid; c < kp; c += TPB) ccs[c] = c < k ? cnorm[c] : pos_inf<T>();
+  for (int c = tid; c < kp; c += TPB) ccs[c] = (c < k && cnorm) ? cnorm[c] : pos_inf<T>();
   __syncthreads();
+  if (cnorm == nullptr) {
+    // No norm buffer given: take the norms from the staged centroids. A staged value is
+    // -2c; halving it is exact, so the sum below (j ascending, multiply and add rounded
+    // separately) is bit for bit what row_norms / post_update would have stored.
+#pragma clang fp contract(off)
+    for (int c = tid; c < k; c += TPB) {
+      const int t = c / MT, i = c - t * MT;
+      T acc = 0;
+      for (int j = 0; j < d; j++) {
+        const int gg = j / DCH, sj = j - gg * DCH;
+        const T v = (T)-0.5 * Cs[((size_t)(t * NV + sj / VW) * 64 + gg * MT + i) * VW + (sj % VW)];
+        acc = acc + v * v;
+      }
+      ccs[c] = acc;
+    }
+    __syncthreads();
+  }
 
   constexpr int ROWS_PER_WAVE = ROWT * MT;
   constexpr int ROWS_PER_WG = NW * ROWS_PER_WAVE;
@@ -1062,7 +1097,7 @@ template <typename T>
 static size_t valu_fused_lds(int d, int k) {
   const int sx = d | 1;
   return (size_t)k * sx * sizeof(double) + ((size_t)k + 1) * sizeof(int) +
-         (size_t)WG * sx * sizeof(T) + 16;
+         ((size_t)k + 1) * sizeof(T) + (size_t)WG * sx * sizeof(T) + 16;
 }
 static int valu_fused_grid(int64_t n, size_t lds, int num_cu) {
   int per_cu = (int)((150 * 1024) / lds);
@@ -1127,6 +1162,7 @@ int launch_assign_accumulate(hipStream_t s, int variant, const T *X, const T *xn
                              const T *cnorm, int *labels, T *mindist, int64_t n, int d,
                              int k, int num_cu, double *psums, int *pcounts, int *slots,
                              int *used) {
+  // cnorm == nullptr: the kernel computes the centroid norms from C itself
   if (n <= 0 || d < 1 || k < 1) return H2O4GPU_KMEANS_EARG;
   const int v = pick_assign_variant<T>(variant, n, d, k);
   if (used) *used = v;

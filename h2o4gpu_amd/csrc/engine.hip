@@ -515,6 +515,7 @@ struct Engine : h2o4gpu_kmeans_handle {
 
   int centroids_changed() {
     PROFILED("row_norms", launch_row_norms<T>(stream, C[cur], cnorm, k, d));
+    cnorm_stale = false;
     have_centroids = true;
     return 0;
   }
@@ -626,9 +627,21 @@ struct Engine : h2o4gpu_kmeans_handle {
     return init_from_rows(idx.data());
   }
 
+  // The fused kernels compute the centroid norms themselves, so a Lloyd loop that needs no
+  // convergence scalar skips the post-update launch and leaves cnorm behind the current
+  // centroids; every other consumer of cnorm refreshes it first.
+  bool cnorm_stale = false;
+  int ensure_cnorm() {
+    if (!cnorm_stale) return 0;
+    PROFILED("row_norms", launch_row_norms<T>(stream, C[cur], cnorm, k, d));
+    cnorm_stale = false;
+    return 0;
+  }
+
   int assign() override {
     KM_HIP_TRY(hipSetDevice(dev));
     if (!have_data || !have_centroids) return H2O4GPU_KMEANS_ESTATE;
+    KM_TRY(ensure_cnorm());
     PROFILED("assign", launch_assign<T>(stream, opt_assign, X, xnorm, C[cur], cnorm,
                                         labels, mindist, n, d, k, num_cu, &last_variant));
     have_mindist = true;
@@ -640,33 +653,38 @@ struct Engine : h2o4gpu_kmeans_handle {
       PROFILED("accumulate", launch_bucketed_accumulate<T>(stream, X, labels, order, order_label,
                                                            bucket_offsets, bucket_cursor,
                                                            bucket_counts, psums, pcounts, n, d, k));
-      return finish_update(1);
+      return finish_update(1, true);
     }
     PROFILED("accumulate", launch_accumulate<T>(stream, plan, X, labels, psums, pcounts, n, d, k));
-    return finish_update(plan.row_blocks);
+    return finish_update(plan.row_blocks, true);
   }
 
-  // one Lloyd step: labels against the current centroids, then the update
-  int step_async() {
+  // one Lloyd step: labels against the current centroids, then the update.
+  // want_shift: the caller will read the convergence scalar of this step.
+  int step_async(bool want_shift) {
     if (opt_fuse && fused_slots<T>(opt_assign, n, d, k, num_cu) > 0) {
       int slots = 0;
       PROFILED("assign_accumulate",
-               launch_assign_accumulate<T>(stream, opt_assign, X, xnorm, C[cur], cnorm, labels,
-                                           mindist, n, d, k, num_cu, psums, pcounts, &slots,
+               launch_assign_accumulate<T>(stream, opt_assign, X, xnorm, C[cur], (const T *)nullptr,
+                                           labels, mindist, n, d, k, num_cu, psums, pcounts, &slots,
                                            &last_variant));
       have_mindist = true;
-      return finish_update(slots);
+      return finish_update(slots, want_shift);
     }
     KM_TRY(assign());
     return update_async();
   }
 
-  int finish_update(int slots) {
+  // post: also run pass 3 (norms of the new centroids + the shift scalar). Without it the
+  // norms are marked stale and the scalar of this step does not exist.
+  int finish_update(int slots, bool post) {
     int nsp = 0;
     PROFILED("finalize", launch_finalize<T>(stream, slots, psums, pcounts, C[cur], C[cur ^ 1],
                                             counts, shift_partials, &nsp, d, k));
-    PROFILED("post_update", launch_post_update<T>(stream, C[cur ^ 1], cnorm, shift_partials,
-                                                  nsp, shift2, d, k));
+    if (post)
+      PROFILED("post_update", launch_post_update<T>(stream, C[cur ^ 1], cnorm, shift_partials,
+                                                    nsp, shift2, d, k));
+    cnorm_stale = !post;
     cur ^= 1;
     return 0;
   }
@@ -700,7 +718,7 @@ struct Engine : h2o4gpu_kmeans_handle {
     } else {
       for (int i = 0; i < max_iterations; i++) {
         log_msg(verbose, LOG_VERBOSE, "KMeans - Iteration %d/%d", i, max_iterations);
-        KM_TRY(step_async());
+        KM_TRY(step_async(false));
         updates++;
         bool done = false;
         if (g_stop_flag) {
@@ -736,7 +754,7 @@ struct Engine : h2o4gpu_kmeans_handle {
     }
     auto queue_iteration = [&](int i) -> int {
       log_msg(verbose, LOG_VERBOSE, "KMeans - Iteration %d/%d", i, max_iterations);
-      KM_TRY(step_async());
+      KM_TRY(step_async(true));
       KM_HIP_TRY(hipMemcpyAsync(host_shift + (i & 1), shift2, sizeof(T), hipMemcpyDeviceToHost, stream));
       KM_HIP_TRY(hipEventRecord(shift_ready[i & 1], stream));
       return 0;
@@ -760,6 +778,7 @@ struct Engine : h2o4gpu_kmeans_handle {
         // labels and minimum distances of the queued iteration are the final relabel
         cur ^= 1;
         PROFILED("row_norms", launch_row_norms<T>(stream, C[cur], cnorm, k, d));
+        cnorm_stale = false;
       } else {
         KM_TRY(assign());
       }
@@ -772,7 +791,7 @@ struct Engine : h2o4gpu_kmeans_handle {
   int iterate(int steps) override {
     KM_HIP_TRY(hipSetDevice(dev));
     if (!have_data || !have_centroids) return H2O4GPU_KMEANS_ESTATE;
-    for (int i = 0; i < steps; i++) KM_TRY(step_async());
+    for (int i = 0; i < steps; i++) KM_TRY(step_async(false));
     return 0;
   }
 
@@ -823,6 +842,7 @@ struct Engine : h2o4gpu_kmeans_handle {
     return rc;
   }
   int run_predict(size_t rows, const void *hX, int *out, T *dX, T *dxn, int *dl, T *dmin) {
+    KM_TRY(ensure_cnorm());
     KM_TRY(upload_rows(dev, stream, dX, hX, rows * d * sizeof(T)));
     PROFILED("row_norms", launch_row_norms<T>(stream, dX, dxn, (int64_t)rows, d));
     PROFILED("assign", launch_assign<T>(stream, opt_assign, dX, dxn, C[cur], cnorm, dl, dmin,
@@ -860,6 +880,7 @@ struct Engine : h2o4gpu_kmeans_handle {
   int run_transform_batch(size_t lo, size_t cur_rows, size_t rows, const void *hX, void *hD,
                           T *dX, T *dxn, T *dD) {
     const T *src = static_cast<const T *>(hX) + lo * d;
+    KM_TRY(ensure_cnorm());
     KM_TRY(upload_rows(dev, stream, dX, src, cur_rows * d * sizeof(T)));
     PROFILED("row_norms", launch_row_norms<T>(stream, dX, dxn, (int64_t)cur_rows, d));
     PROFILED("transform", launch_transform<T>(stream, dX, dxn, C[cur], cnorm, dD,
@@ -876,6 +897,7 @@ struct Engine : h2o4gpu_kmeans_handle {
   int transform_resident(void *d_dist) override {
     KM_HIP_TRY(hipSetDevice(dev));
     if (!have_data || !have_centroids || !d_dist) return H2O4GPU_KMEANS_ESTATE;
+    KM_TRY(ensure_cnorm());
     PROFILED("transform", launch_transform<T>(stream, X, xnorm, C[cur], cnorm,
                                               static_cast<T *>(d_dist), n, n, d, k, num_cu));
     KM_HIP_TRY(hipStreamSynchronize(stream));

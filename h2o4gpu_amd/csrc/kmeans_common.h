@@ -70,7 +70,9 @@ const char *assign_variant_name(int variant);
 // launch_assign, plus per-workgroup partial sums psums[slot][k][d] and counts
 // pcounts[slot][k]; *slots receives the number of slots written. fused_slots()
 // returns the largest slot count the launch can use, or 0 when the shape (or a
-// forced assign variant) rules the fused kernel out.
+// forced assign variant) rules the fused kernel out. cnorm may be null: the kernel then
+// computes the centroid norms from C itself (same values, j ascending), so that a Lloyd
+// loop that needs no convergence scalar can skip launch_post_update.
 template <typename T>
 int fused_slots(int requested_variant, int64_t n, int d, int k, int num_cu);
 template <typename T>
