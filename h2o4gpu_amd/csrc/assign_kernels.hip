@@ -135,10 +135,7 @@ __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
   constexpr int NLD = DREG / VEC;  // loads per thread and block (upper bound)
   const int tid = threadIdx.x;
   for (int e = tid; e < k * sx; e += WG) sums[e] = 0.0;
-  for (int c = tid; c < k; c += WG) {
-    cnt[c] = 0;
-    ccs[c] = cnorm ? cnorm[c] : row_sqnorm<T>(C + (size_t)c * d, d);
-  }
+  for (int c = tid; c < k; c += WG) cnt[c] = 0;
   // LDS offset of the i-th load of this thread: element (tid + i*WG)*VEC of the block
   int off[NLD];
 #pragma unroll
@@ -168,6 +165,8 @@ __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
   int64_t base = (int64_t)blockIdx.x * WG;
   if (base >= n) return;  // the grid never exceeds the number of blocks
   fetch(base);
+  // centroid norms while the first block travels (visible after the barrier below)
+  for (int c = tid; c < k; c += WG) ccs[c] = cnorm ? cnorm[c] : row_sqnorm<T>(C + (size_t)c * d, d);
   const int jrot = (tid & 63) % d;
   for (; base < n; base += stride) {
     const int rows = (int)min<int64_t>(WG, n - base);
