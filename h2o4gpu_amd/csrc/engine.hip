@@ -342,6 +342,20 @@ struct StagingPool {
     }
     return 0;
   }
+
+  // Gives a device's buffers back (before the device is reset: the reset frees them
+  // behind the pool's back). The next transfer allocates new ones.
+  void forget(int dev) {
+    if (dev < 0 || dev >= MAX_DEV) return;
+    std::lock_guard<std::mutex> lock(mu);
+    for (int i = 0; i < 2; i++) {
+      if (done[dev][i]) (void)hipEventDestroy(done[dev][i]);
+      if (buf[dev][i]) (void)hipHostFree(buf[dev][i]);
+      done[dev][i] = nullptr;
+      buf[dev][i] = nullptr;
+    }
+    broken[dev] = false;
+  }
 };
 static StagingPool g_staging;
 
@@ -1396,11 +1410,18 @@ KM_API int get_compute_capability(int d_idx, int *major, int *minor, int *ratiop
   if (ratioperf) *ratioperf = 2;  // fp32 : fp64 matrix rate on MI355X
   return 0;
 }
+// Handles that still exist on the device do not survive a reset; the staging buffers of
+// the upload path are released first and come back with the next transfer.
 KM_API int cudaresetdevice(int wDev, int nDev) {
   (void)nDev;
   if (hipSetDevice(wDev) != hipSuccess) return 1;
+  g_staging.forget(wDev);
   return hipDeviceReset() == hipSuccess ? 0 : 1;
 }
-KM_API int cudaresetdevice_bare(void) { return hipDeviceReset() == hipSuccess ? 0 : 1; }
+KM_API int cudaresetdevice_bare(void) {
+  int dev = 0;
+  if (hipGetDevice(&dev) == hipSuccess) g_staging.forget(dev);
+  return hipDeviceReset() == hipSuccess ? 0 : 1;
+}
 
 }  // extern "C"

@@ -281,3 +281,19 @@ def test_sigint_stops_the_loop_when_handlers_are_enabled(hip):
     assert r["rc"] == 0 and r["labels_in_range"]
     assert 1 <= r["iterations"] < 2_000_000       # stopped early ...
     assert "Signal caught" in proc.stderr         # ... for the stated reason
+
+
+def test_fit_after_device_reset(hip):
+    """cudaresetdevice / cudaresetdevice_bare between fits: the library's pinned staging
+    buffers die with the device context and must be re-created, results unchanged."""
+    import json
+    import os
+    import subprocess
+    import sys
+    here = os.path.dirname(os.path.abspath(__file__))
+    proc = subprocess.run([sys.executable, os.path.join(here, "device_reset_check.py")],
+                          capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    r = json.loads(proc.stdout.strip().splitlines()[-1])
+    assert r["rc"] == [0, 0, 0] and r["reset_rc"] == [0, 0]
+    assert r["same_centroids"] and r["same_labels"]
