@@ -201,7 +201,7 @@ class KMeansH2O:
             self.sklearn_model.cluster_centers_ = self.cluster_centers_
 
     def predict(self, X):
-        lib = self._load_lib()
+        lib = self._require_lib("predict")
         cols, rows = self._validate_centroids(X)
         dev = _device_rows(X)
         if dev is not None:
@@ -215,9 +215,11 @@ class KMeansH2O:
         cluster_centers_ = self._toc(self.cluster_centers_, convert=False)
         c_res = np.zeros(rows, np.int32)
         c_kmeans = lib.make_ptr_float_kmeans if self.double_precision == 0 else lib.make_ptr_double_kmeans
-        c_kmeans(1, self.verbose, self.random_state, self._gpu_id, self.n_gpus, rows, cols,
-                 self._n_clusters, self._max_iter, 0, self.tol, c_X_np, cluster_centers_,
-                 np.empty([], X_np.dtype), c_res)
+        status = c_kmeans(1, self.verbose, self.random_state, self._gpu_id, self.n_gpus, rows, cols,
+                          self._n_clusters, self._max_iter, 0, self.tol, c_X_np, cluster_centers_,
+                          np.empty([], X_np.dtype), c_res)
+        if status:
+            raise RuntimeError("KMeans predict failed in the native library (status %d)" % status)
         return c_res
 
     def sklearn_predict(self, X, y=None):
@@ -228,7 +230,7 @@ class KMeansH2O:
     def transform(self, X, y=None):
         """Squared distances to every centre, shape (rows, n_clusters) (the reference returns
         the squared values, kmeans.py:389-422 with kmeans_h2o4gpu.cu:937-950)."""
-        lib = self._load_lib()
+        lib = self._require_lib("transform")
         cols, rows = self._validate_centroids(X)
         dev = _device_rows(X)
         if dev is not None:
@@ -244,12 +246,11 @@ class KMeansH2O:
                 raise RuntimeError("KMeans transform failed in the native library (status %d)" % status)
             return np.reshape(c_res, (rows, self._n_clusters), order='F')
         c_res = np.zeros(rows * self._n_clusters, X_np.dtype)
-        if self.double_precision == 0:
-            lib.kmeans_transform_float(self.verbose, self._gpu_id, self.n_gpus, rows, cols,
-                                       self._n_clusters, c_X_np, cluster_centers_, c_res)
-        else:
-            lib.kmeans_transform_double(self.verbose, self._gpu_id, self.n_gpus, rows, cols,
-                                        self._n_clusters, c_X_np, cluster_centers_, c_res)
+        fn = lib.kmeans_transform_float if self.double_precision == 0 else lib.kmeans_transform_double
+        status = fn(self.verbose, self._gpu_id, self.n_gpus, rows, cols, self._n_clusters, c_X_np,
+                    cluster_centers_, c_res)
+        if status:
+            raise RuntimeError("KMeans transform failed in the native library (status %d)" % status)
         return np.reshape(c_res, (rows, self._n_clusters), order='F')
 
     def _transform_device(self, X, dev):
@@ -280,7 +281,7 @@ class KMeansH2O:
         return self.fit(X, y).labels_
 
     def _fit(self, data):
-        lib = self._load_lib()
+        lib = self._require_lib("fit")
         c_data = self._toc(data)
         rows = np.shape(data)[0]
         cols = np.shape(data)[1]
@@ -370,6 +371,14 @@ class KMeansH2O:
         from ..libs import ch2o4gpu_gpu
         self._print_verbose(0, "\nUsing GPU KMeans solver with %d GPUs.\n" % self.n_gpus)
         return ch2o4gpu_gpu
+
+    def _require_lib(self, what):
+        lib = self._load_lib()
+        if lib is None:
+            raise RuntimeError("KMeansH2O.%s needs a usable GPU (n_gpus=%r, visible devices %r); "
+                               "use KMeans(backend='sklearn') to run on the CPU"
+                               % (what, self.n_gpus, self.devices))
+        return lib
 
     def _validate_centroids(self, X):
         assert self.cluster_centers_ is not None, "Centroids are None. Run fit() first."
@@ -483,8 +492,6 @@ class KMeans:
 
     def score(self, X, y=None):
         """Opposite of the k-means objective on X (scikit-learn's definition)."""
-        if self.backend == 'sklearn':
-            return self.model.score(X, y)
         return self.model.score(X, y)
 
     def set_params(self, **params):

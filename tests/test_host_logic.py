@@ -117,6 +117,38 @@ def test_nonfinite_data_is_refused(model):
         m.fit(np.array([[0.0, np.nan], [1.0, 2.0]]))
 
 
+def test_without_a_device_the_estimator_raises_and_the_selector_uses_sklearn(monkeypatch):
+    """No device: the GPU estimator refuses to compute (no CPU stand-in for the engine);
+    the backend selector takes scikit-learn only when asked to (n_gpus=0 / backend)."""
+    monkeypatch.setattr("h2o4gpu_amd.util.gpu.device_count", lambda n_gpus=0: (0, 0))
+    X = np.random.default_rng(0).standard_normal((50, 3)).astype(np.float32)
+    m = km.KMeansH2O(n_clusters=2, init="random", random_state=1)
+    with pytest.raises(RuntimeError, match="usable GPU"):
+        m.fit(X)
+    m.cluster_centers_ = X[:2]
+    for call in (m.predict, m.transform, m.score):
+        with pytest.raises(RuntimeError, match="usable GPU"):
+            call(X)
+    with pytest.raises(RuntimeError, match="no usable GPU"):
+        km.KMeans(n_clusters=2)
+    sk = km.KMeans(n_clusters=2, n_gpus=0, random_state=1, n_init=1).fit(X)
+    assert sk.cluster_centers_.shape == (2, 3)
+
+
+def test_native_status_is_not_ignored(model):
+    """The reference drops the entry points' return value (kmeans.py:485-497); here a
+    non-zero status raises."""
+    m, lib = model
+    lib._fill = lambda name, args: -3
+    with pytest.raises(RuntimeError, match="status -3"):
+        m.fit(np.zeros((4, 2), np.float32))
+    m.cluster_centers_ = np.zeros((3, 2), np.float32)
+    with pytest.raises(RuntimeError, match="status -3"):
+        m.predict(np.zeros((4, 2), np.float32))
+    with pytest.raises(RuntimeError, match="status -3"):
+        m.transform(np.zeros((4, 2), np.float32))
+
+
 def test_swig_shim_conversions():
     from h2o4gpu_amd.libs import ch2o4gpu_gpu as shim
     p, keep = shim._in_array(np.empty([]), np.float32)          # 0-d array: converted, not NULL
