@@ -16,6 +16,15 @@ namespace kmhip {
 
 static constexpr int WG = 256;  // threads per workgroup (4 wavefronts)
 
+// Row stride (in values) of a block of rows staged in LDS for one-thread-per-row access.
+// Odd, so that thread t reading row t is conflict-free, and never 2^m - 1: with 31 or 63
+// the staged kernels ran 1.6x slower than with their neighbours (measured: d = 30, 31, 62, 63).
+__host__ __device__ static inline int staged_row_stride(int d) {
+  int sx = d | 1;
+  if (((sx + 1) & sx) == 0) sx += 2;
+  return sx;
+}
+
 // Squared norm of one centroid row, j ascending, multiply and add rounded separately:
 // the value row_norms / post_update would store (kmeans_labels.h:187-199). The fused
 // kernels call it when they are given no norm buffer, which spares the Lloyd loop a launch.
@@ -97,7 +106,7 @@ __global__ __launch_bounds__(WG) void assign_valu_kernel(
 // per-centroid accumulation in one pass over the data.
 //
 // Persistent workgroups walk over blocks of 256 rows. A block is fetched with
-// coalesced (16-byte where possible) loads into registers while the previous
+// coalesced 16-byte loads into registers while the previous
 // block is being processed, then written to LDS with an odd row stride so that
 // thread t reading row t is conflict-free. Every thread runs the same scalar
 // loop as assign_valu_kernel on its row (j ascending, multiply and add rounded
@@ -108,7 +117,8 @@ __global__ __launch_bounds__(WG) void assign_valu_kernel(
 // Sums and counts go to the workgroup's slot psums[blockIdx.x][k][d],
 // pcounts[blockIdx.x][k].
 // This is the HBM-bound regime: 2*k*d flop per row against d*s bytes.
-// FULL: d == DREG, no per-feature guards.
+// This kernel: d == DREG (4, 8, 16, 32 or 64), the row held in registers and the loops
+// over d unrolled; the data must be 16-byte aligned.
 // ---------------------------------------------------------------------------
 template <typename T, int VEC>
 struct BlockLoad {  // VEC is Mfma<T>::VW (one 16-byte load) or 1
@@ -118,21 +128,22 @@ template <typename T>
 struct BlockLoad<T, 1> {
   typedef T type;
 };
-template <typename T, int DREG, int VEC, bool FULL>
+template <typename T, int DREG>
 __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
     const T *__restrict__ X, const T *__restrict__ xnorm, const T *__restrict__ C,
     const T *__restrict__ cnorm, int *__restrict__ labels, T *__restrict__ mindist,
-    double *__restrict__ psums, int *__restrict__ pcounts, int64_t n, int dd, int k) {
+    double *__restrict__ psums, int *__restrict__ pcounts, int64_t n, int k) {
 #pragma clang fp contract(off)
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  const int d = FULL ? DREG : dd;
-  const int sx = d | 1;                                          // row stride of the staged block
+  constexpr int d = DREG;
+  constexpr int VEC = Mfma<T>::VW;
+  const int sx = staged_row_stride(d);                           // row stride of the staged block
   double *sums = reinterpret_cast<double *>(smem_raw);           // [k][sx]
   int *cnt = reinterpret_cast<int *>(sums + (size_t)k * sx);     // [k]
   T *ccs = reinterpret_cast<T *>(cnt + k + (k & 1));             // [k] centroid norms
   T *Xs = ccs + k + (k & 1);                                     // [WG][sx]
   typedef typename BlockLoad<T, VEC>::type ld_t;
-  constexpr int NLD = DREG / VEC;  // loads per thread and block (upper bound)
+  constexpr int NLD = DREG / VEC;  // loads per thread and block
   const int tid = threadIdx.x;
   for (int e = tid; e < k * sx; e += WG) sums[e] = 0.0;
   for (int c = tid; c < k; c += WG) cnt[c] = 0;
@@ -144,7 +155,6 @@ __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
     const int r = el / d;
     off[i] = r * sx + (el - r * d);
   }
-  const int nld = d / VEC;  // loads per thread for a full block (d % VEC == 0)
   ld_t pre[NLD];
   T pre_xx = 0;  // squared norm of this thread's row in the fetched block
   // Loads are never predicated: indices past the end of the data set are
@@ -156,7 +166,7 @@ __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
 #pragma unroll
     for (int i = 0; i < NLD; i++) {
       const int64_t e = tid + i * WG;
-      if (FULL || i < nld) pre[i] = src[e < last ? e : last];
+      pre[i] = src[e < last ? e : last];
     }
     const int64_t r = base + tid;
     pre_xx = xnorm[r < n ? r : n - 1];
@@ -172,15 +182,9 @@ __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
     const int rows = (int)min<int64_t>(WG, n - base);
     __syncthreads();  // the previous block has been consumed
 #pragma unroll
-    for (int i = 0; i < NLD; i++) {
-      if (FULL || i < nld) {  // rows past the end of a last, partial block hold clamped copies
-        if constexpr (VEC == 1) {
-          Xs[off[i]] = pre[i];
-        } else {
+    for (int i = 0; i < NLD; i++) {  // rows past the end of a last, partial block hold clamped copies
 #pragma unroll
-          for (int q = 0; q < VEC; q++) Xs[off[i] + q] = pre[i][q];
-        }
-      }
+      for (int q = 0; q < VEC; q++) Xs[off[i] + q] = pre[i][q];
     }
     const T xx = pre_xx;
     __syncthreads();
@@ -192,7 +196,7 @@ __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
       const T *xrow = Xs + tid * sx;
       T xr[DREG];
 #pragma unroll
-      for (int j = 0; j < DREG; j++) xr[j] = (FULL || j < d) ? xrow[j] : (T)0;
+      for (int j = 0; j < DREG; j++) xr[j] = xrow[j];
       T best = argmin_start<T>();
       int bidx = -1;
 #pragma unroll 2
@@ -200,8 +204,7 @@ __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
         const T *cp = C + (size_t)c * d;
         T dot = 0;
 #pragma unroll
-        for (int j = 0; j < DREG; j++)
-          if (FULL || j < d) dot = dot + xr[j] * cp[j];
+        for (int j = 0; j < DREG; j++) dot = dot + xr[j] * cp[j];
         const T t = xx + ccs[c];
         const T dist = fabs(t - (T)2 * dot);
         if (dist < best) {
@@ -230,6 +233,189 @@ __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
   for (int e = tid; e < k * d; e += WG) {
     const int c = e / d, j = e - c * d;
     dst[e] = sums[(size_t)c * sx + j];
+  }
+  int *cdst = pcounts + (size_t)blockIdx.x * k;
+  for (int c = tid; c < k; c += WG) cdst[c] = cnt[c];
+}
+
+// ---------------------------------------------------------------------------
+// The same Lloyd step for a feature count that is not one of the register sizes
+// above. Two things differ.
+// Loop order: features outside, centroids inside, one running dot product per
+// centroid in registers (KREG of them), the row read from its staged copy in LDS
+// one value at a time and the centroid values, whose addresses are
+// wavefront-uniform, through the scalar path. Nothing is unrolled over d, so no
+// guard sits in the inner loop; every dot product still adds its terms with j
+// ascending, multiply and add rounded separately.
+// Staging: a block of 256 rows is one contiguous run of 256*d values that starts
+// on a 16-byte boundary whatever d is, so it is fetched as a flat array of
+// 16-byte vectors (VEC values each); a vector may straddle two rows, which only
+// matters for the LDS offset of its values. The last, partial block of the data
+// set is fetched value by value.
+// DMAX bounds d (it sizes the register prefetch of the next block); d >= VEC.
+// ---------------------------------------------------------------------------
+template <typename T, int DMAX, int VEC, int KREG>
+__global__ __launch_bounds__(WG) void lloyd_valu_anyd_kernel(
+    const T *__restrict__ X, const T *__restrict__ xnorm, const T *__restrict__ C,
+    const T *__restrict__ cnorm, int *__restrict__ labels, T *__restrict__ mindist,
+    double *__restrict__ psums, int *__restrict__ pcounts, int64_t n, int d, int k) {
+#pragma clang fp contract(off)
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  const int sx = staged_row_stride(d);
+  const int pad = sx - d;                                        // 0 or 1
+  double *sums = reinterpret_cast<double *>(smem_raw);           // [k][sx]
+  int *cnt = reinterpret_cast<int *>(sums + (size_t)k * sx);     // [k]
+  T *ccs = reinterpret_cast<T *>(cnt + k + (k & 1));             // [k]
+  T *Xs = ccs + k + (k & 1);                                     // [WG][sx]
+  typedef typename BlockLoad<T, VEC>::type ld_t;
+  constexpr int NLD = (DMAX + VEC - 1) / VEC;
+  const int tid = threadIdx.x;
+  for (int e = tid; e < k * sx; e += WG) sums[e] = 0.0;
+  for (int c = tid; c < k; c += WG) cnt[c] = 0;
+  const int nld = (d + VEC - 1) / VEC;  // loads per thread and block
+  const int nvec = WG / VEC * d;        // vectors in a full block
+  // el / d for el < 256 * 64 and d >= 2 as one multiply-high (exact while el * d < 2^32)
+  const unsigned dinv = d > 1 ? 0xFFFFFFFFu / (unsigned)d + 1u : 0u;
+  auto row_of = [&](int el) -> int { return d > 1 ? (int)__umulhi((unsigned)el, dinv) : el; };
+  ld_t pre[NLD];
+  T pre_xx = 0, pre_tail = 0;
+  // Complete vectors of the block that starts at row `base`: all of them, except in the
+  // last, partial block of the data set, whose final values may not fill a vector.
+  auto block_vectors = [&](int64_t base) -> int {
+    const int64_t left = n - base;
+    return left >= WG ? nvec : (int)(left * d / VEC);
+  };
+  // Loads are never predicated per lane (indices are clamped instead), so the fetched
+  // block stays in flight across the processing of the current one. The one exception
+  // is the handful of values behind the last complete vector of the data set.
+  auto fetch = [&](int64_t base) {
+    const int vlim = block_vectors(base);  // >= 1: d >= VEC
+    const T *xb = X + base * (int64_t)d;
+    const ld_t *src = reinterpret_cast<const ld_t *>(xb);
+#pragma unroll
+    for (int i = 0; i < NLD; i++) {
+      const int e = tid + i * WG;
+      if (i < nld) pre[i] = src[e < vlim ? e : vlim - 1];
+    }
+    if (VEC > 1 && vlim < nvec) {
+      const int64_t el = (int64_t)vlim * VEC + tid;
+      if (tid < VEC && el < (n - base) * d) pre_tail = xb[el];
+    }
+    const int64_t r = base + tid;
+    pre_xx = xnorm[r < n ? r : n - 1];
+  };
+  const int64_t stride = (int64_t)gridDim.x * WG;
+  int64_t base = (int64_t)blockIdx.x * WG;
+  if (base >= n) return;  // the grid never exceeds the number of blocks
+  fetch(base);
+  // centroid norms while the first block travels (visible after the barrier below)
+  for (int c = tid; c < k; c += WG) ccs[c] = cnorm ? cnorm[c] : row_sqnorm<T>(C + (size_t)c * d, d);
+  // entry c of the register set reads centroid min(c, k-1): in bounds, unused past k
+  int coff[KREG];
+#pragma unroll
+  for (int c = 0; c < KREG; c++) coff[c] = (c < k ? c : k - 1) * d;
+  const int jrot = (tid & 63) % d;
+  for (; base < n; base += stride) {
+    const int rows = (int)min<int64_t>(WG, n - base);
+    __syncthreads();  // the previous block has been consumed
+    const int vlim = block_vectors(base);
+    // Value el of the block lives at LDS offset el + (el / d) * pad. The offsets are
+    // recomputed for every block from a copy of the thread index the optimiser cannot see
+    // through: hoisted out of the loop they would occupy a register per staged value.
+    int tv = tid;
+    asm volatile("" : "+v"(tv));
+    if (VEC == 1 || pad == 0 || d % VEC == 0) {  // no vector is split by padding slots
+#pragma unroll
+      for (int i = 0; i < NLD; i++) {
+        const int e = tv + i * WG;
+        if (i < nld && e < vlim) {
+          const int el = e * VEC;
+          const int off = el + row_of(el) * pad;
+          if constexpr (VEC == 1) {
+            Xs[off] = pre[i];
+          } else {
+#pragma unroll
+            for (int q = 0; q < VEC; q++) Xs[off + q] = pre[i][q];
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NLD; i++) {
+        const int e = tv + i * WG;
+        if (i < nld && e < vlim) {
+          if constexpr (VEC > 1) {
+            const int el = e * VEC;
+            const int r = row_of(el);
+            const int off = el + r * pad;
+            const int inrow = (r + 1) * d - el;  // values of this vector in its first row
+#pragma unroll
+            for (int q = 0; q < VEC; q++) Xs[off + q + (q >= inrow ? pad : 0)] = pre[i][q];
+          }
+        }
+      }
+    }
+    if (VEC > 1 && vlim < nvec) {  // values behind the last complete vector of the data set
+      const int el = vlim * VEC + tid;
+      if (tid < VEC && el < rows * d) Xs[el + row_of(el) * pad] = pre_tail;
+    }
+    const T xx = pre_xx;
+    __syncthreads();
+    fetch(base + stride < n ? base + stride : base);
+    const int64_t row = base + tid;
+    if (tid < rows) {
+      const T *xrow = Xs + tid * sx;
+      T dot[KREG];
+#pragma unroll
+      for (int c = 0; c < KREG; c++) dot[c] = 0;
+      int j = 0;
+      for (; j + 4 <= d; j += 4) {
+        const T x0 = xrow[j], x1 = xrow[j + 1], x2 = xrow[j + 2], x3 = xrow[j + 3];
+#pragma unroll
+        for (int c = 0; c < KREG; c++) {
+          const T *cp = C + coff[c] + j;
+          dot[c] = dot[c] + x0 * cp[0];
+          dot[c] = dot[c] + x1 * cp[1];
+          dot[c] = dot[c] + x2 * cp[2];
+          dot[c] = dot[c] + x3 * cp[3];
+        }
+      }
+      for (; j < d; j++) {
+        const T x0 = xrow[j];
+#pragma unroll
+        for (int c = 0; c < KREG; c++) dot[c] = dot[c] + x0 * C[coff[c] + j];
+      }
+      T best = argmin_start<T>();
+      int bidx = -1;
+#pragma unroll
+      for (int c = 0; c < KREG; c++) {
+        if (c < k) {
+          const T t = xx + ccs[c];
+          const T dist = fabs(t - (T)2 * dot[c]);
+          if (dist < best) {
+            best = dist;
+            bidx = c;
+          }
+        }
+      }
+      labels[row] = bidx;
+      if (mindist) mindist[row] = best;
+      if (bidx >= 0) {
+        double *srow = sums + (size_t)bidx * sx;
+        int jj = jrot;  // rotated start, as in lloyd_valu_fused_kernel
+        for (int q = 0; q < d; q++) {
+          unsafeAtomicAdd(srow + jj, (double)xrow[jj]);
+          jj = (jj + 1 == d) ? 0 : jj + 1;
+        }
+        atomicAdd(&cnt[bidx], 1);
+      }
+    }
+  }
+  __syncthreads();
+  double *dst = psums + (size_t)blockIdx.x * k * d;
+  for (int e = tid; e < k * d; e += WG) {
+    const int c = e / d, jx = e - c * d;
+    dst[e] = sums[(size_t)c * sx + jx];
   }
   int *cdst = pcounts + (size_t)blockIdx.x * k;
   for (int c = tid; c < k; c += WG) cdst[c] = cnt[c];
@@ -1094,12 +1280,12 @@ struct RowstatDispatch<double, FUSE> {
 static bool valu_fused_applies(int d, int k) { return k <= 16 && d <= 64; }
 template <typename T>
 static size_t valu_fused_lds(int d, int k) {
-  const int sx = d | 1;
+  const int sx = staged_row_stride(d);
   return (size_t)k * sx * sizeof(double) + ((size_t)k + 1) * sizeof(int) +
          ((size_t)k + 1) * sizeof(T) + (size_t)WG * sx * sizeof(T) + 16;
 }
 static int valu_fused_grid(int64_t n, size_t lds, int num_cu) {
-  int per_cu = (int)((150 * 1024) / lds);
+  int per_cu = (int)((160 * 1024) / lds);  // a CU has 160 KB of LDS
   if (per_cu > 8) per_cu = 8;
   if (per_cu < 1) per_cu = 1;
   int64_t grid = (int64_t)num_cu * per_cu;
@@ -1129,29 +1315,52 @@ static int launch_valu_fused(hipStream_t s, const T *X, const T *xnorm, const T 
   const int grid = valu_fused_grid(n, lds, num_cu);
   if (slots) *slots = grid;
   const int vw = Mfma<T>::VW;
-  const bool vec = (d % vw == 0) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0);
-#define KM_VF_LAUNCH(DREG, VEC, FULL)                                                       \
-  do {                                                                                      \
-    auto kern = lloyd_valu_fused_kernel<T, DREG, VEC, FULL>;                                \
-    if (lds > 64 * 1024)                                                                    \
-      KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                  \
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(WG), lds, s, X, xnorm, C, cnorm, labels,      \
-                       mindist, psums, pcounts, n, d, k);                                   \
+  const bool aligned = (reinterpret_cast<uintptr_t>(X) & 15) == 0;
+#define KM_VF_SETUP(kern)                                                                  \
+  if (lds > 64 * 1024)                                                                     \
+  KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                     \
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
+  // d is one of the register sizes: the row lives in registers
+#define KM_VF(DREG)                                                                        \
+  do {                                                                                     \
+    auto kern = lloyd_valu_fused_kernel<T, DREG>;                                          \
+    KM_VF_SETUP(kern);                                                                     \
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(WG), lds, s, X, xnorm, C, cnorm, labels,     \
+                       mindist, psums, pcounts, n, k);                                     \
   } while (0)
-#define KM_VF(DREG)                                            \
-  do {                                                         \
-    if (vec && d == DREG) KM_VF_LAUNCH(DREG, Mfma<T>::VW, true); \
-    else if (vec) KM_VF_LAUNCH(DREG, Mfma<T>::VW, false);      \
-    else KM_VF_LAUNCH(DREG, 1, false);                         \
+  // any other d: dot products in registers, KREG >= k of them
+#define KM_VA_LAUNCH(DMAX, VEC, KREG)                                                      \
+  do {                                                                                     \
+    auto kern = lloyd_valu_anyd_kernel<T, DMAX, VEC, KREG>;                                \
+    KM_VF_SETUP(kern);                                                                     \
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(WG), lds, s, X, xnorm, C, cnorm, labels,     \
+                       mindist, psums, pcounts, n, d, k);                                  \
   } while (0)
-  if (d <= 4) KM_VF(4);
-  else if (d <= 8) KM_VF(8);
-  else if (d <= 16) KM_VF(16);
-  else if (d <= 32) KM_VF(32);
-  else KM_VF(64);
-#undef KM_VF_LAUNCH
+#define KM_VA_K(DMAX, VEC)                       \
+  do {                                           \
+    if (k <= 4) KM_VA_LAUNCH(DMAX, VEC, 4);      \
+    else if (k <= 8) KM_VA_LAUNCH(DMAX, VEC, 8); \
+    else KM_VA_LAUNCH(DMAX, VEC, 16);            \
+  } while (0)
+#define KM_VA(DMAX)                                         \
+  do {                                                      \
+    if (aligned && d >= vw) KM_VA_K(DMAX, Mfma<T>::VW);     \
+    else KM_VA_K(DMAX, 1);                                  \
+  } while (0)
+  if (aligned && d == 4) KM_VF(4);
+  else if (aligned && d == 8) KM_VF(8);
+  else if (aligned && d == 16) KM_VF(16);
+  else if (aligned && d == 32) KM_VF(32);
+  else if (aligned && d == 64) KM_VF(64);
+  else if (d <= 16) KM_VA(16);
+  else if (d <= 32) KM_VA(32);
+  else if (d <= 48) KM_VA(48);
+  else KM_VA(64);
+#undef KM_VA
+#undef KM_VA_K
+#undef KM_VA_LAUNCH
 #undef KM_VF
+#undef KM_VF_SETUP
   KM_HIP_TRY(hipGetLastError());
   return 0;
 }

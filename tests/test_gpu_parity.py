@@ -182,7 +182,13 @@ def test_fused_step_equals_separate_kernels(hip, oracle, n, d, k, dtype):
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("n,d,k", [(100000, 16, 8), (5001, 3, 2), (777, 64, 16), (3000, 33, 11), (256, 8, 1),
-                                   (40000, 4, 16), (30001, 8, 7), (9000, 2, 4), (5000, 6, 3), (4000, 1, 2)])
+                                   (40000, 4, 16), (30001, 8, 7), (9000, 2, 4), (5000, 6, 3), (4000, 1, 2),
+                                   # feature counts between the register sizes: rows that straddle the
+                                   # 16-byte vectors of a block, padded and unpadded LDS rows, a last
+                                   # block whose values do not fill a vector
+                                   (5003, 30, 8), (777, 31, 5), (20001, 50, 16), (9001, 46, 3), (6000, 12, 9),
+                                   (4099, 63, 13), (2051, 62, 4), (12345, 20, 8), (1025, 5, 2), (300, 7, 16),
+                                   (255, 13, 6), (257, 15, 1), (100001, 24, 12)])
 def test_small_shape_fused_step_is_bit_exact(hip, oracle, n, d, k, dtype):
     """k <= 16 and d <= 64: the one-pass VALU step. Labels and minimum distances are
     bit-identical to the scalar CPU loop; float32 centroids are bit-identical to the

@@ -36,3 +36,7 @@ def test_device_tensors_give_the_results_of_host_arrays(hip):
         if exact:
             assert r[tag + "_transform_equal"] is True, r
     assert r["strided_refused"] and r["cpu_tensor_ok"]
+    assert len(r["unaligned"]) == 14
+    for case, (labels_equal, diff, predict_equal) in r["unaligned"].items():
+        # sums of float64 rows and of the tiled/bucketed float32 paths repeat to rounding only
+        assert labels_equal and predict_equal and diff <= 1e-6, (case, r["unaligned"][case])

@@ -44,6 +44,28 @@ def main():
             b = KMeans(n_clusters=k, init=init, max_iter=3, tol=0.0, random_state=11).fit(Xd)
             out["%s_%s_close" % (tag, init)] = bool(np.allclose(a.cluster_centers_, b.cluster_centers_,
                                                                 rtol=1e-12, atol=1e-12))
+    # device rows that start 4 or 8 bytes into an allocation (not 16-byte aligned): every
+    # kernel family must take its unaligned path and give the aligned result
+    unaligned = {}
+    for dtype in (np.float32, np.float64):
+        for (k, d, n) in ((8, 16, 20_011), (8, 30, 20_011), (5, 3, 9_001), (40, 32, 20_011),
+                          (200, 24, 20_011), (70, 100, 8_003), (3000, 8, 20_011)):
+            centers = rng.uniform(-30, 30, size=(k, d))
+            X = np.ascontiguousarray((centers[rng.integers(0, k, size=n)] +
+                                      rng.standard_normal((n, d))).astype(dtype))
+            C0 = (centers + 0.25).astype(dtype)
+            base = torch.empty(n * d + 1, dtype=torch.from_numpy(X).dtype, device="cuda:0")
+            Xd = base[1:].view(n, d)
+            Xd.copy_(torch.from_numpy(X))
+            assert Xd.data_ptr() % 16 != 0
+            host = KMeans(n_clusters=k, init=C0, max_iter=3, tol=0.0, random_state=3).fit(X)
+            dev = KMeans(n_clusters=k, init=C0, max_iter=3, tol=0.0, random_state=3).fit(Xd)
+            scale = float(np.abs(host.cluster_centers_).max())
+            diff = float(np.abs(host.cluster_centers_.astype(np.float64) - dev.cluster_centers_).max()) / scale
+            unaligned["%s k=%d d=%d" % (np.dtype(dtype).name, k, d)] = [
+                bool(np.array_equal(host.labels_, dev.labels_)), diff,
+                bool(np.array_equal(host.predict(X), dev.predict(Xd)))]
+    out["unaligned"] = unaligned
     # a non-contiguous view is refused, a CPU tensor goes the host way
     try:
         KMeans(n_clusters=2, init="random", max_iter=1).fit(Xd[:, ::2])
