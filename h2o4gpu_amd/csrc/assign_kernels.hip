@@ -39,6 +39,32 @@ __device__ __forceinline__ T row_sqnorm(const T *__restrict__ x, int d) {
   return acc;
 }
 
+// Features [j, j + VW) of a row of d >= VW values that is aligned to its elements only;
+// features at or past d come back as zero. The load never leaves the row: a vector that
+// would reach past the end is taken from the row's last VW values and shifted down. The
+// shift is skipped when no lane of the wavefront needs it.
+template <typename T>
+__device__ __forceinline__ typename Mfma<T>::vec_t load_row_vector(const T *__restrict__ row, int j,
+                                                                   int d) {
+  constexpr int VW = Mfma<T>::VW;
+  const int jc = min(j, d - VW);
+  const int s = j - jc;  // 0: the vector lies inside the row
+  const typename Mfma<T>::uvec_t v = *reinterpret_cast<const typename Mfma<T>::uvec_t *>(row + jc);
+  typename Mfma<T>::vec_t o;
+#pragma unroll
+  for (int e = 0; e < VW; e++) o[e] = v[e];
+  if (__builtin_amdgcn_ballot_w64(s != 0) != 0) {
+#pragma unroll
+    for (int e = 0; e < VW; e++) {
+      T x = 0;
+#pragma unroll
+      for (int t = e; t < VW; t++) x = (s == t - e) ? v[t] : x;
+      o[e] = x;
+    }
+  }
+  return o;
+}
+
 // ---------------------------------------------------------------------------
 // VALU variant: one thread per row, a chunk of centroids broadcast from LDS.
 // Arithmetic order is j ascending with separate multiply and add, so this
@@ -452,11 +478,11 @@ __device__ __forceinline__ int key_row(unsigned v, int g) {
 // different banks) and writes them to its own slot psums[blockIdx.x][k][d],
 // pcounts[blockIdx.x][k] when it has walked all its row tiles: the centroid
 // update then needs no second pass over the data.
-// LOAD: how a lane fetches its feature slice of a data row. 1: d == DP, 16-byte loads of
-// the slice as it lies in memory. 2: d < DP but d a multiple of the vector width: 16-byte
-// loads, a vector that would start at or past feature d re-reads the row's last valid
-// vector instead (finite x * 0 from the zero-padded centroid side adds nothing, and the
-// padded columns of the fused sums are never written back). 0: scalar loads, zero padded.
+// LOAD: how a lane fetches its feature slice of a data row. 1: d == DP and 16-byte aligned
+// data: 16-byte loads of the slice as it lies in memory. 2: any d >= the vector width, data
+// aligned to its elements: 16-byte loads that stay inside the row (padded features are
+// zero, or finite values meeting zeros on the centroid side).
+// 0: d below the vector width: scalar loads, zero padded.
 template <typename T, int DP, int ROWT, int LOAD, bool FUSE, int NW>
 __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
     const T *__restrict__ X, const T *__restrict__ xnorm,
@@ -582,7 +608,18 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
         const T *src = X + row * (int64_t)d;
 #pragma unroll
         for (int q = 0; q < NV; q++) {
-          const vec_t v = *reinterpret_cast<const vec_t *>(src + min(g * DCH + q * VW, d - VW));
+          const int f0 = g * DCH + q * VW;
+          vec_t v;
+          if (d % VW == 0) {
+            // no vector straddles the end of the row: one that lies past it re-reads the
+            // row's last vector (finite x * 0 from the zero-padded centroid side adds
+            // nothing, and the padded columns of the fused sums are never written back)
+            const typename M::uvec_t u = *reinterpret_cast<const typename M::uvec_t *>(src + min(f0, d - VW));
+#pragma unroll
+            for (int e = 0; e < VW; e++) v[e] = u[e];
+          } else {
+            v = load_row_vector<T>(src, f0, d);
+          }
 #pragma unroll
           for (int e = 0; e < VW; e++) xn[rt][q * VW + e] = v[e];
         }
@@ -782,8 +819,10 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
 // Preconditions (the engine's buffers satisfy them): C holds round_up(k, BC)
 // rows and cnorm round_up(k, BC) entries, the entries past k being +inf, so the
 // loads need no bounds test on the centroid axis; rows past n re-read row n-1.
-// A feature tail (d not a multiple of BK, DTAIL) re-reads in-bounds features on
-// the data side and zeroes the centroid side.
+// A feature tail (d not a multiple of BK, DTAIL) is zero on the centroid side (on both
+// sides when d is not a multiple of the vector width); its loads stay inside the operand
+// row (VECLOAD: 16-byte loads for any d >= the vector width, rows aligned to their
+// elements only).
 // ---------------------------------------------------------------------------
 // BCW = wavefronts along the centroid axis (2 or 4): the workgroup has 2*BCW
 // wavefronts and covers 64*BCW centroids. Data-row blocks are private to a
@@ -824,6 +863,7 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
   constexpr int B_VECS = BR / ROWS_PER_PASS;
   typedef typename M::acc_t acc_t;
   typedef typename M::vec_t vec_t;
+  typedef typename M::uvec_t uvec_t;
 
   extern __shared__ __align__(16) unsigned char smem_raw[];
   T *As = reinterpret_cast<T *>(smem_raw);  // [2][A_ELEMS]
@@ -887,39 +927,37 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
   // instance of the loader (tail_tag true) used for that step alone.
   auto gload = [&](int c0, int st, auto tail_tag) {
     constexpr bool TAILSTEP = DTAIL && decltype(tail_tag)::value;
-    int j = st * BK + jj;
-    bool jok = true;
-    if (TAILSTEP) {
-      jok = j < d;
-      j = VECLOAD ? min(j, d - VW) : j;
-    }
-    const T *cbase = C + (size_t)(c0 + rr0) * d;
-#pragma unroll
-    for (int q = 0; q < A_VECS; q++) {
-      const T *src = cbase + (size_t)q * ROWS_PER_PASS * d;
+    const int j = st * BK + jj;
+    // VECLOAD: 16-byte loads at element-aligned addresses; in the tail step through
+    // load_row_vector, which stays inside the row and returns zero past feature d
+    auto fetch = [&](const T *src, bool zero_past_d) -> vec_t {
       vec_t v;
       if (VECLOAD) {
-        v = *reinterpret_cast<const vec_t *>(src + j);
-        if (TAILSTEP && !jok)
+        if (TAILSTEP && d % VW == 0) {
+          // no vector straddles the end of the row: one past it re-reads the last one and
+          // is zeroed on the centroid side only (finite x * 0 adds nothing)
+          const uvec_t u = *reinterpret_cast<const uvec_t *>(src + min(j, d - VW));
 #pragma unroll
-          for (int e = 0; e < VW; e++) v[e] = 0;
+          for (int e = 0; e < VW; e++) v[e] = (zero_past_d && j >= d) ? (T)0 : u[e];
+        } else if (TAILSTEP) {
+          v = load_row_vector<T>(src, j, d);
+        } else {
+          const uvec_t u = *reinterpret_cast<const uvec_t *>(src + j);
+#pragma unroll
+          for (int e = 0; e < VW; e++) v[e] = u[e];
+        }
       } else {
 #pragma unroll
         for (int e = 0; e < VW; e++) v[e] = (j + e < d) ? src[min(j + e, d - 1)] : (T)0;
       }
-      areg[q] = v;  // scaled by -2 when it is stored to LDS, after this stage's matrix work
-    }
+      return v;
+    };
+    const T *cbase = C + (size_t)(c0 + rr0) * d;
 #pragma unroll
-    for (int q = 0; q < B_VECS; q++) {
-      vec_t v;
-      if (VECLOAD) {
-        v = *reinterpret_cast<const vec_t *>(xrow[q] + j);
-      } else {
+    for (int q = 0; q < A_VECS; q++)  // scaled by -2 when stored to LDS, after this stage's matrix work
+      areg[q] = fetch(cbase + (size_t)q * ROWS_PER_PASS * d, true);
 #pragma unroll
-        for (int e = 0; e < VW; e++) v[e] = xrow[q][min(j + e, d - 1)];
-      }
-      breg[q] = v;
-    }
+    for (int q = 0; q < B_VECS; q++) breg[q] = fetch(xrow[q], false);
   };
   auto lstore = [&](int buf) {
 #pragma unroll
@@ -1192,8 +1230,7 @@ static int launch_rowstat_nw(hipStream_t s, const T *X, const T *xnorm, const T 
   if (slots) *slots = (int)grid;
   const bool xal = (reinterpret_cast<uintptr_t>(X) & 15) == 0;
   const bool vec = (d == DP) && xal && ((reinterpret_cast<uintptr_t>(C) & 15) == 0);
-  const int vw = Mfma<T>::VW;
-  const bool padvec = !vec && xal && d >= vw && d % vw == 0;
+  const bool padvec = !vec && d >= Mfma<T>::VW;
 #define KM_RS_LAUNCH(LOAD)                                                                    \
   do {                                                                                        \
     auto kern = assign_rowstat_kernel<T, DP, ROWT, LOAD, FUSE, NW>;                           \
@@ -1390,9 +1427,7 @@ static int launch_tiled_bcw(hipStream_t s, const T *X, const T *xnorm, const T *
   const size_t lds = (size_t)2 * (Cfg::BC + Cfg::BR) * Cfg::BK * sizeof(T);
   const dim3 grid((unsigned)((n + Cfg::BR - 1) / Cfg::BR),
                   MODE == 1 ? (unsigned)((k + Cfg::BC - 1) / Cfg::BC) : 1u);
-  const int vw = Mfma<T>::VW;
-  const bool vec = (d % vw == 0) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0) &&
-                   ((reinterpret_cast<uintptr_t>(C) & 15) == 0);
+  const bool vec = d >= Mfma<T>::VW;  // 16-byte loads need element alignment only
   const bool tail = (d % Cfg::BK) != 0;
 #define KM_TILED(VEC, TAIL)                                                                  \
   do {                                                                                       \

@@ -27,6 +27,10 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef double doublex4 __attribute__((ext_vector_type(4)));
 typedef double doublex2 __attribute__((ext_vector_type(2)));
+// the same 16 bytes at an address that is only aligned to its elements (gfx950 serves such
+// loads with one instruction)
+typedef float floatx4_u __attribute__((ext_vector_type(4), aligned(4)));
+typedef double doublex2_u __attribute__((ext_vector_type(2), aligned(8)));
 
 template <typename T>
 struct Mfma;
@@ -39,6 +43,7 @@ struct Mfma<float> {
   static constexpr int VW = 4;  // elements in a 16-byte vector
   typedef floatx16 acc_t;
   typedef floatx4 vec_t;
+  typedef floatx4_u uvec_t;
   static __device__ __forceinline__ acc_t mma(float a, float b, acc_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
   }
@@ -56,6 +61,7 @@ struct Mfma<double> {
   static constexpr int VW = 2;
   typedef doublex4 acc_t;
   typedef doublex2 vec_t;
+  typedef doublex2_u uvec_t;
   static __device__ __forceinline__ acc_t mma(double a, double b, acc_t c) {
     return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
   }

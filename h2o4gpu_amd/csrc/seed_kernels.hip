@@ -15,8 +15,8 @@ namespace kmhip {
 static constexpr int WG = 256;
 
 template <typename T, int VEC>
-struct SeedVec {
-  typedef T type __attribute__((ext_vector_type(VEC)));
+struct SeedVec {  // 16 bytes of a row, aligned to the elements only
+  typedef T type __attribute__((ext_vector_type(VEC), aligned(sizeof(T))));
 };
 template <typename T>
 struct SeedVec<T, 1> {
@@ -106,16 +106,20 @@ __global__ __launch_bounds__(WG) void min_dist_update_kernel(
       dot[u] = 0;
     }
     for (int j = col * VEC; j < d; j += lpr * VEC) {
+      // a vector that would reach past the end of the row (d not a multiple of VEC) is
+      // fetched from the row's last VEC values; its elements below `first` belong to
+      // the neighbouring lane
+      const int jc = min(j, d - VEC), first = j - jc;
       vec_t v[U];
 #pragma unroll
-      for (int u = 0; u < U; u++) v[u] = *reinterpret_cast<const vec_t *>(x[u] + j);
+      for (int u = 0; u < U; u++) v[u] = *reinterpret_cast<const vec_t *>(x[u] + jc);
 #pragma unroll
       for (int u = 0; u < U; u++) {
         if constexpr (VEC == 1) {
           dot[u] += v[u] * cs[j];
         } else {
 #pragma unroll
-          for (int e = 0; e < VEC; e++) dot[u] += v[u][e] * cs[j + e];
+          for (int e = 0; e < VEC; e++) dot[u] += e >= first ? v[u][e] * cs[jc + e] : (T)0;
         }
       }
     }
@@ -158,8 +162,8 @@ int launch_min_dist_update(hipStream_t s, const T *X, const T *xnorm, int64_t ce
   hipLaunchKernelGGL((centre_dists_kernel<T>), dim3((unsigned)(t / (WG / 64) + 1)), dim3(WG), 0, s,
                      X, rows, t, (int)centre_row, dcc, d);
   constexpr int VW = 16 / sizeof(T);
-  const bool vec = d % VW == 0 && (reinterpret_cast<uintptr_t>(X) & 15) == 0;
-  const int per_row = vec ? d / VW : d;  // loads that cover a row
+  const bool vec = d >= VW;  // 16-byte loads need element alignment only
+  const int per_row = vec ? (d + VW - 1) / VW : d;  // loads that cover a row
   int lpr = 1;
   while (lpr < per_row && lpr < 64) lpr <<= 1;
   const unsigned blocks = (unsigned)((n + KPP_BLOCK - 1) / KPP_BLOCK);

@@ -113,11 +113,14 @@ int launch_row_norms(hipStream_t s, const T *X, T *out, int64_t n, int d) {
 // 64/LPR rows in flight. With a single centroid chunk every row matches and
 // the ballot is skipped.
 // ---------------------------------------------------------------------------
+// 2 or 4 consecutive row values as one load. The types are aligned to their elements
+// only: a row of d values starts wherever it starts, and gfx950 serves such a load with
+// one instruction.
 template <typename T, int VEC>
 struct VecOf;
-template <> struct VecOf<float, 4> { typedef float type __attribute__((ext_vector_type(4))); };
-template <> struct VecOf<float, 2> { typedef float type __attribute__((ext_vector_type(2))); };
-template <> struct VecOf<double, 2> { typedef double type __attribute__((ext_vector_type(2))); };
+template <> struct VecOf<float, 4> { typedef float type __attribute__((ext_vector_type(4), aligned(4))); };
+template <> struct VecOf<float, 2> { typedef float type __attribute__((ext_vector_type(2), aligned(4))); };
+template <> struct VecOf<double, 2> { typedef double type __attribute__((ext_vector_type(2), aligned(8))); };
 
 template <typename T, int VEC>
 struct RowVec {
@@ -131,27 +134,34 @@ template <typename T, int VEC>
 __device__ __forceinline__ typename RowVec<T, VEC>::type load_vec(const T *p) {
   return *reinterpret_cast<const typename RowVec<T, VEC>::type *>(p);
 }
-template <typename T, int VEC>
-__device__ __forceinline__ void lds_add_vec(double *dst, typename RowVec<T, VEC>::type v) {
+// adds elements first .. VEC-1 of v to dst[first .. VEC-1]
+template <typename T, int VEC, bool RAGGED>
+__device__ __forceinline__ void lds_add_vec(double *dst, typename RowVec<T, VEC>::type v, int first) {
   if constexpr (VEC == 1) {
     lds_add(dst, (double)v);
   } else {
 #pragma unroll
-    for (int e = 0; e < VEC; e++) lds_add(dst + e, (double)v[e]);
+    for (int e = 0; e < VEC; e++)
+      if (!RAGGED || e >= first) lds_add(dst + e, (double)v[e]);
   }
 }
 
-template <typename T, int VEC>
+// RAGGED: d is not a multiple of VEC (d >= VEC). The vector that would reach past the end
+// of the row is fetched from the row's last VEC values instead, and only the elements the
+// lane is responsible for (from `first` on) are added.
+template <typename T, int VEC, bool RAGGED>
 __device__ __forceinline__ void add_row_slice(double *srow, const T *xrow, int col,
                                               int lpr, int d) {
   // lanes col, col+lpr, ... each take VEC consecutive features
-  for (int j = col * VEC; j < d; j += lpr * VEC)
-    lds_add_vec<T, VEC>(srow + j, load_vec<T, VEC>(xrow + j));
+  for (int j = col * VEC; j < d; j += lpr * VEC) {
+    const int jc = RAGGED ? min(j, d - VEC) : j;
+    lds_add_vec<T, VEC, RAGGED>(srow + jc, load_vec<T, VEC>(xrow + jc), j - jc);
+  }
 }
 
 // sd = LDS row stride of the sums (>= d): chosen odd-ish by the host so that
 // rows of different centroids do not all start on the same bank.
-template <typename T, int VEC, int TPB>
+template <typename T, int VEC, bool RAGGED, int TPB>
 __global__ __launch_bounds__(TPB) void accumulate_kernel(
     const T *__restrict__ X, const int *__restrict__ labels,
     double *__restrict__ psums, int *__restrict__ pcounts, int64_t n, int d, int k,
@@ -184,6 +194,8 @@ __global__ __launch_bounds__(TPB) void accumulate_kernel(
     if (single_chunk && narrow) {
       // all loads of U row groups are issued before the first LDS add
       const bool has = col * VEC < d;
+      const int jc = RAGGED ? min(col * VEC, d - VEC) : col * VEC;  // see add_row_slice
+      const int first = col * VEC - jc;
       for (int b = 0; b < 64; b += rps * U) {
         typename RowVec<T, VEC>::type v[U];
         int l[U];
@@ -193,11 +205,11 @@ __global__ __launch_bounds__(TPB) void accumulate_kernel(
           l[u] = src < 64 ? __shfl(lab, src & 63, 64) : -1;
           const int64_t row = g0 + src;
           if (!(l[u] >= 0 && l[u] < nk && row < r1 && has)) l[u] = -1;
-          v[u] = load_vec<T, VEC>(X + (l[u] >= 0 ? row : r0) * (int64_t)d + (has ? col * VEC : 0));
+          v[u] = load_vec<T, VEC>(X + (l[u] >= 0 ? row : r0) * (int64_t)d + (has ? jc : 0));
         }
 #pragma unroll
         for (int u = 0; u < U; u++)
-          if (l[u] >= 0) lds_add_vec<T, VEC>(sums + (size_t)l[u] * sd + col * VEC, v[u]);
+          if (l[u] >= 0) lds_add_vec<T, VEC, RAGGED>(sums + (size_t)l[u] * sd + jc, v[u], first);
       }
     } else if (single_chunk) {
       for (int b = 0; b < 64; b += rps) {
@@ -205,7 +217,7 @@ __global__ __launch_bounds__(TPB) void accumulate_kernel(
         const int l = __shfl(lab, src, 64);
         const int64_t row = g0 + src;
         if (l >= 0 && l < nk && row < r1)
-          add_row_slice<T, VEC>(sums + (size_t)l * sd, X + row * (int64_t)d, col, lpr, d);
+          add_row_slice<T, VEC, RAGGED>(sums + (size_t)l * sd, X + row * (int64_t)d, col, lpr, d);
       }
     } else {
       unsigned long long mask = __ballot(match);
@@ -223,7 +235,7 @@ __global__ __launch_bounds__(TPB) void accumulate_kernel(
         const int l = __shfl(lab, src < 0 ? 0 : src, 64);
         if (src >= 0) {
           const int64_t row = g0 + src;
-          add_row_slice<T, VEC>(sums + (size_t)l * sd, X + row * (int64_t)d, col, lpr, d);
+          add_row_slice<T, VEC, RAGGED>(sums + (size_t)l * sd, X + row * (int64_t)d, col, lpr, d);
         }
       }
     }
@@ -261,9 +273,7 @@ UpdatePlan plan_update(int64_t n, int d, int k, int num_cu) {
   kc = (k + p.k_chunks - 1) / p.k_chunks;  // balanced chunks
   p.kc = kc;
   p.lds_bytes = (size_t)kc * per_centroid;
-  p.vec = 1;
-  if (sizeof(T) == 4 && d % 4 == 0) p.vec = 4;
-  else if (d % 2 == 0) p.vec = 2;
+  p.vec = sizeof(T) == 4 ? (d >= 4 ? 4 : (d >= 2 ? 2 : 1)) : (d >= 2 ? 2 : 1);  // see launch_accumulate
   // enough workgroups to cover the machine a few times, but bounded so the
   // partials buffer (row_blocks * k * d) stays small next to the data
   // (fewer when a workgroup's LDS image leaves room for only one or two per CU)
@@ -281,7 +291,7 @@ UpdatePlan plan_update(int64_t n, int d, int k, int num_cu) {
   return p;
 }
 
-template <typename T, int VEC>
+template <typename T, int VEC, bool RAGGED>
 static int launch_accumulate_vec(hipStream_t s, const UpdatePlan &p, const T *X,
                                  const int *labels, double *psums, int *pcounts,
                                  int64_t n, int d, int k) {
@@ -291,14 +301,14 @@ static int launch_accumulate_vec(hipStream_t s, const UpdatePlan &p, const T *X,
   while (lpr < groups && lpr < 64) lpr <<= 1;
   // a large LDS image means one workgroup per CU: make it 16 wavefronts
   if (p.lds_bytes > 64 * 1024) {
-    auto kern = accumulate_kernel<T, VEC, 1024>;
+    auto kern = accumulate_kernel<T, VEC, RAGGED, 1024>;
     KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                    hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)p.lds_bytes));
     hipLaunchKernelGGL(kern, dim3(p.row_blocks, p.k_chunks), dim3(1024), p.lds_bytes, s, X, labels,
                        psums, pcounts, n, d, k, p.kc, rows_per_block, lpr, p.sd);
   } else {
-    auto kern = accumulate_kernel<T, VEC, WG>;
+    auto kern = accumulate_kernel<T, VEC, RAGGED, WG>;
     hipLaunchKernelGGL(kern, dim3(p.row_blocks, p.k_chunks), dim3(WG), p.lds_bytes, s, X, labels,
                        psums, pcounts, n, d, k, p.kc, rows_per_block, lpr, p.sd);
   }
@@ -306,22 +316,25 @@ static int launch_accumulate_vec(hipStream_t s, const UpdatePlan &p, const T *X,
   return 0;
 }
 
+// Lanes take 16 bytes of a row each wherever a row holds that much (8 bytes for float rows
+// of 2 or 3 values); the rows need element alignment only.
 template <>
 int launch_accumulate<float>(hipStream_t s, const UpdatePlan &p, const float *X,
                              const int *labels, double *psums, int *pcounts,
                              int64_t n, int d, int k) {
-  const bool aligned = (reinterpret_cast<uintptr_t>(X) & 15) == 0;
-  if (p.vec == 4 && aligned) return launch_accumulate_vec<float, 4>(s, p, X, labels, psums, pcounts, n, d, k);
-  if (p.vec >= 2 && aligned && d % 2 == 0) return launch_accumulate_vec<float, 2>(s, p, X, labels, psums, pcounts, n, d, k);
-  return launch_accumulate_vec<float, 1>(s, p, X, labels, psums, pcounts, n, d, k);
+  if (d >= 4 && d % 4 == 0) return launch_accumulate_vec<float, 4, false>(s, p, X, labels, psums, pcounts, n, d, k);
+  if (d >= 4) return launch_accumulate_vec<float, 4, true>(s, p, X, labels, psums, pcounts, n, d, k);
+  if (d == 2) return launch_accumulate_vec<float, 2, false>(s, p, X, labels, psums, pcounts, n, d, k);
+  if (d == 3) return launch_accumulate_vec<float, 2, true>(s, p, X, labels, psums, pcounts, n, d, k);
+  return launch_accumulate_vec<float, 1, false>(s, p, X, labels, psums, pcounts, n, d, k);
 }
 template <>
 int launch_accumulate<double>(hipStream_t s, const UpdatePlan &p, const double *X,
                               const int *labels, double *psums, int *pcounts,
                               int64_t n, int d, int k) {
-  const bool aligned = (reinterpret_cast<uintptr_t>(X) & 15) == 0;
-  if (p.vec >= 2 && aligned) return launch_accumulate_vec<double, 2>(s, p, X, labels, psums, pcounts, n, d, k);
-  return launch_accumulate_vec<double, 1>(s, p, X, labels, psums, pcounts, n, d, k);
+  if (d >= 2 && d % 2 == 0) return launch_accumulate_vec<double, 2, false>(s, p, X, labels, psums, pcounts, n, d, k);
+  if (d >= 2) return launch_accumulate_vec<double, 2, true>(s, p, X, labels, psums, pcounts, n, d, k);
+  return launch_accumulate_vec<double, 1, false>(s, p, X, labels, psums, pcounts, n, d, k);
 }
 
 // ---------------------------------------------------------------------------
@@ -445,13 +458,25 @@ __global__ __launch_bounds__(WG) void segment_sum_kernel(
 #pragma unroll
       for (int e = 0; e < VEC; e++) acc[q][e] = 0.0;
     int cur = __shfl(my_lab, 0, 64);
+    // Lane slot q covers features [j, j + VEC). When d is not a multiple of VEC the last
+    // such vector would reach past the row: it is fetched from the row's last VEC values
+    // instead (offset jc) and only its elements from `first` on belong to this lane.
+    int jc[NVEC], first[NVEC];
+    bool active[NVEC];
+#pragma unroll
+    for (int q = 0; q < NVEC; q++) {
+      const int j = d0 + (q * 64 + lane) * VEC;
+      active[q] = j < d;
+      jc[q] = active[q] ? min(j, d - VEC) : 0;
+      first[q] = active[q] ? j - jc[q] : 0;
+    }
     auto flush = [&](int label) {
 #pragma unroll
       for (int q = 0; q < NVEC; q++) {
-        const int j = d0 + (q * 64 + lane) * VEC;
 #pragma unroll
         for (int e = 0; e < VEC; e++) {
-          if (j + e < d) unsafeAtomicAdd(gsum + (size_t)label * d + j + e, acc[q][e]);
+          if (active[q] && e >= first[q])
+            unsafeAtomicAdd(gsum + (size_t)label * d + jc[q] + e, acc[q][e]);
           acc[q][e] = 0.0;
         }
       }
@@ -467,11 +492,7 @@ __global__ __launch_bounds__(WG) void segment_sum_kernel(
         lab[u] = __shfl(my_lab, i, 64);
         const T *x = X + (int64_t)row * d;
 #pragma unroll
-        for (int q = 0; q < NVEC; q++) {
-          int j = d0 + (q * 64 + lane) * VEC;
-          if (j + VEC > d) j = 0;  // masked below
-          v[u][q] = load_vec<T, VEC>(x + j);
-        }
+        for (int q = 0; q < NVEC; q++) v[u][q] = load_vec<T, VEC>(x + jc[q]);  // inactive: masked below
       }
 #pragma unroll
       for (int u = 0; u < U; u++) {
@@ -482,8 +503,7 @@ __global__ __launch_bounds__(WG) void segment_sum_kernel(
         }
 #pragma unroll
         for (int q = 0; q < NVEC; q++) {
-          const int j = d0 + (q * 64 + lane) * VEC;
-          if (j + VEC <= d) {
+          if (active[q]) {
             if constexpr (VEC == 1) {
               acc[q][0] += (double)v[u][q];
             } else {
@@ -530,12 +550,12 @@ int launch_bucketed_accumulate(hipStream_t s, const T *X, const int *labels, int
   // shorter than n: the grid covers n positions and every wavefront bounds itself by
   // the device-side total
   const unsigned sblocks = (unsigned)((n + 255) / 256);
-  const bool aligned = (reinterpret_cast<uintptr_t>(X) & 15) == 0;
+  // 16-byte loads for any d that holds a whole vector (rows need element alignment only)
 #define KM_SEG(VEC, NVEC)                                                                   \
   hipLaunchKernelGGL((segment_sum_kernel<T, VEC, NVEC>), dim3(sblocks), dim3(WG), 0, s, X, \
                      order, order_label, gsum, total, d)
   if constexpr (sizeof(T) == 4) {
-    if (d % 4 == 0 && aligned) {
+    if (d >= 4) {
       if (d <= 256) KM_SEG(4, 1);
       else if (d <= 512) KM_SEG(4, 2);
       else KM_SEG(4, 4);
@@ -543,7 +563,7 @@ int launch_bucketed_accumulate(hipStream_t s, const T *X, const int *labels, int
       KM_SEG(1, 4);
     }
   } else {
-    if (d % 2 == 0 && aligned) {
+    if (d >= 2) {
       if (d <= 128) KM_SEG(2, 1);
       else if (d <= 256) KM_SEG(2, 2);
       else KM_SEG(2, 4);

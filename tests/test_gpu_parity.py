@@ -22,6 +22,8 @@ ASSIGN_CASES = [
     (1000, 16, 8), (777, 5, 3), (4096, 32, 256), (5000, 32, 100), (3001, 64, 64),
     (2000, 24, 33), (1500, 128, 40), (2500, 100, 70), (1200, 256, 130), (900, 300, 257),
     (64, 8, 64), (1, 4, 1), (130, 2, 2), (3000, 40, 600), (2100, 66, 1030),
+    # rows that are not a whole number of 16-byte vectors
+    (1800, 255, 140), (1300, 101, 300), (900, 30, 70), (1100, 127, 1030), (700, 9, 40), (513, 63, 20),
 ]
 
 
@@ -62,7 +64,8 @@ def test_assign_matches_oracle(hip, oracle, n, d, k, variant, dtype):
 @pytest.mark.parametrize("buckets", [1, 0])
 @pytest.mark.parametrize("n,d,k", [(5000, 32, 256), (3000, 16, 8), (2000, 7, 5), (4000, 256, 300),
                                    (1000, 784, 130), (70000, 64, 64), (300, 3, 300), (9000, 1100, 70),
-                                   (5000, 130, 90), (6000, 51, 700), (3000, 256, 700), (9000, 40, 5000)])
+                                   (5000, 130, 90), (6000, 51, 700), (3000, 256, 700), (9000, 40, 5000),
+                                   (4000, 301, 50), (3000, 101, 2000), (2000, 1101, 60), (2500, 5, 40)])
 def test_update_matches_oracle(hip, oracle, n, d, k, buckets, dtype):
     X = blobs(n, d, k, dtype, seed=7 * n + k)
     C = np.ascontiguousarray(X[RNG.choice(n, size=k, replace=False)])
@@ -271,7 +274,8 @@ def test_transform_matches_oracle(hip, oracle, n, d, k, dtype):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
-@pytest.mark.parametrize("n,d,k,seed", [(5000, 6, 12, 3), (20000, 32, 40, 11), (3000, 100, 25, 5), (1500, 3, 7, 0)])
+@pytest.mark.parametrize("n,d,k,seed", [(5000, 6, 12, 3), (20000, 32, 40, 11), (3000, 100, 25, 5), (1500, 3, 7, 0),
+                                        (4000, 101, 20, 2), (2500, 7, 9, 4)])
 def test_kmeanspp_seeding(hip, oracle, n, d, k, seed, dtype):
     """k-means++ on the device: same draw rule as the CPU restatement (same generator
     calls, same fixed-tree block sums), so the chosen rows agree; the minimum distances
