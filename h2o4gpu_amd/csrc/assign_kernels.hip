@@ -500,7 +500,7 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
   constexpr bool VECLOAD = LOAD == 1;
 
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  T *Cs = reinterpret_cast<T *>(smem_raw);  // [KT][NV][64][VW]
+  T *Cs = reinterpret_cast<T *>(smem_raw);  // [KT][NV][64][VW], see cs_slot
   T *ccs = Cs + (size_t)kp * DP;            // [kp]
   constexpr int SD = DP + 1;
   // (FUSE) sums in double: ds_add_f64 is the fast LDS floating-point atomic on gfx950
@@ -513,6 +513,15 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
   const int r = lane % MT;
   const int g = lane / MT;
   const int KT = kp / MT;
+  // Feature j lies in 16-byte vector j / VW of its row, and the vectors are dealt to the
+  // KL lane groups in turn: vector v belongs to lane group v % KL and is that group's
+  // step v / KL. A row of d < DP features thus fills the first nq steps of every lane
+  // group; the steps after them hold nothing and are skipped, matrix work included.
+  const int nq = LOAD == 1 ? NV : ((d + VW - 1) / VW + KL - 1) / KL;
+  auto cs_slot = [&](int c, int j) -> size_t {  // place of centroid c, feature j in Cs
+    const int t = c / MT, i = c - t * MT, v = j / VW;
+    return ((size_t)(t * NV + v / KL) * 64 + (v % KL) * MT + i) * VW + (j - v * VW);
+  };
 
   if (FUSE) {
     for (int e = tid; e < k * SD; e += TPB) sums[e] = 0.0;
@@ -536,26 +545,23 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
         const int e = e0 + u * TPB;
         if (e < nvec) {
           const int c = e / VPR, j = (e - c * VPR) * VW;
-          const int t = c / MT, i = c - t * MT, gg = j / DCH, s = j - gg * DCH;
-          reinterpret_cast<vec_t *>(Cs)[(size_t)(t * NV + s / VW) * 64 + gg * MT + i] = v[u] * (T)-2;
+          reinterpret_cast<vec_t *>(Cs)[cs_slot(c, j) / VW] = v[u] * (T)-2;
         }
       }
     }
     // centroid rows k .. kp-1 of the last tile: zeros
     for (int e = k * VPR + tid; e < kp * VPR; e += TPB) {
       const int c = e / VPR, j = (e - c * VPR) * VW;
-      const int t = c / MT, i = c - t * MT, gg = j / DCH, s = j - gg * DCH;
       vec_t z;
 #pragma unroll
       for (int q = 0; q < VW; q++) z[q] = 0;
-      reinterpret_cast<vec_t *>(Cs)[(size_t)(t * NV + s / VW) * 64 + gg * MT + i] = z;
+      reinterpret_cast<vec_t *>(Cs)[cs_slot(c, j) / VW] = z;
     }
   } else {
     for (int e = tid; e < kp * DP; e += TPB) {
       const int c = e / DP, j = e - c * DP;
       const T v = (c < k && j < d) ? (T)-2 * C[(size_t)c * d + j] : (T)0;
-      const int t = c / MT, i = c - t * MT, gg = j / DCH, s = j - gg * DCH;
-      Cs[((size_t)(t * NV + s / VW) * 64 + gg * MT + i) * VW + (s % VW)] = v;
+      Cs[cs_slot(c, j)] = v;
     }
   }
   for (int c = tid; c < kp; c += TPB) ccs[c] = (c < k && cnorm) ? cnorm[c] : pos_inf<T>();
@@ -566,11 +572,9 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
     // separately) is bit for bit what row_norms / post_update would have stored.
 #pragma clang fp contract(off)
     for (int c = tid; c < k; c += TPB) {
-      const int t = c / MT, i = c - t * MT;
       T acc = 0;
       for (int j = 0; j < d; j++) {
-        const int gg = j / DCH, sj = j - gg * DCH;
-        const T v = (T)-0.5 * Cs[((size_t)(t * NV + sj / VW) * 64 + gg * MT + i) * VW + (sj % VW)];
+        const T v = (T)-0.5 * Cs[cs_slot(c, j)];
         acc = acc + v * v;
       }
       ccs[c] = acc;
@@ -597,10 +601,10 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
       // rows past the end re-read the last row; their results are never stored
       const int64_t row = min(wrow0 + rt * MT + r, n - 1);
       if (VECLOAD) {
-        const vec_t *src = reinterpret_cast<const vec_t *>(X + row * (int64_t)DP + g * DCH);
+        const vec_t *src = reinterpret_cast<const vec_t *>(X + row * (int64_t)DP);
 #pragma unroll
         for (int q = 0; q < NV; q++) {
-          vec_t v = src[q];
+          vec_t v = src[q * KL + g];
 #pragma unroll
           for (int e = 0; e < VW; e++) xn[rt][q * VW + e] = v[e];
         }
@@ -608,7 +612,9 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
         const T *src = X + row * (int64_t)d;
 #pragma unroll
         for (int q = 0; q < NV; q++) {
-          const int f0 = g * DCH + q * VW;
+          // (steps from nq on are never used, but their loads are issued all the same,
+          // clamped into the row: a branch here would make every load wait for the last)
+          const int f0 = (q * KL + g) * VW;
           vec_t v;
           if (d % VW == 0) {
             // no vector straddles the end of the row: one that lies past it re-reads the
@@ -627,7 +633,7 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
         const T *src = X + row * (int64_t)d;
 #pragma unroll
         for (int s = 0; s < DCH; s++) {
-          const int j = g * DCH + s;
+          const int j = ((s / VW) * KL + g) * VW + s % VW;
           xn[rt][s] = j < d ? src[j] : (T)0;
         }
       }
@@ -682,12 +688,14 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
       const vec_t *ap = reinterpret_cast<const vec_t *>(Cs) + (size_t)t * NV * 64 + lane;
 #pragma unroll
       for (int q = 0; q < NV; q++) {
-        const vec_t a = ap[q * 64];
+        if (LOAD == 1 || q < nq) {  // (no early exit: the loop must unroll, x lives in registers)
+          const vec_t a = ap[q * 64];
 #pragma unroll
-        for (int e = 0; e < VW; e++) {
+          for (int e = 0; e < VW; e++) {
 #pragma unroll
-          for (int rt = 0; rt < ROWT; rt++)
-            acc[rt] = M::mma(a[e], x[rt][q * VW + e], acc[rt]);
+            for (int rt = 0; rt < ROWT; rt++)
+              acc[rt] = M::mma(a[e], x[rt][q * VW + e], acc[rt]);
+          }
         }
       }
     };
@@ -787,9 +795,17 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
         if (mindist) mindist[row] = bv;
       }
       if (FUSE && row < n && bidx[rt] >= 0) {
-        double *srow = sums + (size_t)bidx[rt] * SD + g * DCH;
+        double *srow = sums + (size_t)bidx[rt] * SD;
 #pragma unroll
-        for (int s = 0; s < DCH; s++) unsafeAtomicAdd(srow + s, (double)x[rt][s]);
+        for (int q = 0; q < NV; q++) {
+          if (LOAD == 1 || q < nq) {
+#pragma unroll
+            for (int e = 0; e < VW; e++) {
+              const int f = (q * KL + g) * VW + e;  // the feature this register holds
+              if (LOAD == 1 || f < d) unsafeAtomicAdd(srow + f, (double)x[rt][q * VW + e]);
+            }
+          }
+        }
         if (g == 0) atomicAdd(&cnt[bidx[rt]], 1);
       }
     }
@@ -879,6 +895,8 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
   const int g = lane / MT;
   const int64_t row0 = (int64_t)blockIdx.x * BR;
   const int nstage = (d + BK - 1) / BK;
+  // steps of the last stage that hold features: its ceil(rest / VW) vectors, KL per step
+  const int nq_tail = ((d - (nstage - 1) * BK + VW - 1) / VW + KL - 1) / KL;
 
   // staging role of this thread: operand row rr0 + q*ROWS_PER_PASS, features
   // [jj, jj+VW) of the stage. The 16-byte vector lands in LDS at tile rr/MT,
@@ -889,7 +907,10 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
 #pragma unroll
   for (int q = 0; q < (A_VECS > B_VECS ? A_VECS : B_VECS); q++) {
     const int rr = rr0 + q * ROWS_PER_PASS;
-    const int t = rr / MT, i = rr - t * MT, gg = jj / DCH, s = jj - gg * DCH;
+    // the stage's 16-byte vectors are dealt to the KL lane groups in turn (vector v:
+    // lane group v % KL, step v / KL), so a short last stage fills the first steps of
+    // every lane group and the steps after them can be skipped
+    const int t = rr / MT, i = rr - t * MT, gg = (jj / VW) % KL, s = (jj / VW) / KL * VW;
     // The 8 threads that stage one operand row write 8 different (vector, lane group)
     // combinations; unswizzled they land 1 KB apart, i.e. on the same banks. XOR-ing the
     // combination number into the low 3 bits of the lane slot spreads them over all
@@ -997,6 +1018,7 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
       const vec_t *bp = reinterpret_cast<const vec_t *>(Bs + buf * B_ELEMS);
 #pragma unroll
       for (int q = 0; q < NV; q++) {
+        if (DTAIL && st + 1 == nstage && q >= nq_tail) continue;  // nothing but zeros there
         vec_t a[CT], b[RT];
 #pragma unroll
         for (int ct = 0; ct < CT; ct++) a[ct] = ap[((wc * CT + ct) * NV + q) * 64 + rd_slot[q]];

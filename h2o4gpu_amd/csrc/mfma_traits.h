@@ -15,9 +15,11 @@
 //   v_mfma_f64_16x16x4_f64 : MT = 16, KL = 4 k-slices, 4 accumulators / lane,
 //       accumulator v of lane l is D[i = 4*v + l/16][j = l%16]
 // The k index a lane group contributes is free as long as A and B agree, so
-// lane group g is given the contiguous slice [g*DCH, (g+1)*DCH) of the feature
-// axis: a data row is then fetched with plain 16-byte loads and needs no
-// shuffle on its way into the matrix core.
+// the feature axis is cut into 16-byte vectors that are dealt to the KL lane
+// groups in turn (vector v: lane group v % KL, step v / KL): a data row is
+// fetched with plain 16-byte loads, needs no shuffle on its way into the matrix
+// core, and a row (or a last d-step) shorter than the padded width leaves whole
+// steps empty, which the kernels skip.
 #pragma once
 #include <hip/hip_runtime.h>
 
