@@ -152,10 +152,24 @@ __device__ __forceinline__ void lds_add_vec(double *dst, typename RowVec<T, VEC>
 template <typename T, int VEC, bool RAGGED>
 __device__ __forceinline__ void add_row_slice(double *srow, const T *xrow, int col,
                                               int lpr, int d) {
-  // lanes col, col+lpr, ... each take VEC consecutive features
-  for (int j = col * VEC; j < d; j += lpr * VEC) {
-    const int jc = RAGGED ? min(j, d - VEC) : j;
-    lds_add_vec<T, VEC, RAGGED>(srow + jc, load_vec<T, VEC>(xrow + jc), j - jc);
+  // lanes col, col+lpr, ... each take VEC consecutive features; four loads are issued
+  // before the first add (a load past the end of the row is clamped into it and unused;
+  // eight in flight measured slower: short rows then mostly fetch clamped duplicates)
+  constexpr int U = 4;
+  const int step = lpr * VEC;
+  for (int j0 = col * VEC; j0 < d; j0 += U * step) {
+    typename RowVec<T, VEC>::type v[U];
+    int jc[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      jc[u] = VEC > 1 ? min(j0 + u * step, d - VEC) : min(j0 + u * step, d - 1);
+      v[u] = load_vec<T, VEC>(xrow + jc[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const int j = j0 + u * step;
+      if (j < d) lds_add_vec<T, VEC, RAGGED>(srow + jc[u], v[u], j - jc[u]);
+    }
   }
 }
 
