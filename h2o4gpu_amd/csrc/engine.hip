@@ -336,6 +336,15 @@ struct StagingPool {
     w->done.wait(lock, [&] { return w->pending == 0; });
   }
 
+  // Transfers below MIN_STAGED go the plain way. Above it the pieces are a quarter of the
+  // transfer, at least 4 MB (what the copy threads need to be worth waking) and at most CHUNK.
+  static constexpr size_t MIN_STAGED = 24u << 20;
+  static size_t piece_size(size_t bytes) {
+    size_t p = (bytes / 4 + ((1u << 20) - 1)) & ~(size_t)((1u << 20) - 1);
+    if (p < (4u << 20)) p = 4u << 20;
+    return p > CHUNK ? CHUNK : p;
+  }
+
   // Pinned buffers and events of a device, created on first use (caller holds mu).
   bool ensure(int dev) {
     if (broken[dev]) return false;
@@ -353,16 +362,17 @@ struct StagingPool {
 
   // Returns 0 on success; a positive value means "staging unavailable, use a plain copy".
   int upload(int dev, hipStream_t stream, void *dst, const void *src, size_t bytes) {
-    if (dev < 0 || dev >= MAX_DEV || bytes < 4 * CHUNK) return 1;
+    if (dev < 0 || dev >= MAX_DEV || bytes < MIN_STAGED) return 1;
     std::lock_guard<std::mutex> lock(mu);
     if (!ensure(dev)) return 1;
     unsigned hw = std::thread::hardware_concurrency();
     const char *env = getenv("H2O4GPU_KMEANS_UPLOAD_THREADS");
     int threads = env ? atoi(env) : (int)std::min(8u, hw ? hw : 1u);
     if (threads < 1) threads = 1;
+    const size_t piece = piece_size(bytes);
     size_t off = 0;
     for (int i = 0; off < bytes; i ^= 1) {
-      const size_t len = std::min(CHUNK, bytes - off);
+      const size_t len = std::min(piece, bytes - off);
       KM_HIP_TRY(hipEventSynchronize(done[dev][i]));  // the DMA that last read this buffer
       parallel_copy(static_cast<char *>(buf[dev][i]), static_cast<const char *>(src) + off, len,
                     threads);
@@ -379,24 +389,25 @@ struct StagingPool {
 
   // The way back: the DMA engine fills one buffer while host threads copy the other out.
   int download(int dev, hipStream_t stream, void *dst, const void *src, size_t bytes) {
-    if (dev < 0 || dev >= MAX_DEV || bytes < 4 * CHUNK) return 1;
+    if (dev < 0 || dev >= MAX_DEV || bytes < MIN_STAGED) return 1;
     std::lock_guard<std::mutex> lock(mu);
     if (!ensure(dev)) return 1;
     unsigned hw = std::thread::hardware_concurrency();
     const char *env = getenv("H2O4GPU_KMEANS_UPLOAD_THREADS");
     int threads = env ? atoi(env) : (int)std::min(8u, hw ? hw : 1u);
     if (threads < 1) threads = 1;
-    const size_t chunks = (bytes + CHUNK - 1) / CHUNK;
+    const size_t piece = piece_size(bytes);
+    const size_t chunks = (bytes + piece - 1) / piece;
     for (size_t c = 0; c <= chunks; c++) {
       const int b = (int)(c & 1);
       if (c < chunks) {
-        const size_t off = c * CHUNK, len = std::min(CHUNK, bytes - off);
+        const size_t off = c * piece, len = std::min(piece, bytes - off);
         KM_HIP_TRY(hipMemcpyAsync(buf[dev][b], static_cast<const char *>(src) + off, len,
                                   hipMemcpyDeviceToHost, stream));
         KM_HIP_TRY(hipEventRecord(done[dev][b], stream));
       }
       if (c >= 1) {  // chunk c-1 sits in the other buffer
-        const size_t off = (c - 1) * CHUNK, len = std::min(CHUNK, bytes - off);
+        const size_t off = (c - 1) * piece, len = std::min(piece, bytes - off);
         KM_HIP_TRY(hipEventSynchronize(done[dev][b ^ 1]));
         parallel_copy(static_cast<char *>(dst) + off, static_cast<const char *>(buf[dev][b ^ 1]), len,
                       threads);
@@ -879,7 +890,7 @@ struct Engine : h2o4gpu_kmeans_handle {
   }
   int d2h(void *dst, const void *src, size_t bytes) {
     KM_HIP_TRY(hipSetDevice(dev));
-    KM_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, stream));
+    KM_TRY(download_rows(dev, stream, dst, src, bytes));  // staged when large (labels of 10M rows)
     KM_HIP_TRY(hipStreamSynchronize(stream));
     return 0;
   }
@@ -923,7 +934,7 @@ struct Engine : h2o4gpu_kmeans_handle {
     PROFILED("row_norms", launch_row_norms<T>(stream, dX, dxn, (int64_t)rows, d));
     PROFILED("assign", launch_assign<T>(stream, opt_assign, dX, dxn, C[cur], cnorm, dl, dmin,
                                         (int64_t)rows, d, k, num_cu, &last_variant));
-    KM_HIP_TRY(hipMemcpyAsync(out, dl, rows * sizeof(int), hipMemcpyDeviceToHost, stream));
+    KM_TRY(download_rows(dev, stream, out, dl, rows * sizeof(int)));
     KM_HIP_TRY(hipStreamSynchronize(stream));
     return 0;
   }
@@ -1254,6 +1265,46 @@ KM_API int h2o4gpu_kmeans_random_start_rows(int seed, size_t rows, int k, int *o
     return H2O4GPU_KMEANS_EARG;
   first_rows_of_shuffle((int64_t)rows, k, (unsigned)seed, out);
   return 0;
+}
+
+// 1 if every value is finite, 0 if one is an infinity or a NaN, negative on bad arguments.
+// Host memory, host threads: the estimator's input check (solvers/utils.py:144-158 in the
+// reference, two numpy passes with a temporary the size of the data) as one parallel pass.
+KM_API int h2o4gpu_kmeans_host_all_finite(const void *data, size_t count, int elem_size) {
+  if ((!data && count) || (elem_size != 4 && elem_size != 8)) return H2O4GPU_KMEANS_EARG;
+  unsigned hw = std::thread::hardware_concurrency();
+  int threads = (int)std::min(8u, hw ? hw : 1u);
+  if (count < (1u << 20)) threads = 1;
+  std::atomic<int> bad(0);
+  auto scan = [&](size_t lo, size_t hi) {
+    // a value is non-finite exactly when its exponent bits are all ones
+    constexpr size_t BLOCK = 1 << 16;
+    for (size_t b = lo; b < hi && !bad.load(std::memory_order_relaxed); b += BLOCK) {
+      const size_t e = std::min(hi, b + BLOCK);
+      unsigned long long any = 0;
+      if (elem_size == 4) {
+        const uint32_t *p = static_cast<const uint32_t *>(data);
+        for (size_t i = b; i < e; i++) any |= (p[i] & 0x7F800000u) == 0x7F800000u;
+      } else {
+        const uint64_t *p = static_cast<const uint64_t *>(data);
+        for (size_t i = b; i < e; i++) any |= (p[i] & 0x7FF0000000000000ull) == 0x7FF0000000000000ull;
+      }
+      if (any) bad.store(1, std::memory_order_relaxed);
+    }
+  };
+  std::vector<std::thread> pool;
+  const size_t per = (count + threads - 1) / threads;
+  try {
+    for (int t = 1; t < threads; t++)
+      if (per * t < count) pool.emplace_back(scan, per * t, std::min(count, per * (t + 1)));
+  } catch (...) {
+    for (auto &th : pool) th.join();
+    pool.clear();
+    scan(per, count);  // whatever the threads would have covered
+  }
+  scan(0, std::min(per, count));
+  for (auto &th : pool) th.join();
+  return bad.load() ? 0 : 1;
 }
 
 KM_API int h2o4gpu_kmeans_last_fit_info(double *inertia, int *iterations) {

@@ -79,6 +79,27 @@ def kmeans_transform_owned(verbose, gpu_id, n_gpu, m, n, k, srcdata, centroids, 
     return rc, _adopt(slot, int(m) * int(k) if rc == 0 else 0, dtype)
 
 
+def kmeans_fit_owned(verbose, seed, gpu_id, n_gpu, mTrain, n, k, max_iterations, init_from_data,
+                     threshold, srcdata, centroids, dtype):
+    """make_ptr_float/double_kmeans(dopredict=0, ...) without preallocated outputs: returns
+    (status, centroids [min(k, mTrain) * n], labels [mTrain]), both owning the library's
+    buffers. Not part of the reference's module; the estimator uses it to skip zero-filling
+    and copying the result arrays."""
+    dtype = np.dtype(dtype)
+    fn_name = "make_ptr_float_kmeans" if dtype == np.float32 else "make_ptr_double_kmeans"
+    lib = _k.lib()
+    src_p, _src_keep = _in_array(srcdata, dtype)
+    cen_p, _cen_keep = _in_array(centroids, dtype)
+    pc_slot, pl_slot = ctypes.c_void_p(), ctypes.c_void_p()
+    rc = getattr(lib, fn_name)(0, int(verbose), int(seed), int(gpu_id), int(n_gpu), int(mTrain), int(n),
+                               int(k), int(max_iterations), int(init_from_data), float(threshold), src_p,
+                               cen_p, ctypes.byref(pc_slot), ctypes.byref(pl_slot))
+    ok = rc == 0
+    k_eff = min(int(k), int(mTrain))
+    return rc, _adopt(pc_slot, k_eff * int(n) if ok else 0, dtype), \
+        _adopt(pl_slot, int(mTrain) if ok else 0, np.int32)
+
+
 def _make_ptr(fn_name, dtype, dopredict, verbose, seed, gpu_id, n_gpu, mTrain, n, k, max_iterations,
               init_from_data, threshold, srcdata, centroids, pred_centroids, pred_labels):
     lib = _k.lib()

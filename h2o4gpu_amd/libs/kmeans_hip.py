@@ -40,6 +40,7 @@ PROTOTYPES = {
     "cudaresetdevice_bare": (c_int, []),
     "h2o4gpu_kmeans_device_count": (c_int, []),
     "h2o4gpu_kmeans_last_fit_info": (c_int, [P(c_double), P(c_int)]),
+    "h2o4gpu_kmeans_host_all_finite": (c_int, [c_void_p, c_size_t, c_int]),
     "h2o4gpu_kmeans_random_start_rows": (c_int, [c_int, c_size_t, c_int, c_void_p]),
     "h2o4gpu_kmeans_create": (c_int, [P(c_void_p), c_int, c_size_t, c_size_t, c_int, c_int, c_int]),
     "h2o4gpu_kmeans_destroy": (c_int, [c_void_p]),
@@ -286,6 +287,16 @@ def random_start_rows(seed, rows, k):
     out = np.empty(k, np.int32)
     _check("random_start_rows", lib().h2o4gpu_kmeans_random_start_rows(int(seed), int(rows), int(k), _vp(out)))
     return out
+
+
+def host_all_finite(arr):
+    """True when every value of a C-contiguous float32/float64 host array is finite (one
+    parallel pass on host threads; no device is touched)."""
+    if arr.dtype not in (np.float32, np.float64) or not arr.flags.c_contiguous:
+        raise TypeError("host_all_finite wants a C-contiguous float32 or float64 array")
+    rc = lib().h2o4gpu_kmeans_host_all_finite(_vp(arr), int(arr.size), int(arr.itemsize))
+    _check("host_all_finite", min(rc, 0))
+    return rc == 1
 
 
 def last_fit_info():

@@ -69,9 +69,21 @@ def _device_rows(X):
 def _check_data_content(do_check, name, data):
     """Reference solvers/utils.py:144-158."""
     if do_check == 1 and np.size(data):
-        # same two assertions as the reference, from the extremes (a NaN propagates into
-        # both, an infinity into one of them): two passes and no boolean temporary the
-        # size of the data
+        # the library's parallel pass over the raw values where it can be used ...
+        if isinstance(data, np.ndarray) and data.dtype in (np.float32, np.float64) \
+                and data.flags.c_contiguous:
+            try:
+                from ..libs import kmeans_hip
+                finite = kmeans_hip.host_all_finite(data)
+            except Exception:  # no native library here: numpy below  # pylint: disable=broad-except
+                finite = None
+            if finite is not None:
+                # (the reference's first assertion fires for NaN as well as for infinities)
+                assert finite, "%s contains Inf" % name
+                return
+        # ... else the same two assertions as the reference, from the extremes (a NaN
+        # propagates into both, an infinity into one of them): two passes and no boolean
+        # temporary the size of the data
         lo, hi = np.min(data), np.max(data)
         assert np.isfinite(lo) and np.isfinite(hi), "%s contains Inf" % name
         assert not (np.isnan(lo) or np.isnan(hi)), "%s contains NA" % name
@@ -301,12 +313,22 @@ class KMeansH2O:
         # (kmeans.py:722-725). Restarts are pointless when the start is given.
         restarts = 1 if c_init == 2 else max(1, int(self.n_init or 1))
         best = None
+        owned = getattr(lib, "kmeans_fit_owned", None)
         for r in range(restarts):
-            pred_centers = np.zeros(cols * self._n_clusters, data.dtype)
-            pred_labels = np.zeros(rows, dtype=np.int32)
-            status = fn(0, self.verbose, self.random_state + r, self._gpu_id, self.n_gpus, rows,
-                        cols, self._n_clusters, self._max_iter, c_init, self.tol, c_data, centroids,
-                        pred_centers, pred_labels)
+            if owned is not None:  # adopt the library's buffers: no zero-fill, no copy
+                status, pred_centers, pred_labels = owned(
+                    self.verbose, self.random_state + r, self._gpu_id, self.n_gpus, rows, cols,
+                    self._n_clusters, self._max_iter, c_init, self.tol, c_data, centroids, data.dtype)
+                if status == 0 and pred_centers.size < cols * self._n_clusters:
+                    # more clusters asked for than rows: the library clamps k (kmeans_h2o4gpu.cu:630-635)
+                    pred_centers = np.concatenate([pred_centers, np.zeros(
+                        cols * self._n_clusters - pred_centers.size, data.dtype)])
+            else:
+                pred_centers = np.zeros(cols * self._n_clusters, data.dtype)
+                pred_labels = np.zeros(rows, dtype=np.int32)
+                status = fn(0, self.verbose, self.random_state + r, self._gpu_id, self.n_gpus, rows,
+                            cols, self._n_clusters, self._max_iter, c_init, self.tol, c_data, centroids,
+                            pred_centers, pred_labels)
             if status != 0:
                 raise RuntimeError("KMeans fit failed in the native library (status %d)" % status)
             # a module that offers only the reference's entry points has no such getter

@@ -80,6 +80,14 @@ int h2o4gpu_kmeans_random_start_rows(int seed, size_t rows, int k, int *out);
  * has no slot to return it. */
 int h2o4gpu_kmeans_last_fit_info(double *inertia, int *iterations);
 
+/* 1 when all `count` values of a host array (elem_size 4: float, 8: double) are
+ * finite, 0 when one is an infinity or a NaN, negative on bad arguments. Host
+ * threads only, no device is touched.
+ * Replaces, for the estimator: _check_data_content,
+ * src/interface_py/h2o4gpu/solvers/utils.py:144-158 (two numpy passes and a
+ * boolean temporary the size of the data). */
+int h2o4gpu_kmeans_host_all_finite(const void *data, size_t count, int elem_size);
+
 /* Squared distances |xx + cc - 2 x.c| of every row to every centroid, no
  * sqrt, centroid-major: (*preds)[c * m + i]. malloc()ed, caller owns.
  * Replaces: kmeans_transform<T>, src/gpu/kmeans/kmeans_h2o4gpu.cu:891-975. */

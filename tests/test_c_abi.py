@@ -83,3 +83,26 @@ def test_random_start_rows_equal_the_standard_library_shuffle(hip, oracle):
                 got = hip.random_start_rows(seed, n, k)
                 assert np.array_equal(got, want), (n, k, seed)
     assert hip.lib().h2o4gpu_kmeans_random_start_rows(1, 5, 6, None) == -2
+
+
+def test_host_all_finite_matches_numpy():
+    """The estimator's input check as one parallel pass over the raw values: same verdict
+    as np.isfinite(...).all() (reference solvers/utils.py:144-158), no device involved."""
+    from h2o4gpu_amd.libs import kmeans_hip
+    rng = np.random.default_rng(3)
+    for dt in (np.float32, np.float64):
+        a = rng.standard_normal(2_500_003).astype(dt)          # large enough for several threads
+        assert kmeans_hip.host_all_finite(a) is True
+        for pos in (0, 1, a.size // 3, a.size - 1):
+            for bad in (np.inf, -np.inf, np.nan):
+                b = a.copy()
+                b[pos] = bad
+                assert kmeans_hip.host_all_finite(b) is False
+        info = np.finfo(dt)
+        edge = np.array([info.max, -info.max, info.tiny, info.smallest_subnormal, 0.0, -0.0], dt)
+        assert kmeans_hip.host_all_finite(edge) is True
+        assert kmeans_hip.host_all_finite(np.zeros(0, dt)) is True
+    with pytest.raises(TypeError):
+        kmeans_hip.host_all_finite(np.zeros(4, np.int32))
+    with pytest.raises(TypeError):
+        kmeans_hip.host_all_finite(np.zeros((4, 4), np.float32)[:, ::2])
