@@ -675,9 +675,6 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
       bkey[rt] = 0x7F7FFFF0u;  // FLT_MAX with the index bits cleared
       btile[rt] = -1;
     }
-    // Two accumulator sets: the matrix-core work of centroid tile t is issued
-    // together with the argmin epilogue of tile t-1, so that one wavefront
-    // alone keeps both the MFMA pipe and the VALU busy.
     auto tile_mma = [&](acc_t (&acc)[ROWT], int t) {
 #pragma unroll
       for (int v = 0; v < NACC; v++) {
@@ -740,32 +737,13 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
         }
       }
     };
-#ifndef KM_PIPE
-#define KM_PIPE 0
-#endif
-    if (!KM_PIPE) {
-      for (int t = 0; t < KT; t++) {
-        acc_t acc[ROWT];
-        tile_mma(acc, t);
-        tile_argmin(acc, t);
-      }
-    } else {
-      acc_t accA[ROWT], accB[ROWT];
-      tile_mma(accA, 0);
-      int t = 1;
-      for (; t + 1 < KT; t += 2) {
-        tile_mma(accB, t);
-        tile_argmin(accA, t - 1);
-        tile_mma(accA, t + 1);
-        tile_argmin(accB, t);
-      }
-      if (t < KT) {
-        tile_mma(accB, t);
-        tile_argmin(accA, t - 1);
-        tile_argmin(accB, t);
-      } else {
-        tile_argmin(accA, t - 1);
-      }
+    // (Software-pipelining tile t's matrix work against tile t-1's argmin with a second
+    // accumulator set measured no faster: the two do not overlap on this hardware, and
+    // the extra registers cost occupancy.)
+    for (int t = 0; t < KT; t++) {
+      acc_t acc[ROWT];
+      tile_mma(acc, t);
+      tile_argmin(acc, t);
     }
     if constexpr (sizeof(T) == 4) {
 #pragma unroll
@@ -1232,10 +1210,7 @@ static size_t rowstat_fused_lds(int d, int k) {
 // Persistent grid of the row-stationary kernels: as many workgroups as stay
 // resident (two 4-wave workgroups per CU while two LDS images fit, otherwise
 // one 8-wave workgroup per CU), never more than there are row tiles.
-#ifndef KM_TWO_PER_CU_LIMIT
-#define KM_TWO_PER_CU_LIMIT (80 * 1024)
-#endif
-static bool rowstat_two_per_cu(size_t lds) { return lds <= (size_t)KM_TWO_PER_CU_LIMIT; }
+static bool rowstat_two_per_cu(size_t lds) { return lds <= (size_t)80 * 1024; }
 
 template <typename T, int DP, int ROWT, bool FUSE, int NW>
 static int launch_rowstat_nw(hipStream_t s, const T *X, const T *xnorm, const T *C,
@@ -1308,10 +1283,7 @@ struct RowstatDispatch<float, FUSE> {
     switch (rowstat_dp<float>(d)) {
       KM_ROWSTAT_CASE(float, 8, 2);
       KM_ROWSTAT_CASE(float, 16, 2);
-#ifndef KM_ROWT_F32_32
-#define KM_ROWT_F32_32 2
-#endif
-      KM_ROWSTAT_CASE(float, 32, KM_ROWT_F32_32);
+      KM_ROWSTAT_CASE(float, 32, 2);
       KM_ROWSTAT_CASE(float, 64, 1);  // one row tile: fits 16 wavefronts per CU
       KM_ROWSTAT_CASE(float, 128, 1);
     }

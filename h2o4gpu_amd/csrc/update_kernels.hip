@@ -268,9 +268,7 @@ __global__ __launch_bounds__(TPB) void accumulate_kernel(
 // centroids start on different banks.
 static int update_lds_stride(int d) { return d | 1; }
 static constexpr size_t UPDATE_LDS_MAX = 150 * 1024;
-#ifndef KM_MAX_LDS_CHUNKS
-#define KM_MAX_LDS_CHUNKS 8
-#endif
+static constexpr int KM_MAX_LDS_CHUNKS = 8;
 
 template <typename T>
 UpdatePlan plan_update(int64_t n, int d, int k, int num_cu) {
