@@ -831,7 +831,10 @@ struct TiledCfg {
   // staged tile pair and its staging instructions weighed twice as much (2M x 256, k = 1024
   // double: 0.75 -> 0.81 of peak with 128 rows, a few spilled registers included)
   static constexpr int BR = 128;
-  static constexpr int BK = sizeof(T) == 4 ? 32 : 16;
+  // features per stage. The 64-centroid form serves bandwidth-bound shapes (k <= 64): half
+  // the stage depth halves its LDS image, so twice as many workgroups keep loads in flight
+  // (500k x 784, k = 10: 0.62 -> 0.49 ms; a quarter of the depth was slower again).
+  static constexpr int BK = (sizeof(T) == 4 ? 32 : 16) / (BCW == 1 ? 2 : 1);
 };
 
 template <typename T, int MODE, bool VECLOAD, bool DTAIL, int BCW>
