@@ -98,6 +98,7 @@ struct UpdatePlan {
   int k_chunks;     // ceil(k / kc)
   int vec;          // elements per load (1, 2 or 4)
   int sd;           // LDS row stride of the sums, in elements
+  int threads;      // workgroup size of the accumulate kernel (256, 512 or 1024)
   size_t lds_bytes;
 };
 template <typename T>

@@ -289,7 +289,12 @@ UpdatePlan plan_update(int64_t n, int d, int k, int num_cu) {
   // enough workgroups to cover the machine a few times, but bounded so the
   // partials buffer (row_blocks * k * d) stays small next to the data
   // (fewer when a workgroup's LDS image leaves room for only one or two per CU)
-  const int per_cu = p.lds_bytes > 80 * 1024 ? 1 : (p.lds_bytes > 40 * 1024 ? 2 : 4);
+  // An LDS image above 40 KB leaves room for at most three 4-wave workgroups per CU: one
+  // 16-wave workgroup per CU then keeps more loads in flight (500k x 784, k = 10, 63 KB:
+  // 0.48 -> 0.43 ms); below that, four 4-wave workgroups per CU.
+  const bool wide = p.lds_bytes > 40 * 1024;
+  p.threads = wide ? 1024 : 256;
+  const int per_cu = wide ? 1 : 4;
   int64_t want = (int64_t)num_cu * per_cu / p.k_chunks;
   if (want < 1) want = 1;
   int64_t max_by_rows = (n + 1023) / 1024;  // at least 1024 rows per block
@@ -311,19 +316,20 @@ static int launch_accumulate_vec(hipStream_t s, const UpdatePlan &p, const T *X,
   int groups = (d + VEC - 1) / VEC;  // lanes wanted per row
   int lpr = 1;
   while (lpr < groups && lpr < 64) lpr <<= 1;
-  // a large LDS image means one workgroup per CU: make it 16 wavefronts
-  if (p.lds_bytes > 64 * 1024) {
-    auto kern = accumulate_kernel<T, VEC, RAGGED, 1024>;
-    KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   (int)p.lds_bytes));
-    hipLaunchKernelGGL(kern, dim3(p.row_blocks, p.k_chunks), dim3(1024), p.lds_bytes, s, X, labels,
-                       psums, pcounts, n, d, k, p.kc, rows_per_block, lpr, p.sd);
-  } else {
-    auto kern = accumulate_kernel<T, VEC, RAGGED, WG>;
-    hipLaunchKernelGGL(kern, dim3(p.row_blocks, p.k_chunks), dim3(WG), p.lds_bytes, s, X, labels,
-                       psums, pcounts, n, d, k, p.kc, rows_per_block, lpr, p.sd);
-  }
+  // workgroup size from the plan: 16 wavefronts when only one workgroup fits a CU
+#define KM_ACC_LAUNCH(TPB)                                                                      \
+  do {                                                                                          \
+    auto kern = accumulate_kernel<T, VEC, RAGGED, TPB>;                                         \
+    if (p.lds_bytes > 64 * 1024)                                                                \
+      KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                      \
+                                     hipFuncAttributeMaxDynamicSharedMemorySize,                \
+                                     (int)p.lds_bytes));                                        \
+    hipLaunchKernelGGL(kern, dim3(p.row_blocks, p.k_chunks), dim3(TPB), p.lds_bytes, s, X,      \
+                       labels, psums, pcounts, n, d, k, p.kc, rows_per_block, lpr, p.sd);       \
+  } while (0)
+  if (p.threads == 1024) KM_ACC_LAUNCH(1024);
+  else KM_ACC_LAUNCH(256);
+#undef KM_ACC_LAUNCH
   KM_HIP_TRY(hipGetLastError());
   return 0;
 }
