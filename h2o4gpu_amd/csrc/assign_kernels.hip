@@ -638,7 +638,7 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
         }
       }
       xxn[rt] = xnorm[row];
-      if (merge) {  // the row's result from the earlier chunks travels with the prefetch
+      if (!FUSE && merge) {  // the row's result from the earlier chunks travels with the prefetch
         pmn[rt] = mindist[row];
         pln[rt] = labels[row];
       }
@@ -768,7 +768,7 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
         // this chunk is strictly closer (earlier chunks hold the lower indices).
         T bv = best[rt];
         int bi = bidx[rt] < 0 ? -1 : bidx[rt] + c_off;
-        if (merge) argmin_merge(bv, bi, pm[rt], pl[rt]);
+        if (!FUSE && merge) argmin_merge(bv, bi, pm[rt], pl[rt]);  // (a fused step is never chunked)
         labels[row] = bi;
         if (mindist) mindist[row] = bv;
       }
