@@ -583,7 +583,6 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
   }
 
   constexpr int ROWS_PER_WAVE = ROWT * MT;
-  constexpr int ROWS_PER_WG = NW * ROWS_PER_WAVE;
   // The rows of the next tile are fetched while the current tile is swept, so
   // the only exposed memory latency is that of the first tile.
   T xn[ROWT][DCH];
@@ -644,10 +643,16 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
       }
     }
   };
-  const int64_t base0 = (int64_t)blockIdx.x * ROWS_PER_WG;
-  if (base0 < n) fetch_rows(base0 + (int64_t)wave * ROWS_PER_WAVE);
-  for (int64_t base = base0; base < n; base += (int64_t)gridDim.x * ROWS_PER_WG) {
-    const int64_t wrow0 = base + (int64_t)wave * ROWS_PER_WAVE;
+  // Row tiles of ROWS_PER_WAVE rows are dealt out one per workgroup before the next
+  // wavefront slot gets any: wavefront w of workgroup b takes tiles w*G + b, then every
+  // G*NW-th after it. In the last, partial round the remaining tiles thus spread over all
+  // CUs and SIMDs instead of filling the first few workgroups, whose four wavefronts per
+  // SIMD would share one matrix pipe while the rest of the chip idles.
+  const int64_t tile_stride = (int64_t)gridDim.x * NW;
+  const int64_t row_stride = tile_stride * ROWS_PER_WAVE;
+  const int64_t wrow_first = ((int64_t)wave * gridDim.x + blockIdx.x) * ROWS_PER_WAVE;
+  if (wrow_first < n) fetch_rows(wrow_first);
+  for (int64_t wrow0 = wrow_first; wrow0 < n; wrow0 += row_stride) {
     T x[ROWT][DCH];
     T xx[ROWT];
     T pm[ROWT];
@@ -660,10 +665,7 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
       pm[rt] = pmn[rt];
       pl[rt] = pln[rt];
     }
-    {
-      const int64_t nbase = base + (int64_t)gridDim.x * ROWS_PER_WG;
-      if (nbase < n) fetch_rows(nbase + (int64_t)wave * ROWS_PER_WAVE);
-    }
+    if (wrow0 + row_stride < n) fetch_rows(wrow0 + row_stride);
     T best[ROWT];
     int bidx[ROWT];
     unsigned bkey[ROWT];  // float32 path: running minimum key and its tile
@@ -1222,8 +1224,10 @@ static int launch_rowstat_nw(hipStream_t s, const T *X, const T *xnorm, const T 
                              size_t lds, int c_off, int merge) {
   const int MT = Mfma<T>::MT;
   const int kp = (k + MT - 1) / MT * MT;
-  const int rows_per_wg = NW * ROWT * MT;
-  const int64_t tiles = (n + rows_per_wg - 1) / rows_per_wg;
+  // (row tiles go round the workgroups before a second wavefront of any gets one, so a
+  // small data set spreads over as many CUs as it has tiles)
+  const int rows_per_wave = ROWT * MT;
+  const int64_t tiles = (n + rows_per_wave - 1) / rows_per_wave;
   int64_t grid = (int64_t)num_cu * (NW == 4 ? 2 : 1);
   if (grid > tiles) grid = tiles;
   if (grid < 1) grid = 1;
