@@ -31,7 +31,7 @@ PEAK_MFMA_TFLOPS = {"f32": 157.3, "f64": 78.6}
 # 1.0 for WRITE_SIZE on this box). Keyed by (workload, dtype, kernel); other
 # combinations report null.
 MEASURED_TRAFFIC_BYTES = {
-    ("C3", "f32", "assign_accumulate"): (651690 * 2.0 + 97837 * 1.0) * 1024.0,
+    ("C3", "f32", "assign_accumulate"): (644709 * 2.0 + 94765 * 1.0) * 1024.0,
     # tiled kernel: the row slice is re-read once per 128-centroid block and misses L2
     # (profiles/assign_tiled_c4.md); the figure is L2-miss traffic, HBM or memory-side cache
     ("C4", "f32", "assign"): (7342683 * 2.0 + 15625 * 1.0) * 1024.0,
