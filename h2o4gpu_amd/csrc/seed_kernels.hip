@@ -60,7 +60,36 @@ __global__ __launch_bounds__(WG) void centre_dists_kernel(const T *__restrict__ 
 // skipped only when the bound holds with a 1e-4 margin; where the stored minimum is
 // itself within rounding of zero the kept value can exceed what a recomputation would
 // give by less than that rounding error.
-template <typename T, int VEC>
+// SUB: rows per workgroup. KPP_BLOCK: the workgroup also writes its block sum. Smaller
+// (long rows, where 1024 of them per workgroup leave a 500,000-row data set with two
+// workgroups per CU): the block sums come from block_sums_kernel afterwards.
+template <typename T>
+__device__ __forceinline__ void block_sum(const T *__restrict__ mind, double *__restrict__ bsums,
+                                          int64_t block, int64_t n, double *red) {
+  const int tid = threadIdx.x;
+  const int64_t b0 = block * KPP_BLOCK;
+  double acc = 0;
+#pragma unroll
+  for (int q = 0; q < KPP_BLOCK / WG; q++) {
+    const int64_t row = b0 + tid + q * WG;
+    if (row < n) acc += (double)mind[row];
+  }
+  red[tid] = acc;
+  __syncthreads();
+  for (int off = WG / 2; off > 0; off >>= 1) {
+    if (tid < off) red[tid] += red[tid + off];
+    __syncthreads();
+  }
+  if (tid == 0) bsums[block] = red[0];
+}
+template <typename T>
+__global__ __launch_bounds__(WG) void block_sums_kernel(const T *__restrict__ mind,
+                                                       double *__restrict__ bsums, int64_t n) {
+  __shared__ double red[WG];
+  block_sum<T>(mind, bsums, blockIdx.x, n, red);
+}
+
+template <typename T, int VEC, int SUB>
 __global__ __launch_bounds__(WG) void min_dist_update_kernel(
     const T *__restrict__ X, const T *__restrict__ xnorm, int64_t centre_row,
     T *__restrict__ mind, int *__restrict__ nearest, const T *__restrict__ dcc, int t,
@@ -68,7 +97,7 @@ __global__ __launch_bounds__(WG) void min_dist_update_kernel(
   extern __shared__ __align__(16) unsigned char smem_raw[];
   T *cs = reinterpret_cast<T *>(smem_raw);  // [d]
   __shared__ double red[WG];
-  __shared__ int list[KPP_BLOCK];
+  __shared__ int list[SUB];
   __shared__ int cnt;
   typedef typename SeedVec<T, VEC>::type vec_t;
   const int tid = threadIdx.x;
@@ -77,9 +106,9 @@ __global__ __launch_bounds__(WG) void min_dist_update_kernel(
   if (tid == 0) cnt = 0;
   const T cc = xnorm[centre_row];
   __syncthreads();
-  const int64_t b0 = (int64_t)blockIdx.x * KPP_BLOCK;
+  const int64_t b0 = (int64_t)blockIdx.x * SUB;
 #pragma unroll
-  for (int q = 0; q < KPP_BLOCK / WG; q++) {
+  for (int q = 0; q < SUB / WG; q++) {
     const int r = tid + q * WG;
     const int64_t row = b0 + r;
     if (row < n) {
@@ -137,20 +166,10 @@ __global__ __launch_bounds__(WG) void min_dist_update_kernel(
       }
     }
   }
-  __syncthreads();
-  double acc = 0;
-#pragma unroll
-  for (int q = 0; q < KPP_BLOCK / WG; q++) {
-    const int64_t row = b0 + tid + q * WG;
-    if (row < n) acc += (double)mind[row];
-  }
-  red[tid] = acc;
-  __syncthreads();
-  for (int off = WG / 2; off > 0; off >>= 1) {
-    if (tid < off) red[tid] += red[tid + off];
+  if (SUB == KPP_BLOCK) {
     __syncthreads();
+    block_sum<T>(mind, bsums, blockIdx.x, n, red);
   }
-  if (tid == 0) bsums[blockIdx.x] = red[0];
 }
 
 template <typename T>
@@ -167,14 +186,20 @@ int launch_min_dist_update(hipStream_t s, const T *X, const T *xnorm, int64_t ce
   int lpr = 1;
   while (lpr < per_row && lpr < 64) lpr <<= 1;
   const unsigned blocks = (unsigned)((n + KPP_BLOCK - 1) / KPP_BLOCK);
-  if (vec)
-    hipLaunchKernelGGL((min_dist_update_kernel<T, VW>), dim3(blocks), dim3(WG),
-                       (size_t)d * sizeof(T), s, X, xnorm, centre_row, mind, nearest, dcc, t, bsums,
-                       n, d, init, lpr);
-  else
-    hipLaunchKernelGGL((min_dist_update_kernel<T, 1>), dim3(blocks), dim3(WG),
-                       (size_t)d * sizeof(T), s, X, xnorm, centre_row, mind, nearest, dcc, t, bsums,
-                       n, d, init, lpr);
+  // long rows: 256 rows per workgroup, block sums afterwards (500k x 784: 489 workgroups
+  // of 1024 rows are fewer than two per CU)
+  const bool fine = (size_t)d * sizeof(T) >= 1024 && n >= 4 * KPP_BLOCK;
+#define KM_MDU(VECW, SUB)                                                                      \
+  hipLaunchKernelGGL((min_dist_update_kernel<T, VECW, SUB>),                                   \
+                     dim3((unsigned)((n + SUB - 1) / SUB)), dim3(WG), (size_t)d * sizeof(T), s, \
+                     X, xnorm, centre_row, mind, nearest, dcc, t, bsums, n, d, init, lpr)
+  if (vec && fine) KM_MDU(VW, 256);
+  else if (vec) KM_MDU(VW, KPP_BLOCK);
+  else if (fine) KM_MDU(1, 256);
+  else KM_MDU(1, KPP_BLOCK);
+#undef KM_MDU
+  if (fine)
+    hipLaunchKernelGGL((block_sums_kernel<T>), dim3(blocks), dim3(WG), 0, s, mind, bsums, n);
   KM_HIP_TRY(hipGetLastError());
   return 0;
 }

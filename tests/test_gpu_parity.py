@@ -275,7 +275,8 @@ def test_transform_matches_oracle(hip, oracle, n, d, k, dtype):
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("n,d,k,seed", [(5000, 6, 12, 3), (20000, 32, 40, 11), (3000, 100, 25, 5), (1500, 3, 7, 0),
-                                        (4000, 101, 20, 2), (2500, 7, 9, 4)])
+                                        (4000, 101, 20, 2), (2500, 7, 9, 4),
+                                        (6000, 300, 12, 7), (4100, 257, 6, 8)])  # long rows: 256-row workgroups
 def test_kmeanspp_seeding(hip, oracle, n, d, k, seed, dtype):
     """k-means++ on the device: same draw rule as the CPU restatement (same generator
     calls, same fixed-tree block sums), so the chosen rows agree; the minimum distances
