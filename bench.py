@@ -137,8 +137,10 @@ def main():
     ap.add_argument("--cpu-iters", type=int, default=0, help="CPU baseline iterations (0 = about 12 s worth)")
     ap.add_argument("--sklearn-rows", type=int, default=10_000_000,
                     help="rows of the workload the scikit-learn leg runs on")
-    ap.add_argument("--end-to-end", action="store_true",
-                    help="also time one whole fit through make_ptr_*_kmeans (upload included)")
+    ap.add_argument("--no-end-to-end", dest="end_to_end", action="store_false",
+                    help="skip the whole fit through make_ptr_*_kmeans (upload included, field c_abi_fit)")
+    ap.add_argument("--end-to-end", dest="end_to_end", action="store_true", help=argparse.SUPPRESS)
+    ap.set_defaults(end_to_end=True)
     args = ap.parse_args()
 
     if args.gpus != 1:
