@@ -154,7 +154,7 @@ template <typename T>
 struct BlockLoad<T, 1> {
   typedef T type;
 };
-template <typename T, int DREG>
+template <typename T, int DREG, bool SUMS>
 __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
     const T *__restrict__ X, const T *__restrict__ xnorm, const T *__restrict__ C,
     const T *__restrict__ cnorm, int *__restrict__ labels, T *__restrict__ mindist,
@@ -164,15 +164,18 @@ __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
   constexpr int d = DREG;
   constexpr int VEC = Mfma<T>::VW;
   const int sx = staged_row_stride(d);                           // row stride of the staged block
+  // SUMS false: assignment only (predict, final relabel, inertia): no sums, no counts
   double *sums = reinterpret_cast<double *>(smem_raw);           // [k][sx]
-  int *cnt = reinterpret_cast<int *>(sums + (size_t)k * sx);     // [k]
-  T *ccs = reinterpret_cast<T *>(cnt + k + (k & 1));             // [k] centroid norms
+  int *cnt = reinterpret_cast<int *>(sums + (SUMS ? (size_t)k * sx : 0));  // [k]
+  T *ccs = reinterpret_cast<T *>(cnt + (SUMS ? k + (k & 1) : 0));          // [k] centroid norms
   T *Xs = ccs + k + (k & 1);                                     // [WG][sx]
   typedef typename BlockLoad<T, VEC>::type ld_t;
   constexpr int NLD = DREG / VEC;  // loads per thread and block
   const int tid = threadIdx.x;
-  for (int e = tid; e < k * sx; e += WG) sums[e] = 0.0;
-  for (int c = tid; c < k; c += WG) cnt[c] = 0;
+  if (SUMS) {
+    for (int e = tid; e < k * sx; e += WG) sums[e] = 0.0;
+    for (int c = tid; c < k; c += WG) cnt[c] = 0;
+  }
   // LDS offset of the i-th load of this thread: element (tid + i*WG)*VEC of the block
   int off[NLD];
 #pragma unroll
@@ -240,7 +243,7 @@ __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
       }
       labels[row] = bidx;
       if (mindist) mindist[row] = best;
-      if (bidx >= 0) {
+      if (SUMS && bidx >= 0) {
         // Lane l starts at feature l mod d: with only a handful of centroids the
         // lanes of a wavefront would otherwise all add to the same few addresses
         // at once, and same-address LDS atomics are served one lane at a time.
@@ -254,6 +257,7 @@ __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
       }
     }
   }
+  if (!SUMS) return;
   __syncthreads();
   double *dst = psums + (size_t)blockIdx.x * k * d;
   for (int e = tid; e < k * d; e += WG) {
@@ -280,7 +284,7 @@ __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
 // set is fetched value by value.
 // DMAX bounds d (it sizes the register prefetch of the next block); d >= VEC.
 // ---------------------------------------------------------------------------
-template <typename T, int DMAX, int VEC, int KREG>
+template <typename T, int DMAX, int VEC, int KREG, bool SUMS>
 __global__ __launch_bounds__(WG) void lloyd_valu_anyd_kernel(
     const T *__restrict__ X, const T *__restrict__ xnorm, const T *__restrict__ C,
     const T *__restrict__ cnorm, int *__restrict__ labels, T *__restrict__ mindist,
@@ -289,15 +293,17 @@ __global__ __launch_bounds__(WG) void lloyd_valu_anyd_kernel(
   extern __shared__ __align__(16) unsigned char smem_raw[];
   const int sx = staged_row_stride(d);
   const int pad = sx - d;                                        // 0 or 1
-  double *sums = reinterpret_cast<double *>(smem_raw);           // [k][sx]
-  int *cnt = reinterpret_cast<int *>(sums + (size_t)k * sx);     // [k]
-  T *ccs = reinterpret_cast<T *>(cnt + k + (k & 1));             // [k]
+  double *sums = reinterpret_cast<double *>(smem_raw);           // [k][sx]; SUMS false: none
+  int *cnt = reinterpret_cast<int *>(sums + (SUMS ? (size_t)k * sx : 0));  // [k]
+  T *ccs = reinterpret_cast<T *>(cnt + (SUMS ? k + (k & 1) : 0));          // [k]
   T *Xs = ccs + k + (k & 1);                                     // [WG][sx]
   typedef typename BlockLoad<T, VEC>::type ld_t;
   constexpr int NLD = (DMAX + VEC - 1) / VEC;
   const int tid = threadIdx.x;
-  for (int e = tid; e < k * sx; e += WG) sums[e] = 0.0;
-  for (int c = tid; c < k; c += WG) cnt[c] = 0;
+  if (SUMS) {
+    for (int e = tid; e < k * sx; e += WG) sums[e] = 0.0;
+    for (int c = tid; c < k; c += WG) cnt[c] = 0;
+  }
   const int nld = (d + VEC - 1) / VEC;  // loads per thread and block
   const int nvec = WG / VEC * d;        // vectors in a full block
   // el / d for el < 256 * 64 and d >= 2 as one multiply-high (exact while el * d < 2^32)
@@ -426,7 +432,7 @@ __global__ __launch_bounds__(WG) void lloyd_valu_anyd_kernel(
       }
       labels[row] = bidx;
       if (mindist) mindist[row] = best;
-      if (bidx >= 0) {
+      if (SUMS && bidx >= 0) {
         double *srow = sums + (size_t)bidx * sx;
         int jj = jrot;  // rotated start, as in lloyd_valu_fused_kernel
         for (int q = 0; q < d; q++) {
@@ -437,6 +443,7 @@ __global__ __launch_bounds__(WG) void lloyd_valu_anyd_kernel(
       }
     }
   }
+  if (!SUMS) return;
   __syncthreads();
   double *dst = psums + (size_t)blockIdx.x * k * d;
   for (int e = tid; e < k * d; e += WG) {
@@ -1317,9 +1324,9 @@ struct RowstatDispatch<double, FUSE> {
 
 static bool valu_fused_applies(int d, int k) { return k <= 16 && d <= 64; }
 template <typename T>
-static size_t valu_fused_lds(int d, int k) {
+static size_t valu_fused_lds(int d, int k, bool sums = true) {
   const int sx = staged_row_stride(d);
-  return (size_t)k * sx * sizeof(double) + ((size_t)k + 1) * sizeof(int) +
+  return (sums ? (size_t)k * sx * sizeof(double) + ((size_t)k + 1) * sizeof(int) : 0) +
          ((size_t)k + 1) * sizeof(T) + (size_t)WG * sx * sizeof(T) + 16;
 }
 static int valu_fused_grid(int64_t n, size_t lds, int num_cu) {
@@ -1345,11 +1352,12 @@ int fused_slots(int requested_variant, int64_t n, int d, int k, int num_cu) {
   return 2 * num_cu;  // upper bound of the grid = number of partial slots
 }
 
-template <typename T>
+// SUMS false: the same kernels without sums and counts (psums, pcounts, slots unused).
+template <typename T, bool SUMS>
 static int launch_valu_fused(hipStream_t s, const T *X, const T *xnorm, const T *C,
                              const T *cnorm, int *labels, T *mindist, int64_t n, int d, int k,
                              int num_cu, double *psums, int *pcounts, int *slots) {
-  const size_t lds = valu_fused_lds<T>(d, k);
+  const size_t lds = valu_fused_lds<T>(d, k, SUMS);
   const int grid = valu_fused_grid(n, lds, num_cu);
   if (slots) *slots = grid;
   const int vw = Mfma<T>::VW;
@@ -1361,7 +1369,7 @@ static int launch_valu_fused(hipStream_t s, const T *X, const T *xnorm, const T 
   // d is one of the register sizes: the row lives in registers
 #define KM_VF(DREG)                                                                        \
   do {                                                                                     \
-    auto kern = lloyd_valu_fused_kernel<T, DREG>;                                          \
+    auto kern = lloyd_valu_fused_kernel<T, DREG, SUMS>;                                    \
     KM_VF_SETUP(kern);                                                                     \
     hipLaunchKernelGGL(kern, dim3(grid), dim3(WG), lds, s, X, xnorm, C, cnorm, labels,     \
                        mindist, psums, pcounts, n, k);                                     \
@@ -1369,7 +1377,7 @@ static int launch_valu_fused(hipStream_t s, const T *X, const T *xnorm, const T 
   // any other d: dot products in registers, KREG >= k of them
 #define KM_VA_LAUNCH(DMAX, VEC, KREG)                                                      \
   do {                                                                                     \
-    auto kern = lloyd_valu_anyd_kernel<T, DMAX, VEC, KREG>;                                \
+    auto kern = lloyd_valu_anyd_kernel<T, DMAX, VEC, KREG, SUMS>;                          \
     KM_VF_SETUP(kern);                                                                     \
     hipLaunchKernelGGL(kern, dim3(grid), dim3(WG), lds, s, X, xnorm, C, cnorm, labels,     \
                        mindist, psums, pcounts, n, d, k);                                  \
@@ -1413,8 +1421,8 @@ int launch_assign_accumulate(hipStream_t s, int variant, const T *X, const T *xn
   const int v = pick_assign_variant<T>(variant, n, d, k);
   if (used) *used = v;
   if (v == ASSIGN_VALU && valu_fused_applies(d, k))
-    return launch_valu_fused<T>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu, psums,
-                                pcounts, slots);
+    return launch_valu_fused<T, true>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu,
+                                      psums, pcounts, slots);
   if (v != ASSIGN_ROWSTAT) return H2O4GPU_KMEANS_EARG;
   return RowstatDispatch<T, true>::run(s, X, xnorm, C, cnorm, labels, mindist, n, d, k,
                                        num_cu, psums, pcounts, slots);
@@ -1471,6 +1479,12 @@ int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
   if (used) *used = v;
   switch (v) {
     case ASSIGN_VALU:
+      // The staged kernels of the fused step, minus the sums: the one-thread-per-row
+      // kernel with its strided loads takes two to three times as long (8M x 32, k = 8:
+      // 0.68 vs 0.23 ms) except for rows of a few values, where staging does not pay.
+      if (valu_fused_applies(d, k) && (d >= 8 || d * sizeof(T) == 32))
+        return launch_valu_fused<T, false>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu,
+                                           nullptr, nullptr, nullptr);
       return launch_valu<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k);
     case ASSIGN_ROWSTAT: {
       const int kc = rowstat_chunk<T>(d, k);
