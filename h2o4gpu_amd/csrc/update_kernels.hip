@@ -26,6 +26,27 @@ static constexpr int WG = 256;
 // the result does not depend on the order in which wavefronts arrive.
 __device__ __forceinline__ void lds_add(double *p, double v) { unsafeAtomicAdd(p, v); }
 
+// 2 or 4 consecutive row values as one load. The types are aligned to their elements
+// only: a row of d values starts wherever it starts, and gfx950 serves such a load with
+// one instruction.
+template <typename T, int VEC>
+struct VecOf;
+template <> struct VecOf<float, 4> { typedef float type __attribute__((ext_vector_type(4), aligned(4))); };
+template <> struct VecOf<float, 2> { typedef float type __attribute__((ext_vector_type(2), aligned(4))); };
+template <> struct VecOf<double, 2> { typedef double type __attribute__((ext_vector_type(2), aligned(8))); };
+
+template <typename T, int VEC>
+struct RowVec {
+  typedef typename VecOf<T, VEC>::type type;
+};
+template <typename T>
+struct RowVec<T, 1> {
+  typedef T type;
+};
+template <typename T, int VEC>
+__device__ __forceinline__ typename RowVec<T, VEC>::type load_vec(const T *p) {
+  return *reinterpret_cast<const typename RowVec<T, VEC>::type *>(p);
+}
 // ---------------------------------------------------------------------------
 // out[i] = sum_j X[i][j]^2, j ascending, multiply and add rounded separately
 // (what self_dots does, kmeans_labels.h:187-199). One thread per row; used once
@@ -75,9 +96,75 @@ __global__ __launch_bounds__(WG) void row_norms_coalesced_kernel(
   if (col == 0 && row < n) out[row] = acc;
 }
 
+// Same result for short rows (d <= 64) of a large matrix: a block of 256 rows is one
+// contiguous run of 256*d values, fetched as a flat array of 16-byte vectors (the block
+// starts on a 16-byte boundary whatever d is; VEC = 1 for data that is not 16-byte aligned)
+// into LDS with an odd row stride, and every thread then sums its own row in j order.
+template <typename T, int VEC>
+__global__ __launch_bounds__(WG) void row_norms_staged_kernel(const T *__restrict__ X,
+                                                             T *__restrict__ out, int64_t n, int d) {
+#pragma clang fp contract(off)
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  T *Xs = reinterpret_cast<T *>(smem_raw);  // [WG][sx]
+  typedef typename RowVec<T, VEC>::type ld_t;
+  int sx = d | 1;
+  if (((sx + 1) & sx) == 0) sx += 2;  // never 2^m - 1 (measured slow as an LDS row stride)
+  const int pad = sx - d;
+  const int tid = threadIdx.x;
+  const unsigned dinv = d > 1 ? 0xFFFFFFFFu / (unsigned)d + 1u : 0u;  // el / d by multiply-high
+  auto row_of = [&](int el) -> int { return d > 1 ? (int)__umulhi((unsigned)el, dinv) : el; };
+  for (int64_t base = (int64_t)blockIdx.x * WG; base < n; base += (int64_t)gridDim.x * WG) {
+    const int rows = (int)min<int64_t>(WG, n - base);
+    const T *xb = X + base * (int64_t)d;
+    const int total = rows * d;     // values of this block
+    const int nvec = total / VEC;   // complete vectors
+    __syncthreads();                // the previous block has been consumed
+    for (int e = tid; e < nvec; e += WG) {
+      const ld_t v = *reinterpret_cast<const ld_t *>(xb + (size_t)e * VEC);
+      const int el = e * VEC;
+      if constexpr (VEC == 1) {
+        Xs[el + row_of(el) * pad] = v;
+      } else {
+#pragma unroll
+        for (int q = 0; q < VEC; q++) Xs[el + q + row_of(el + q) * pad] = v[q];
+      }
+    }
+    if (tid < total - nvec * VEC) {  // values behind the last complete vector of the data set
+      const int el = nvec * VEC + tid;
+      Xs[el + row_of(el) * pad] = xb[el];
+    }
+    __syncthreads();
+    if (tid < rows) {
+      const T *x = Xs + tid * sx;
+      T acc = 0;
+      for (int j = 0; j < d; j++) {
+        const T v = x[j];
+        acc = acc + v * v;
+      }
+      out[base + tid] = acc;
+    }
+  }
+}
+
 template <typename T>
 int launch_row_norms(hipStream_t s, const T *X, T *out, int64_t n, int d) {
   if (n <= 0) return 0;
+  if (d >= 4 && d <= 64 && n * (int64_t)d >= (1 << 22)) {
+    int sx = d | 1;
+    if (((sx + 1) & sx) == 0) sx += 2;
+    const size_t lds = (size_t)WG * sx * sizeof(T);
+    int64_t grid = (n + WG - 1) / WG;
+    if (grid > 256 * 8) grid = 256 * 8;
+    constexpr int VW = 16 / sizeof(T);
+    if ((reinterpret_cast<uintptr_t>(X) & 15) == 0)
+      hipLaunchKernelGGL((row_norms_staged_kernel<T, VW>), dim3((unsigned)grid), dim3(WG), lds, s, X, out,
+                         n, d);
+    else
+      hipLaunchKernelGGL((row_norms_staged_kernel<T, 1>), dim3((unsigned)grid), dim3(WG), lds, s, X, out,
+                         n, d);
+    KM_HIP_TRY(hipGetLastError());
+    return 0;
+  }
   // (a thread per row is enough for a handful of short rows; long rows always go
   // through the cooperative kernel, a single thread would walk them serially)
   if (d >= 8 && (n * (int64_t)d >= 65536 || d >= 64)) {
@@ -113,27 +200,6 @@ int launch_row_norms(hipStream_t s, const T *X, T *out, int64_t n, int d) {
 // 64/LPR rows in flight. With a single centroid chunk every row matches and
 // the ballot is skipped.
 // ---------------------------------------------------------------------------
-// 2 or 4 consecutive row values as one load. The types are aligned to their elements
-// only: a row of d values starts wherever it starts, and gfx950 serves such a load with
-// one instruction.
-template <typename T, int VEC>
-struct VecOf;
-template <> struct VecOf<float, 4> { typedef float type __attribute__((ext_vector_type(4), aligned(4))); };
-template <> struct VecOf<float, 2> { typedef float type __attribute__((ext_vector_type(2), aligned(4))); };
-template <> struct VecOf<double, 2> { typedef double type __attribute__((ext_vector_type(2), aligned(8))); };
-
-template <typename T, int VEC>
-struct RowVec {
-  typedef typename VecOf<T, VEC>::type type;
-};
-template <typename T>
-struct RowVec<T, 1> {
-  typedef T type;
-};
-template <typename T, int VEC>
-__device__ __forceinline__ typename RowVec<T, VEC>::type load_vec(const T *p) {
-  return *reinterpret_cast<const typename RowVec<T, VEC>::type *>(p);
-}
 // adds elements first .. VEC-1 of v to dst[first .. VEC-1]
 template <typename T, int VEC, bool RAGGED>
 __device__ __forceinline__ void lds_add_vec(double *dst, typename RowVec<T, VEC>::type v, int first) {

@@ -191,7 +191,9 @@ def test_fused_step_equals_separate_kernels(hip, oracle, n, d, k, dtype):
                                    # block whose values do not fill a vector
                                    (5003, 30, 8), (777, 31, 5), (20001, 50, 16), (9001, 46, 3), (6000, 12, 9),
                                    (4099, 63, 13), (2051, 62, 4), (12345, 20, 8), (1025, 5, 2), (300, 7, 16),
-                                   (255, 13, 6), (257, 15, 1), (100001, 24, 12)])
+                                   (255, 13, 6), (257, 15, 1), (100001, 24, 12),
+                                   # large enough for the staged row-norm kernel (4M values and more)
+                                   (300001, 16, 8), (140003, 30, 5), (70001, 63, 9), (1050000, 4, 3)])
 def test_small_shape_fused_step_is_bit_exact(hip, oracle, n, d, k, dtype):
     """k <= 16 and d <= 64: the one-pass VALU step. Labels and minimum distances are
     bit-identical to the scalar CPU loop; float32 centroids are bit-identical to the
