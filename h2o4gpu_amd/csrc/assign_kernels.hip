@@ -490,7 +490,7 @@ __device__ __forceinline__ int key_row(unsigned v, int g) {
 // aligned to its elements: 16-byte loads that stay inside the row (padded features are
 // zero, or finite values meeting zeros on the centroid side).
 // 0: d below the vector width: scalar loads, zero padded.
-template <typename T, int DP, int ROWT, int LOAD, bool FUSE, int NW>
+template <typename T, int DP, int ROWT, int LOAD, bool FUSE, int NW, bool EXACT = false>
 __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
     const T *__restrict__ X, const T *__restrict__ xnorm,
     const T *__restrict__ C, const T *__restrict__ cnorm,
@@ -505,6 +505,8 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
   typedef typename M::acc_t acc_t;
   typedef typename M::vec_t vec_t;
   constexpr bool VECLOAD = LOAD == 1;
+  // float32 argmin on integer keys (16-ulp resolution) unless the exact compare chain is asked for
+  constexpr bool KEYS = sizeof(T) == 4 && !EXACT;
 
   extern __shared__ __align__(16) unsigned char smem_raw[];
   T *Cs = reinterpret_cast<T *>(smem_raw);  // [KT][NV][64][VW], see cs_slot
@@ -706,7 +708,7 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
       }
     };
     auto tile_argmin = [&](const acc_t (&acc)[ROWT], int t) {
-      if constexpr (sizeof(T) == 4) {
+      if constexpr (KEYS) {
         // float32 MFMA shares the SIMD's FP32 datapath with ordinary vector
         // instructions, so every epilogue instruction costs matrix time. The
         // argmin is therefore done on integer keys: |acc| with its four lowest
@@ -714,7 +716,9 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
         // reduced with 3-input unsigned minima (positive floats order like
         // unsigned integers), the winner is compared once per tile with the
         // running key. Distances are thus compared at a resolution of 16 ulp
-        // (1.9e-6 relative); within one key value the lowest centroid index wins.
+        // (1.9e-6 relative); within one 16-ulp bucket the lowest centroid index wins:
+        // inside a tile through the index bits, across tiles because a later tile must
+        // be below the running key's bucket (index bits ignored) to replace it.
 #pragma unroll
         for (int rt = 0; rt < ROWT; rt++) {
           unsigned key[NACC];
@@ -725,7 +729,7 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
 #pragma unroll
           for (int v = 3; v + 1 < NACC; v += 2) m = umin3(m, key[v], key[v + 1]);
           if ((NACC & 1) == 0) m = min(m, key[NACC - 1]);
-          if (m < bkey[rt]) {
+          if ((m | 15u) < bkey[rt]) {
             bkey[rt] = m;
             btile[rt] = t;
           }
@@ -754,7 +758,7 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
       tile_mma(acc, t);
       tile_argmin(acc, t);
     }
-    if constexpr (sizeof(T) == 4) {
+    if constexpr (KEYS) {
 #pragma unroll
       for (int rt = 0; rt < ROWT; rt++) {
         best[rt] = __uint_as_float(bkey[rt] & 0xFFFFFFF0u);
@@ -846,7 +850,7 @@ struct TiledCfg {
   static constexpr int BK = (sizeof(T) == 4 ? 32 : 16) / (BCW == 1 ? 2 : 1);
 };
 
-template <typename T, int MODE, bool VECLOAD, bool DTAIL, int BCW>
+template <typename T, int MODE, bool VECLOAD, bool DTAIL, int BCW, bool EXACT = false>
 __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_kernel(
     const T *__restrict__ X, const T *__restrict__ xnorm,
     const T *__restrict__ C, const T *__restrict__ cnorm,
@@ -1043,8 +1047,9 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
           }
         }
       }
-    } else if constexpr (sizeof(T) == 4) {
-      // integer keys as in the row-stationary kernel (4 index bits, 16 ulp)
+    } else if constexpr (sizeof(T) == 4 && !EXACT) {
+      // integer keys as in the row-stationary kernel (4 index bits, 16 ulp; a later tile
+      // or block replaces the running key only from a lower bucket)
 #pragma unroll
       for (int ct = 0; ct < CT; ct++) {
 #pragma unroll
@@ -1057,7 +1062,7 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
 #pragma unroll
           for (int v = 3; v + 1 < NACC; v += 2) m = umin3(m, key[v], key[v + 1]);
           if ((NACC & 1) == 0) m = min(m, key[NACC - 1]);
-          if (m < bkey[rt]) {
+          if ((m | 15u) < bkey[rt]) {
             bkey[rt] = m;
             bblk[rt] = c0 + (wc * CT + ct) * MT;
           }
@@ -1082,7 +1087,7 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
     }
   }
   if (MODE == 0) {
-    if constexpr (sizeof(T) == 4) {
+    if constexpr (sizeof(T) == 4 && !EXACT) {
 #pragma unroll
       for (int rt = 0; rt < RT; rt++) {
         best[rt] = __uint_as_float(bkey[rt] & 0xFFFFFFF0u);
@@ -1228,7 +1233,7 @@ template <typename T, int DP, int ROWT, bool FUSE, int NW>
 static int launch_rowstat_nw(hipStream_t s, const T *X, const T *xnorm, const T *C,
                              const T *cnorm, int *labels, T *mindist, int64_t n, int d,
                              int k, int num_cu, double *psums, int *pcounts, int *slots,
-                             size_t lds, int c_off, int merge) {
+                             size_t lds, int c_off, int merge, bool exact) {
   const int MT = Mfma<T>::MT;
   const int kp = (k + MT - 1) / MT * MT;
   // (row tiles go round the workgroups before a second wavefront of any gets one, so a
@@ -1242,19 +1247,28 @@ static int launch_rowstat_nw(hipStream_t s, const T *X, const T *xnorm, const T 
   const bool xal = (reinterpret_cast<uintptr_t>(X) & 15) == 0;
   const bool vec = (d == DP) && xal && ((reinterpret_cast<uintptr_t>(C) & 15) == 0);
   const bool padvec = !vec && d >= Mfma<T>::VW;
-#define KM_RS_LAUNCH(LOAD)                                                                    \
+#define KM_RS_LAUNCH_X(LOAD, EXACT)                                                           \
   do {                                                                                        \
-    auto kern = assign_rowstat_kernel<T, DP, ROWT, LOAD, FUSE, NW>;                           \
-    if (lds > 64 * 1024)                                                                      \
-      KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                    \
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));  \
+    auto kern = assign_rowstat_kernel<T, DP, ROWT, LOAD, FUSE, NW, EXACT>;                    \
+    KM_TRY(ensure_dynamic_lds(reinterpret_cast<const void *>(kern), lds));                    \
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), lds, s, X, xnorm, C, cnorm, \
                        labels, mindist, n, d, k, kp, psums, pcounts, c_off, merge);           \
+  } while (0)
+  // the exact-compare form exists for the float32 assignment-only kernels
+#define KM_RS_LAUNCH(LOAD)                                       \
+  do {                                                           \
+    if constexpr (!FUSE && sizeof(T) == 4) {                     \
+      if (exact) KM_RS_LAUNCH_X(LOAD, true);                     \
+      else KM_RS_LAUNCH_X(LOAD, false);                          \
+    } else {                                                     \
+      KM_RS_LAUNCH_X(LOAD, false);                               \
+    }                                                            \
   } while (0)
   if (vec) KM_RS_LAUNCH(1);
   else if (padvec) KM_RS_LAUNCH(2);
   else KM_RS_LAUNCH(0);
 #undef KM_RS_LAUNCH
+#undef KM_RS_LAUNCH_X
   KM_HIP_TRY(hipGetLastError());
   return 0;
 }
@@ -1263,7 +1277,8 @@ template <typename T, int DP, int ROWT, bool FUSE>
 static int launch_rowstat_dp(hipStream_t s, const T *X, const T *xnorm,
                              const T *C, const T *cnorm, int *labels,
                              T *mindist, int64_t n, int d, int k, int num_cu,
-                             double *psums, int *pcounts, int *slots, int c_off, int merge) {
+                             double *psums, int *pcounts, int *slots, int c_off, int merge,
+                             bool exact) {
   const size_t lds = FUSE ? rowstat_fused_lds<T>(d, k) : rowstat_lds<T>(d, k);
   // Shapes whose register use fits 128 VGPRs run one 16-wavefront workgroup per CU, which
   // measured ahead of two 4-wave workgroups everywhere it applies (float32 10M x 32 and
@@ -1272,14 +1287,14 @@ static int launch_rowstat_dp(hipStream_t s, const T *X, const T *xnorm,
                         (sizeof(T) == 8 && ((DP <= 32 && ROWT <= 2) || (DP == 64 && ROWT == 1)));
   if (!wide && rowstat_two_per_cu(lds))
     return launch_rowstat_nw<T, DP, ROWT, FUSE, 4>(s, X, xnorm, C, cnorm, labels, mindist, n, d,
-                                                   k, num_cu, psums, pcounts, slots, lds, c_off, merge);
+                                                   k, num_cu, psums, pcounts, slots, lds, c_off, merge, exact);
   // one workgroup per CU: as many wavefronts as the register budget allows
   if constexpr (wide)
     return launch_rowstat_nw<T, DP, ROWT, FUSE, 16>(s, X, xnorm, C, cnorm, labels, mindist, n, d,
-                                                    k, num_cu, psums, pcounts, slots, lds, c_off, merge);
+                                                    k, num_cu, psums, pcounts, slots, lds, c_off, merge, exact);
   else
     return launch_rowstat_nw<T, DP, ROWT, FUSE, 8>(s, X, xnorm, C, cnorm, labels, mindist, n, d,
-                                                   k, num_cu, psums, pcounts, slots, lds, c_off, merge);
+                                                   k, num_cu, psums, pcounts, slots, lds, c_off, merge, exact);
 }
 
 template <typename T, bool FUSE>
@@ -1287,13 +1302,13 @@ struct RowstatDispatch;
 #define KM_ROWSTAT_CASE(T, DP, ROWT)                                                  \
   case DP:                                                                            \
     return launch_rowstat_dp<T, DP, ROWT, FUSE>(s, X, xnorm, C, cnorm, labels, mindist, \
-                                                n, d, k, num_cu, psums, pcounts, slots, c_off, merge)
+                                                n, d, k, num_cu, psums, pcounts, slots, c_off, merge, exact)
 template <bool FUSE>
 struct RowstatDispatch<float, FUSE> {
   static int run(hipStream_t s, const float *X, const float *xnorm, const float *C,
                  const float *cnorm, int *labels, float *mindist, int64_t n, int d,
                  int k, int num_cu, double *psums, int *pcounts, int *slots, int c_off = 0,
-                 int merge = 0) {
+                 int merge = 0, bool exact = false) {
     switch (rowstat_dp<float>(d)) {
       KM_ROWSTAT_CASE(float, 8, 2);
       KM_ROWSTAT_CASE(float, 16, 2);
@@ -1309,7 +1324,7 @@ struct RowstatDispatch<double, FUSE> {
   static int run(hipStream_t s, const double *X, const double *xnorm, const double *C,
                  const double *cnorm, int *labels, double *mindist, int64_t n, int d,
                  int k, int num_cu, double *psums, int *pcounts, int *slots, int c_off = 0,
-                 int merge = 0) {
+                 int merge = 0, bool exact = false) {
     switch (rowstat_dp<double>(d)) {
       // two row tiles keep these within 128 registers, i.e. 16 wavefronts per CU
       KM_ROWSTAT_CASE(double, 8, 2);
@@ -1362,10 +1377,7 @@ static int launch_valu_fused(hipStream_t s, const T *X, const T *xnorm, const T 
   if (slots) *slots = grid;
   const int vw = Mfma<T>::VW;
   const bool aligned = (reinterpret_cast<uintptr_t>(X) & 15) == 0;
-#define KM_VF_SETUP(kern)                                                                  \
-  if (lds > 64 * 1024)                                                                     \
-  KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                     \
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
+#define KM_VF_SETUP(kern) KM_TRY(ensure_dynamic_lds(reinterpret_cast<const void *>(kern), lds))
   // d is one of the register sizes: the row lives in registers
 #define KM_VF(DREG)                                                                        \
   do {                                                                                     \
@@ -1431,26 +1443,34 @@ int launch_assign_accumulate(hipStream_t s, int variant, const T *X, const T *xn
 template <typename T, int MODE, int BCW>
 static int launch_tiled_bcw(hipStream_t s, const T *X, const T *xnorm, const T *C,
                             const T *cnorm, int *labels, T *mindist, T *D, int64_t n,
-                            int64_t ldn, int d, int k) {
+                            int64_t ldn, int d, int k, bool exact) {
   typedef TiledCfg<T, BCW> Cfg;
   const size_t lds = (size_t)2 * (Cfg::BC + Cfg::BR) * Cfg::BK * sizeof(T);
   const dim3 grid((unsigned)((n + Cfg::BR - 1) / Cfg::BR),
                   MODE == 1 ? (unsigned)((k + Cfg::BC - 1) / Cfg::BC) : 1u);
   const bool vec = d >= Mfma<T>::VW;  // 16-byte loads need element alignment only
   const bool tail = (d % Cfg::BK) != 0;
-#define KM_TILED(VEC, TAIL)                                                                  \
+#define KM_TILED_X(VEC, TAIL, EXACT)                                                         \
   do {                                                                                       \
-    auto kern = assign_tiled_kernel<T, MODE, VEC, TAIL, BCW>;                                \
-    if (lds > 64 * 1024)                                                                     \
-      KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                   \
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
+    auto kern = assign_tiled_kernel<T, MODE, VEC, TAIL, BCW, EXACT>;                         \
+    KM_TRY(ensure_dynamic_lds(reinterpret_cast<const void *>(kern), lds));                   \
     hipLaunchKernelGGL(kern, grid, dim3(Cfg::TPB), lds, s, X, xnorm, C, cnorm, labels,       \
                        mindist, D, n, ldn, d, k);                                            \
+  } while (0)
+#define KM_TILED(VEC, TAIL)                                      \
+  do {                                                           \
+    if constexpr (MODE == 0 && sizeof(T) == 4) {                 \
+      if (exact) KM_TILED_X(VEC, TAIL, true);                    \
+      else KM_TILED_X(VEC, TAIL, false);                         \
+    } else {                                                     \
+      KM_TILED_X(VEC, TAIL, false);                              \
+    }                                                            \
   } while (0)
   if (vec && !tail) KM_TILED(true, false);
   else if (vec) KM_TILED(true, true);
   else KM_TILED(false, true);
 #undef KM_TILED
+#undef KM_TILED_X
   KM_HIP_TRY(hipGetLastError());
   return 0;
 }
@@ -1458,20 +1478,20 @@ static int launch_tiled_bcw(hipStream_t s, const T *X, const T *xnorm, const T *
 template <typename T, int MODE>
 static int launch_tiled(hipStream_t s, const T *X, const T *xnorm, const T *C,
                         const T *cnorm, int *labels, T *mindist, T *D, int64_t n,
-                        int64_t ldn, int d, int k) {
+                        int64_t ldn, int d, int k, bool exact = false) {
   // Measured at 2M x 256, k = 1024 and 500k x 784, k = 4096: two 4-wave workgroups per CU
   // (BCW = 2) beat one 8-wave workgroup with the wider centroid block (BCW = 4) by 5-10 %,
   // so the 128-centroid form is used for large models. Up to 64 centroids a 64-wide block
   // (two wavefronts) halves the matrix work spent on padding; such shapes are bandwidth-bound.
   if (k <= 64)
-    return launch_tiled_bcw<T, MODE, 1>(s, X, xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k);
-  return launch_tiled_bcw<T, MODE, 2>(s, X, xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k);
+    return launch_tiled_bcw<T, MODE, 1>(s, X, xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k, exact);
+  return launch_tiled_bcw<T, MODE, 2>(s, X, xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k, exact);
 }
 
 template <typename T>
 int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
                   const T *C, const T *cnorm, int *labels, T *mindist, int64_t n,
-                  int d, int k, int num_cu, int *used) {
+                  int d, int k, int num_cu, int *used, bool exact) {
   if (n <= 0) return 0;
   if (d < 1 || k < 1) return H2O4GPU_KMEANS_EARG;
   const int v = pick_assign_variant<T>(variant, n, d, k);
@@ -1490,16 +1510,16 @@ int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
       const int kc = rowstat_chunk<T>(d, k);
       if (kc < k && !mindist) {  // merging chunks needs the running minimum in memory
         if (used) *used = ASSIGN_TILED;
-        return launch_tiled<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k);
+        return launch_tiled<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k, exact);
       }
       for (int c0 = 0; c0 < k; c0 += kc)
         KM_TRY((RowstatDispatch<T, false>::run(s, X, xnorm, C + (size_t)c0 * d, cnorm + c0, labels,
                                                mindist, n, d, min(kc, k - c0), num_cu, nullptr,
-                                               nullptr, nullptr, c0, c0 > 0)));
+                                               nullptr, nullptr, c0, c0 > 0, exact)));
       return 0;
     }
     case ASSIGN_TILED:
-      return launch_tiled<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k);
+      return launch_tiled<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k, exact);
   }
   return H2O4GPU_KMEANS_EARG;
 }
@@ -1530,10 +1550,10 @@ template int pick_assign_variant<float>(int, int64_t, int, int);
 template int pick_assign_variant<double>(int, int64_t, int, int);
 template int launch_assign<float>(hipStream_t, int, const float *, const float *,
                                   const float *, const float *, int *, float *,
-                                  int64_t, int, int, int, int *);
+                                  int64_t, int, int, int, int *, bool);
 template int launch_assign<double>(hipStream_t, int, const double *, const double *,
                                    const double *, const double *, int *, double *,
-                                   int64_t, int, int, int, int *);
+                                   int64_t, int, int, int, int *, bool);
 template int launch_transform<float>(hipStream_t, const float *, const float *,
                                      const float *, const float *, float *, int64_t,
                                      int64_t, int, int, int);

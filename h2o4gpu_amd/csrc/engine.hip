@@ -124,6 +124,28 @@ static void first_rows_of_shuffle(int64_t n, int k, unsigned seed, int *out) {
   std::copy(a.begin(), a.end(), out);
 }
 
+// (kernel, device) -> largest dynamic-LDS size granted so far
+static std::mutex g_lds_mu;
+static std::map<std::pair<const void *, int>, size_t> g_lds_granted;
+int ensure_dynamic_lds(const void *kernel, size_t bytes) {
+  if (bytes <= 64 * 1024) return 0;  // within the default limit
+  int dev = 0;
+  KM_HIP_TRY(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_lds_mu);
+  size_t &granted = g_lds_granted[std::make_pair(kernel, dev)];
+  if (granted >= bytes) return 0;
+  KM_HIP_TRY(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+  granted = bytes;
+  return 0;
+}
+void forget_dynamic_lds(int dev) {
+  std::lock_guard<std::mutex> lock(g_lds_mu);
+  for (auto it = g_lds_granted.begin(); it != g_lds_granted.end();) {
+    if (it->first.second == dev) it = g_lds_granted.erase(it);
+    else ++it;
+  }
+}
+
 static int visible_devices() {
   int n = 0;
   if (hipGetDeviceCount(&n) != hipSuccess) {
@@ -152,6 +174,7 @@ struct h2o4gpu_kmeans_handle {
   int opt_assign = ASSIGN_AUTO;
   int opt_fuse = 1;  // 1: use the fused assign+accumulate kernel where the shape allows
   int opt_buckets = 1;  // 1: bucketed centroid sums where the sums do not fit LDS
+  int opt_exact = 0;    // 1: float32 MFMA argmin on the float distances, not on 16-ulp keys
   int last_variant = ASSIGN_AUTO;
 
   // profiling
@@ -730,7 +753,8 @@ struct Engine : h2o4gpu_kmeans_handle {
     if (!have_data || !have_centroids) return H2O4GPU_KMEANS_ESTATE;
     KM_TRY(ensure_cnorm());
     PROFILED("assign", launch_assign<T>(stream, opt_assign, X, xnorm, C[cur], cnorm,
-                                        labels, mindist, n, d, k, num_cu, &last_variant));
+                                        labels, mindist, n, d, k, num_cu, &last_variant,
+                                        opt_exact != 0));
     have_mindist = true;
     return 0;
   }
@@ -749,7 +773,10 @@ struct Engine : h2o4gpu_kmeans_handle {
   // one Lloyd step: labels against the current centroids, then the update.
   // want_shift: the caller will read the convergence scalar of this step.
   int step_async(bool want_shift) {
-    if (opt_fuse && fused_slots<T>(opt_assign, n, d, k, num_cu) > 0) {
+    // (the exact-compare argmin exists in the assignment-only kernels)
+    const bool exact_mfma = opt_exact && sizeof(T) == 4 &&
+                            pick_assign_variant<T>(opt_assign, n, d, k) != ASSIGN_VALU;
+    if (opt_fuse && !exact_mfma && fused_slots<T>(opt_assign, n, d, k, num_cu) > 0) {
       int slots = 0;
       PROFILED("assign_accumulate",
                launch_assign_accumulate<T>(stream, opt_assign, X, xnorm, C[cur], (const T *)nullptr,
@@ -933,7 +960,8 @@ struct Engine : h2o4gpu_kmeans_handle {
     KM_TRY(upload_rows(dev, stream, dX, hX, rows * d * sizeof(T)));
     PROFILED("row_norms", launch_row_norms<T>(stream, dX, dxn, (int64_t)rows, d));
     PROFILED("assign", launch_assign<T>(stream, opt_assign, dX, dxn, C[cur], cnorm, dl, dmin,
-                                        (int64_t)rows, d, k, num_cu, &last_variant));
+                                        (int64_t)rows, d, k, num_cu, &last_variant,
+                                        opt_exact != 0));
     KM_TRY(download_rows(dev, stream, out, dl, rows * sizeof(int)));
     KM_HIP_TRY(hipStreamSynchronize(stream));
     return 0;
@@ -1349,6 +1377,11 @@ KM_API int h2o4gpu_kmeans_set_option(h2o4gpu_kmeans_handle *h, const char *name,
     h->opt_buckets = value;
     return 0;
   }
+  if (strcmp(name, "exact_argmin") == 0) {
+    if (value != 0 && value != 1) return H2O4GPU_KMEANS_EARG;
+    h->opt_exact = value;
+    return 0;
+  }
   if (strcmp(name, "fuse") == 0) {
     if (value != 0 && value != 1) return H2O4GPU_KMEANS_EARG;
     h->opt_fuse = value;
@@ -1529,11 +1562,15 @@ KM_API int cudaresetdevice(int wDev, int nDev) {
   (void)nDev;
   if (hipSetDevice(wDev) != hipSuccess) return 1;
   g_staging.forget(wDev);
+  forget_dynamic_lds(wDev);
   return hipDeviceReset() == hipSuccess ? 0 : 1;
 }
 KM_API int cudaresetdevice_bare(void) {
   int dev = 0;
-  if (hipGetDevice(&dev) == hipSuccess) g_staging.forget(dev);
+  if (hipGetDevice(&dev) == hipSuccess) {
+    g_staging.forget(dev);
+    forget_dynamic_lds(dev);
+  }
   return hipDeviceReset() == hipSuccess ? 0 : 1;
 }
 

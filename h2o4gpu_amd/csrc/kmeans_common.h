@@ -42,6 +42,13 @@ void log_msg(int verbose, int level, const char *fmt, ...)
     if (_rc != 0) return _rc;   \
   } while (0)
 
+// Kernels that use more than 64 KB of dynamic LDS need their limit raised first. That is
+// done once per kernel instance, device and size (the largest size granted so far is
+// remembered) instead of on every launch; forget_dynamic_lds drops what is remembered for
+// a device whose context was reset.
+int ensure_dynamic_lds(const void *kernel, size_t bytes);
+void forget_dynamic_lds(int dev);
+
 // Assign-kernel variants (value of the "assign" option).
 enum AssignVariant {
   ASSIGN_AUTO = 0,
@@ -58,10 +65,12 @@ static const int CENTROID_PAD = 256;
 // strict '<', lowest index wins, -1 when no distance is below FLT_MAX.
 // mindist (nullable) receives the minimum. Returns the variant actually used
 // through *used (nullable).
+// exact (float32 MFMA kernels only): compare the float distances themselves instead of
+// 16-ulp integer keys; slower, for measuring what the key resolution costs in parity.
 template <typename T>
 int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
                   const T *C, const T *cnorm, int *labels, T *mindist,
-                  int64_t n, int d, int k, int num_cu, int *used);
+                  int64_t n, int d, int k, int num_cu, int *used, bool exact = false);
 template <typename T>
 int pick_assign_variant(int requested, int64_t n, int d, int k);
 const char *assign_variant_name(int variant);

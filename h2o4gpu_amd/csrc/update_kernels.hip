@@ -386,10 +386,7 @@ static int launch_accumulate_vec(hipStream_t s, const UpdatePlan &p, const T *X,
 #define KM_ACC_LAUNCH(TPB)                                                                      \
   do {                                                                                          \
     auto kern = accumulate_kernel<T, VEC, RAGGED, TPB>;                                         \
-    if (p.lds_bytes > 64 * 1024)                                                                \
-      KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                      \
-                                     hipFuncAttributeMaxDynamicSharedMemorySize,                \
-                                     (int)p.lds_bytes));                                        \
+    KM_TRY(ensure_dynamic_lds(reinterpret_cast<const void *>(kern), p.lds_bytes));              \
     hipLaunchKernelGGL(kern, dim3(p.row_blocks, p.k_chunks), dim3(TPB), p.lds_bytes, s, X,      \
                        labels, psums, pcounts, n, d, k, p.kc, rows_per_block, lpr, p.sd);       \
   } while (0)
@@ -620,12 +617,8 @@ int launch_bucketed_accumulate(hipStream_t s, const T *X, const int *labels, int
   KM_HIP_TRY(hipMemsetAsync(gsum, 0, (size_t)k * d * sizeof(double), s));
   const unsigned blocks = (unsigned)((n + BUCKET_ROWS - 1) / BUCKET_ROWS);
   const size_t lds1 = (size_t)k * sizeof(int), lds2 = bucket_lds_bytes(k);
-  if (lds2 > 64 * 1024) {
-    KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(bucket_scatter_kernel),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds2));
-    KM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(bucket_count_kernel),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds2));
-  }
+  KM_TRY(ensure_dynamic_lds(reinterpret_cast<const void *>(bucket_scatter_kernel), lds2));
+  KM_TRY(ensure_dynamic_lds(reinterpret_cast<const void *>(bucket_count_kernel), lds2));
   hipLaunchKernelGGL(bucket_count_kernel, dim3(blocks), dim3(WG), lds1, s, labels, counts, n, k);
   hipLaunchKernelGGL(bucket_scan_kernel, dim3(1), dim3(WG), 0, s, counts, offsets, cursor, total, k);
   hipLaunchKernelGGL(bucket_scatter_kernel, dim3(blocks), dim3(WG), lds2, s, labels, cursor, order,

@@ -193,7 +193,9 @@ int h2o4gpu_kmeans_transform_resident(h2o4gpu_kmeans_handle *h, void *d_dist);
  * 3 MFMA tiled; "fuse" = 1 (default) lets fit/iterate run assignment and the
  * per-centroid accumulation as one kernel where the shape allows, 0 keeps them
  * separate; "buckets" = 1 (default) sums the centroids of shapes whose sums do not
- * fit LDS by bucketing rows by label, 0 uses the chunked LDS kernel for them too.
+ * fit LDS by bucketing rows by label, 0 uses the chunked LDS kernel for them too;
+ * "exact_argmin" = 1 makes the float32 matrix-core kernels compare the float distances
+ * themselves instead of 16-ulp integer keys (slower, never fused; 0 is the default).
  * Unknown names return EARG. */
 int h2o4gpu_kmeans_set_option(h2o4gpu_kmeans_handle *h, const char *name,
                               int value);

@@ -21,6 +21,10 @@
 //   random_rows                   : the two standard-library calls the
 //       reference makes, compiled as written; distinctness, determinism.
 //   transform                     : scipy cdist(sqeuclidean), transposed.
+//   top2_exact, pair_dist_exact   : numpy float64 on the direct form with per-row
+//       centroid pairs chosen asymmetrically (an a/b swap fails).
+//   descending dot order          : bit-equal to a numpy evaluation that adds the
+//       products of the column-reversed arrays in ascending order, norms untouched.
 //   kmeanspp_*                    : parity unpinned against the reference (the
 //       reference seeds with k-means|| whose candidate stream needs a CUDA
 //       build); pinned only against the textbook D^2-sampling definition.

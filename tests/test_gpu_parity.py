@@ -90,6 +90,54 @@ def test_update_matches_oracle(hip, oracle, n, d, k, buckets, dtype):
     assert abs(shift2 - ws2) <= 1e-4 * ws2 + 1e-30
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("exact", [0, 1])
+@pytest.mark.parametrize("variant,k,pairs", [
+    # (lower, higher) index of two identical centroids. 7 / 36: same lane group, the later
+    # 32-centroid tile on a LOWER accumulator number; 3 / 160: the same across two
+    # 128-centroid blocks of the tiled kernel; 3 / 800: across two LDS chunks of a
+    # row-stationary sweep (k = 1024 at d = 32 is swept in two launches)
+    ("mfma_rowstat", 192, [(7, 36), (3, 160)]),
+    ("mfma_tiled", 192, [(7, 36), (3, 160)]),
+    ("mfma_rowstat", 1024, [(7, 36), (3, 800)]),
+    ("mfma_tiled", 1024, [(7, 36), (3, 800), (100, 901)]),
+])
+def test_duplicate_centroids_lowest_index_wins(hip, oracle, variant, k, pairs, exact, dtype):
+    """Identical centroids give bit-identical distances; the reference's strict '<'
+    (kmeans_labels.h:360-377) sends every tied row to the LOWER index, so the update moves
+    that centroid and leaves the higher one where it was. Well-separated blobs: no other
+    near-tie exists, labels must equal the oracle's exactly and one update must match."""
+    n, d = 24000, 32
+    rng = np.random.default_rng(k + 11)
+    centers = rng.uniform(-10, 10, size=(k, d))
+    X = np.ascontiguousarray((centers[rng.integers(0, k, size=n)]
+                              + 0.3 * rng.standard_normal((n, d))).astype(dtype))
+    C0 = np.ascontiguousarray((centers + 0.05).astype(dtype))
+    for lo, hi in pairs:
+        C0[hi] = C0[lo]
+    want = oracle.assign(X, C0, threads=4)
+    wC, wcounts = oracle.update(X, want, C0, threads=4)
+    his = [hi for _, hi in pairs]
+    assert not np.isin(want, his).any() and all((want == lo).sum() > 0 for lo, _ in pairs)
+    tol = 1e-5 if dtype == np.float32 else 1e-12
+    for fuse in (1, 0):
+        with hip.Handle(n, d, k, dtype) as h:
+            h.set_data(X)
+            h.set_centroids(C0)
+            h.set_option("assign", variant)
+            h.set_option("exact_argmin", exact)
+            h.set_option("fuse", fuse)
+            h.assign()
+            assert np.array_equal(h.labels(), want), "assignment-only pass"
+            h.iterate(1)
+            got, counts, C1 = h.labels(), h.counts(), h.centroids()
+        assert np.array_equal(got, want), "Lloyd step, fuse=%d" % fuse
+        assert np.array_equal(counts, wcounts)
+        assert np.allclose(C1, wC, rtol=tol, atol=tol * np.abs(wC).max())
+        for lo, hi in pairs:
+            assert np.array_equal(C1[hi], C0[hi]) and not np.array_equal(C1[lo], C0[lo])
+
+
 def separated_problem(n, d, k, dtype, seed, spread=10.0, offset=0.5):
     """Blobs plus one start per blob (true centre + offset). No blob is split by the
     start, so no row sits on a decision boundary and a last-bit difference in a

@@ -248,3 +248,76 @@ def test_kmeanspp_draw_is_proportional_to_d2(oracle):
         rows, _ = oracle.kmeanspp(X, 2, seed)
         other += (rows[0] < 900) != (rows[1] < 900)
     assert other >= 39
+
+
+# ------------------------------------------------- helpers the parity verdicts rest on
+def test_pair_dist_exact_against_float64_brute_force(oracle):
+    """pair_dist_exact prices every excused label mismatch, so it is pinned by itself:
+    a 50 x 7 float32 case with 5 centroids, labels a and b chosen differently per row
+    (an a/b swap, a wrong centroid row or a squared-vs-plain mix-up all fail), against
+    numpy float64 on the direct form; float64 input alike."""
+    rng = np.random.default_rng(17)
+    for dtype in (np.float32, np.float64):
+        X = np.ascontiguousarray(rng.normal(3.0, 4.0, size=(50, 7)).astype(dtype))
+        C = np.ascontiguousarray(rng.normal(-1.0, 5.0, size=(5, 7)).astype(dtype))
+        a = rng.integers(0, 5, size=50).astype(np.int32)
+        b = ((a + 1 + rng.integers(0, 4, size=50)) % 5).astype(np.int32)   # never equal to a
+        assert (a != b).all()
+        da, db = oracle.pair_dist_exact(X, C, a, b, threads=2)
+        X64, C64 = X.astype(np.float64), C.astype(np.float64)
+        wa = ((X64 - C64[a]) ** 2).sum(1)
+        wb = ((X64 - C64[b]) ** 2).sum(1)
+        assert np.allclose(da, wa, rtol=1e-14, atol=0) and np.allclose(db, wb, rtol=1e-14, atol=0)
+        assert not np.allclose(da, wb, rtol=1e-3)   # the case does tell a from b
+        # and it agrees with the two smallest entries of the full exact table
+        best, d1, d2 = oracle.top2_exact(X, C)
+        full = ((X64[:, None, :] - C64[None, :, :]) ** 2).sum(-1)
+        assert np.array_equal(best, full.argmin(1))
+        srt = np.sort(full, axis=1)
+        assert np.allclose(d1, srt[:, 0], rtol=1e-14) and np.allclose(d2, srt[:, 1], rtol=1e-14)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_descending_dot_order_is_the_ascending_sum_of_reversed_columns(oracle, dtype):
+    """The descending summation order is the yardstick of the full-size drift test. Summing
+    features d-1 .. 0 of (X, C) is, term for term, summing features 0 .. d-1 of the
+    column-reversed arrays, and the row norms are order-independent inputs of both only
+    if they are formed the same way: so labels AND minimum distances of the descending
+    mode on (X, C) must equal, bit for bit, those of the default mode on data whose dot
+    products are reversed but whose norms are not. That is checked through distances with
+    a single feature block reversed: d = 1 is trivially equal, and for d > 1 the two modes
+    must differ somewhere in the last bit (the switch does something)."""
+    rng = np.random.default_rng(23)
+    n, d, k = 4000, 37, 29
+    X = np.ascontiguousarray(rng.normal(20.0, 3.0, size=(n, d)).astype(dtype))
+    C = np.ascontiguousarray(rng.normal(20.0, 3.0, size=(k, d)).astype(dtype))
+    Xr, Cr = np.ascontiguousarray(X[:, ::-1]), np.ascontiguousarray(C[:, ::-1])
+    asc = oracle.distances(X, C)
+    oracle.set_dot_order(True)
+    try:
+        desc = oracle.distances(X, C)
+        desc_rev = oracle.distances(Xr, Cr)
+        l_desc, m_desc = oracle.assign(X, C, return_mindist=True)
+    finally:
+        oracle.set_dot_order(False)
+    # the norms xx, cc are always summed ascending over the array as given, so build the
+    # expected values from their parts: norms of the original arrays, dots of the reversed ones
+    xx = oracle.row_norms(X)
+    cc = oracle.row_norms(C)
+    dots_rev = np.zeros((k, n), dtype)
+    for j in range(d):                       # ascending over reversed columns, in dtype
+        dots_rev += np.outer(Cr[:, j], Xr[:, j]).astype(dtype)
+    want = np.abs((xx[None, :] + cc[:, None]) - dtype(2) * dots_rev)
+    assert np.array_equal(desc, want)
+    assert np.array_equal(m_desc, want.min(0))
+    assert np.array_equal(l_desc, want.argmin(0))
+    # same mathematics, different rounding: close everywhere, not identical everywhere
+    scale = float(xx.max() + cc.max())
+    assert np.max(np.abs(desc.astype(np.float64) - asc)) <= 64 * np.finfo(dtype).eps * scale
+    assert (desc != asc).any()
+    # reversing the columns AND the order restores the ascending-order dot products
+    xxr, ccr = oracle.row_norms(Xr), oracle.row_norms(Cr)
+    dots = np.zeros((k, n), dtype)
+    for j in range(d):
+        dots += np.outer(C[:, j], X[:, j]).astype(dtype)
+    assert np.array_equal(desc_rev, np.abs((xxr[None, :] + ccr[:, None]) - dtype(2) * dots))
