@@ -1193,6 +1193,97 @@ static int transform_entry(int verbose, int gpu_id, size_t rows, size_t cols, in
 
 
 // ---------------------------------------------------------------------------
+// C ABI, part 4: assignment of device-resident rows without any allocation
+// ---------------------------------------------------------------------------
+// Everything predict_host obtains from hipMalloc beyond the caller's inputs and outputs
+// (row norms, running minimum distances, the zero-padded copy of the centroids and their
+// norms) lives in this fixed array instead. Every device the library runs on holds its
+// own copy for the life of the process. In host code the name `scratch` is only a
+// stand-in for the symbol: the device address is asked for once per device and it is
+// that address, never the name, that kernels receive.
+static __device__ __align__(256) unsigned char scratch[H2O4GPU_KMEANS_NOALLOC_SCRATCH_BYTES];
+
+struct NoAllocDevice {
+  unsigned char *ptr = nullptr;  // device address of `scratch` on this device
+  int num_cu = 0;
+};
+static std::mutex g_noalloc_mu;
+static NoAllocDevice g_noalloc[StagingPool::MAX_DEV];
+static void forget_noalloc(int dev) {
+  std::lock_guard<std::mutex> lock(g_noalloc_mu);
+  if (dev >= 0 && dev < StagingPool::MAX_DEV) g_noalloc[dev] = NoAllocDevice();
+}
+
+// Cpad [kpad][d] = C [k][d] followed by zero rows; cnorm [k, kpad) = +inf.
+template <typename T>
+__global__ __launch_bounds__(256) void stage_model_kernel(const T *__restrict__ C, T *__restrict__ Cpad,
+                                                          T *__restrict__ cnorm, int k, int kpad, int d) {
+  const size_t kd = (size_t)k * d, total = (size_t)kpad * d;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  const size_t t0 = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  for (size_t e = t0; e < total; e += stride) Cpad[e] = e < kd ? C[e] : (T)0;
+  for (size_t c = (size_t)k + t0; c < (size_t)kpad; c += stride)
+    cnorm[c] = std::numeric_limits<T>::infinity();
+}
+
+// Address of this device's copy of `scratch` and the device's CU count, looked up on the
+// first call on a device (which must be current). A plain function, not a template: the
+// device compilation only gives a file-scope static variable a symbol the runtime can find
+// when it sees ordinary host code name it.
+static int noalloc_device(NoAllocDevice *out) {
+  int dev = 0;
+  KM_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= StagingPool::MAX_DEV) return H2O4GPU_KMEANS_EDEVICE;
+  std::lock_guard<std::mutex> lock(g_noalloc_mu);
+  if (!g_noalloc[dev].ptr) {
+    void *p = nullptr;
+    KM_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    hipDeviceProp_t prop;
+    KM_HIP_TRY(hipGetDeviceProperties(&prop, dev));
+    g_noalloc[dev].num_cu = prop.multiProcessorCount;
+    g_noalloc[dev].ptr = static_cast<unsigned char *>(p);
+  }
+  *out = g_noalloc[dev];
+  return 0;
+}
+
+template <typename T>
+static int predict_device_noalloc(size_t rows, size_t cols, int k, const T *dX, const T *dC,
+                                  int *d_labels, hipStream_t stream) {
+  NoAllocDevice nd;
+  KM_TRY(noalloc_device(&nd));
+  const int d = (int)cols;
+  const size_t kpad = ((size_t)k + CENTROID_PAD - 1) / CENTROID_PAD * CENTROID_PAD;
+  auto up = [](size_t b) { return (b + 255) / 256 * 256; };
+  const size_t b_model = up(kpad * cols * sizeof(T)), b_cnorm = up(kpad * sizeof(T));
+  const size_t b_rows = up(rows * sizeof(T));
+  const size_t need = b_model + b_cnorm + 2 * b_rows;
+  if (need > (size_t)H2O4GPU_KMEANS_NOALLOC_SCRATCH_BYTES) {
+    log_msg(LOG_ERROR, LOG_ERROR,
+            "predict_device_noalloc: rows=%zu cols=%zu k=%d need %zu bytes of scratch, the "
+            "library's fixed buffer holds %zu; split the rows or use a handle",
+            rows, cols, k, need, (size_t)H2O4GPU_KMEANS_NOALLOC_SCRATCH_BYTES);
+    return H2O4GPU_KMEANS_ESCRATCH;
+  }
+  T *Cpad = reinterpret_cast<T *>(nd.ptr);
+  T *cnorm = reinterpret_cast<T *>(nd.ptr + b_model);
+  T *xnorm = reinterpret_cast<T *>(nd.ptr + b_model + b_cnorm);
+  T *mind = reinterpret_cast<T *>(nd.ptr + b_model + b_cnorm + b_rows);
+  // the array keeps the previous call's contents: everything read below is written first
+  // (model rows and padding, all kpad norms, one norm per row; the running minimum is
+  // written before it is read by every kernel that uses it)
+  const size_t total = kpad * cols;
+  const unsigned blocks = (unsigned)std::min<size_t>((total + 255) / 256, 2048);
+  hipLaunchKernelGGL((stage_model_kernel<T>), dim3(blocks), dim3(256), 0, stream, dC, Cpad, cnorm, k,
+                     (int)kpad, d);
+  KM_HIP_TRY(hipGetLastError());
+  KM_TRY(launch_row_norms<T>(stream, Cpad, cnorm, k, d));
+  KM_TRY(launch_row_norms<T>(stream, dX, xnorm, (int64_t)rows, d));
+  return launch_assign<T>(stream, ASSIGN_AUTO, dX, xnorm, Cpad, cnorm, d_labels, mind, (int64_t)rows, d,
+                          k, nd.num_cu, nullptr);
+}
+
+// ---------------------------------------------------------------------------
 // C ABI, part 3
 // ---------------------------------------------------------------------------
 extern "C" {
@@ -1467,6 +1558,22 @@ KM_API int h2o4gpu_kmeans_copy_probe(int gpu_id, size_t bytes, int reps, float *
   return rc;
 }
 
+KM_API int h2o4gpu_kmeans_predict_device_noalloc(int elem_size, size_t rows, size_t cols, int k,
+                                                 const void *d_X, const void *d_centroids,
+                                                 int *d_labels, void *stream) {
+  if (!d_X || !d_centroids || !d_labels || rows < 1 || cols < 1 || k < 1 ||
+      rows > 2147483647ull || cols > 1000000ull)
+    return H2O4GPU_KMEANS_EARG;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (elem_size == 4)
+    return predict_device_noalloc<float>(rows, cols, k, static_cast<const float *>(d_X),
+                                         static_cast<const float *>(d_centroids), d_labels, s);
+  if (elem_size == 8)
+    return predict_device_noalloc<double>(rows, cols, k, static_cast<const double *>(d_X),
+                                          static_cast<const double *>(d_centroids), d_labels, s);
+  return H2O4GPU_KMEANS_EARG;
+}
+
 KM_API int make_ptr_float_kmeans(int dopredict, int verbose, int seed, int gpu_id, int n_gpu,
                                  size_t mTrain, size_t n, int k, int max_iterations,
                                  int init_from_data, float threshold, const float *srcdata,
@@ -1563,6 +1670,7 @@ KM_API int cudaresetdevice(int wDev, int nDev) {
   if (hipSetDevice(wDev) != hipSuccess) return 1;
   g_staging.forget(wDev);
   forget_dynamic_lds(wDev);
+  forget_noalloc(wDev);
   return hipDeviceReset() == hipSuccess ? 0 : 1;
 }
 KM_API int cudaresetdevice_bare(void) {
@@ -1570,6 +1678,7 @@ KM_API int cudaresetdevice_bare(void) {
   if (hipGetDevice(&dev) == hipSuccess) {
     g_staging.forget(dev);
     forget_dynamic_lds(dev);
+    forget_noalloc(dev);
   }
   return hipDeviceReset() == hipSuccess ? 0 : 1;
 }

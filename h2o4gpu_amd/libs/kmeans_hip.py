@@ -70,7 +70,11 @@ PROTOTYPES = {
     "h2o4gpu_kmeans_kernel_time": (c_int, [c_void_p, c_char_p, P(c_int), P(c_double)]),
     "h2o4gpu_kmeans_assign_variant": (c_char_p, [c_void_p]),
     "h2o4gpu_kmeans_copy_probe": (c_int, [c_int, c_size_t, c_int, P(c_float)]),
+    "h2o4gpu_kmeans_predict_device_noalloc": (c_int, [c_int, c_size_t, c_size_t, c_int, c_void_p,
+                                                      c_void_p, c_void_p, c_void_p]),
 }
+
+NOALLOC_SCRATCH_BYTES = 16 << 20
 
 _lib = None
 _libc = None
@@ -81,7 +85,7 @@ class KMeansHipError(RuntimeError):
 
     def __init__(self, fn, code):
         names = {-1: "allocation failed", -2: "bad argument", -3: "HIP device error",
-                 -4: "call order / missing state"}
+                 -4: "call order / missing state", -5: "beyond the fixed scratch buffer"}
         RuntimeError.__init__(self, "%s returned %d (%s)" % (fn, code, names.get(code, "?")))
         self.code = code
 
@@ -310,3 +314,12 @@ def last_fit_info():
 
 def device_count():
     return int(lib().h2o4gpu_kmeans_device_count())
+
+
+def predict_device_noalloc(dtype, rows, cols, k, d_X, d_centroids, d_labels, stream=None):
+    """Queues the assignment of device-resident rows (raw device addresses) on `stream`
+    without allocating anything; see part 4 of the C header."""
+    rc = lib().h2o4gpu_kmeans_predict_device_noalloc(np.dtype(dtype).itemsize, int(rows), int(cols),
+                                                     int(k), c_void_p(d_X), c_void_p(d_centroids),
+                                                     c_void_p(d_labels), c_void_p(stream))
+    _check("predict_device_noalloc", rc)

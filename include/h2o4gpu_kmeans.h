@@ -26,6 +26,7 @@ extern "C" {
 #define H2O4GPU_KMEANS_EARG (-2)     /* bad argument */
 #define H2O4GPU_KMEANS_EDEVICE (-3)  /* HIP runtime error / no usable device */
 #define H2O4GPU_KMEANS_ESTATE (-4)   /* call order (e.g. fit before data) */
+#define H2O4GPU_KMEANS_ESCRATCH (-5) /* input beyond the fixed scratch of a no-allocation call */
 
 /* ---------------------------------------------------------------------------
  * Part 1 - drop-in entry points.
@@ -219,6 +220,34 @@ const char *h2o4gpu_kmeans_assign_variant(h2o4gpu_kmeans_handle *h);
  * copy (used to calibrate byte counters and to report achievable HBM rate). */
 int h2o4gpu_kmeans_copy_probe(int gpu_id, size_t bytes, int reps,
                               float *milliseconds);
+
+/* ---------------------------------------------------------------------------
+ * Part 4 - assignment without any allocation.
+ * No counterpart in the reference. For callers that cannot allocate device
+ * memory: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc. Same result as h2o4gpu_kmeans_predict_host on the same rows
+ * and centroids: d_labels[i] = index of the nearest of the k centroids
+ * (d_centroids [k][cols]) to row i of d_X [rows][cols]; all three live in
+ * device memory of the CURRENT device and are only element-aligned at least.
+ * The work is queued on `stream` (a hipStream_t, NULL = the default stream) and
+ * the call returns without waiting for it. It calls no hipMalloc / hipFree and
+ * creates no stream or event: row norms, running minima, the padded copy of the
+ * centroids and their norms live in one fixed array of
+ * H2O4GPU_KMEANS_NOALLOC_SCRATCH_BYTES inside the library (one copy per device,
+ * held until the process ends). Needed:
+ *   round256(roundup(k,256)*cols*elem) + round256(roundup(k,256)*elem)
+ *   + 2*round256(rows*elem) bytes;
+ * more returns H2O4GPU_KMEANS_ESCRATCH and queues nothing. All calls on one
+ * device share that array: calls that overlap in time on one device (other
+ * threads, other streams) race; serialise them. The first call on a device
+ * looks up the array's address and the device's properties and should be made
+ * outside graph capture.
+ * ------------------------------------------------------------------------- */
+#define H2O4GPU_KMEANS_NOALLOC_SCRATCH_BYTES (16u << 20)
+int h2o4gpu_kmeans_predict_device_noalloc(int elem_size, size_t rows, size_t cols,
+                                          int k, const void *d_X,
+                                          const void *d_centroids, int *d_labels,
+                                          void *stream);
 
 #ifdef __cplusplus
 }

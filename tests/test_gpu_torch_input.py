@@ -15,7 +15,9 @@ def test_device_tensors_give_the_results_of_host_arrays(hip):
     """Runs in a child process so that PyTorch's copy of the HIP runtime is loaded
     before the engine there and never into this process (a first import of torch on a
     fresh machine can take minutes, hence the long limit)."""
-    pytest.importorskip("torch")
+    import importlib.util
+    if importlib.util.find_spec("torch") is None:   # (looked up, not imported, see above)
+        pytest.skip("PyTorch is not installed")
     proc = subprocess.run([sys.executable, os.path.join(HERE, "torch_device_input_check.py")],
                           capture_output=True, text=True, timeout=850)
     assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-4000:]
