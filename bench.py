@@ -6,7 +6,7 @@ update) over the whole resident data set. The default workload is the headline
 shape: 10,000,000 x 32 float32 Gaussian blobs, k = 256, seeded-random row
 initialisation. Prints one JSON line.
 
-    python bench.py [--gpus 1] [--steps 30] [--warmup 3] [--workload C3]
+    python bench.py [--gpus 1] [--steps 30] [--warmup 3] [--workload C3] [--no-traffic]
 """
 import argparse
 import json
@@ -25,18 +25,88 @@ from h2o4gpu_amd.libs import kmeans_hip  # noqa: E402
 PEAK_HBM_GBPS = 8000.0
 PEAK_MFMA_TFLOPS = {"f32": 157.3, "f64": 78.6}
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE runs of this script (profiles/assign_accumulate_rowstat_c3.md): raw
-# counter x calibration factor of a plain 1 GiB copy kernel (2.0 for FETCH_SIZE,
-# 1.0 for WRITE_SIZE on this box). Keyed by (workload, dtype, kernel); other
-# combinations report null.
-MEASURED_TRAFFIC_BYTES = {
-    ("C3", "f32", "assign_accumulate"): (644709 * 2.0 + 94765 * 1.0) * 1024.0,
-    # tiled kernel: the row slice is re-read once per 128-centroid block and misses L2
-    # (profiles/assign_tiled_c4.md); the figure is L2-miss traffic, HBM or memory-side cache
-    ("C4", "f32", "assign"): (7342683 * 2.0 + 15625 * 1.0) * 1024.0,
-    ("C5", "f32", "assign"): (25662000 * 2.0 + 3906 * 1.0) * 1024.0,
+WORKLOAD_TEXT = {
+    "C1": "Gaussian blobs, seeded-random row start",
+    "C2": "Gaussian blobs (Dirichlet sizes), seeded-random row start",
+    "C3": "Gaussian blobs (equal sizes), seeded-random row start",
+    "C4": "Gaussian blobs + 10% uniform outliers, k-means++ start from a fixed seed",
+    "C5": "image-like rows (70% zeros, integers 1..255), seeded-random row start",
 }
+
+
+def measure_traffic(argv_tail, timeout_s=240):
+    """HBM bytes per launch of the Lloyd-step kernel of this very workload, measured now:
+    two child runs of this script under `rocprofv3 --pmc` (FETCH_SIZE, then WRITE_SIZE, KiB
+    per dispatch), each scaled by what the same counter reads for the library's plain copy
+    kernel of 1 GiB in the same run. Must be called before this process touches the GPU.
+    Returns (bytes or None, details)."""
+    import csv
+    import glob
+    import shutil
+    import subprocess
+    import tempfile
+    rocprof = shutil.which("rocprofv3") or "/opt/rocm/bin/rocprofv3"
+    if not os.path.exists(rocprof):
+        return None, {"skipped": "rocprofv3 not found"}
+    if any(key.startswith(("ROCPROF", "ROCP_")) for key in os.environ):
+        return None, {"skipped": "this run is itself being profiled"}
+    details = {}
+    total = 0.0
+    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+        tmp = tempfile.mkdtemp(prefix="km_traffic_", dir="/tmp")
+        cmd = [rocprof, "--pmc", counter, "--output-format", "csv", "-d", tmp, "-o", "x", "--",
+               sys.executable, os.path.abspath(__file__), "--traffic-child"] + argv_tail
+        env = dict(os.environ, TMPDIR="/tmp")
+        try:
+            proc = subprocess.run(cmd, cwd="/tmp", env=env, stdout=subprocess.PIPE,
+                                  stderr=subprocess.STDOUT, timeout=timeout_s)
+            files = glob.glob(os.path.join(tmp, "**", "*counter_collection.csv"), recursive=True)
+            if proc.returncode != 0 or not files:
+                return None, {"skipped": "%s pass failed (rc %d)" % (counter, proc.returncode)}
+            per_kernel = {}
+            for row in csv.DictReader(open(files[0])):
+                if row["Counter_Name"] != counter:
+                    continue
+                per_kernel.setdefault(row["Kernel_Name"], []).append(float(row["Counter_Value"]))
+        except Exception as exc:  # pylint: disable=broad-except
+            return None, {"skipped": "%s pass: %r" % (counter, exc)}
+        finally:
+            shutil.rmtree(tmp, ignore_errors=True)
+        copy = [v for name, v in per_kernel.items() if "copy_probe_kernel" in name]
+        step = [(len(v), name, v) for name, v in per_kernel.items()
+                if ("assign_" in name or "lloyd_valu" in name)]
+        if not copy or not step:
+            return None, {"skipped": "%s pass: kernels not found" % counter}
+        # the Lloyd-step kernel is the assign/step kernel with the most dispatches
+        _, name, vals = max(step)
+        copy_kib = sum(copy[0]) / len(copy[0])
+        factor = (1 << 20) / copy_kib            # the copy kernel reads and writes 1 GiB = 2^20 KiB
+        kib = sum(vals) / len(vals)
+        details[counter] = {"kernel": name.split("(")[0][-90:], "raw_kib_per_dispatch": kib,
+                            "copy_kernel_raw_kib": copy_kib, "scale": factor, "dispatches": len(vals)}
+        total += kib * factor * 1024.0
+    return total, details
+
+
+def traffic_child(args):
+    """The run the counters are read from: a few Lloyd steps of the workload plus the copy
+    kernel that calibrates the counter."""
+    dtype = np.float32 if args.dtype == "f32" else np.float64
+    X, k, _ = datasets.make(args.workload, args.scale, dtype)
+    n, d = X.shape
+    h = kmeans_hip.Handle(n, d, k, dtype)
+    h.set_data(X)
+    h.set_centroids(datasets.seeded_row_init(X, k, datasets.SHAPES[args.workload][3]))
+    h.set_option("assign", args.assign)
+    if args.no_fuse:
+        h.set_option("fuse", 0)
+    if args.exact_argmin:
+        h.set_option("exact_argmin", 1)
+    h.iterate(4)
+    h.assign()
+    h.close()
+    kmeans_hip.copy_probe(1 << 30, 2)
+    return 0
 
 
 def log(msg):
@@ -129,6 +199,8 @@ def main():
     ap.add_argument("--scale", type=float, default=1.0, help="row-count scale (1.0 = full shape)")
     ap.add_argument("--dtype", default="f32", choices=["f32", "f64"])
     ap.add_argument("--assign", default="auto", choices=sorted(kmeans_hip.ASSIGN_VARIANTS))
+    ap.add_argument("--exact-argmin", action="store_true",
+                    help="float32 matrix-core kernels: compare float distances instead of 16-ulp keys")
     ap.add_argument("--no-fuse", action="store_true",
                     help="keep assignment and accumulation as separate kernels")
     ap.add_argument("--transform-rows", type=int, default=0,
@@ -137,6 +209,9 @@ def main():
     ap.add_argument("--cpu-iters", type=int, default=0, help="CPU baseline iterations (0 = about 12 s worth)")
     ap.add_argument("--sklearn-rows", type=int, default=10_000_000,
                     help="rows of the workload the scikit-learn leg runs on")
+    ap.add_argument("--no-traffic", action="store_true",
+                    help="skip the two rocprofv3 counter passes behind roofline.traffic")
+    ap.add_argument("--traffic-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--no-end-to-end", dest="end_to_end", action="store_false",
                     help="skip the whole fit through make_ptr_*_kmeans (upload included, field c_abi_fit)")
     ap.add_argument("--end-to-end", dest="end_to_end", action="store_true", help=argparse.SUPPRESS)
@@ -147,6 +222,18 @@ def main():
         print("bench.py: this engine runs on one GPU; --gpus %d is not supported "
               "(collectives and sharding are not part of this build)" % args.gpus, file=sys.stderr)
         return 2
+    if args.traffic_child:
+        return traffic_child(args)
+    # the counter passes run in child processes, before this process initialises the GPU
+    traffic, traffic_details = None, {"skipped": "--no-traffic"}
+    if not args.no_traffic:
+        tail = ["--workload", args.workload, "--scale", str(args.scale), "--dtype", args.dtype,
+                "--assign", args.assign] + (["--no-fuse"] if args.no_fuse else []) + \
+               (["--exact-argmin"] if args.exact_argmin else [])
+        t0 = time.perf_counter()
+        traffic, traffic_details = measure_traffic(tail)
+        log("traffic passes: %s in %.1f s" % ("%.4g bytes per launch" % traffic if traffic else
+                                              traffic_details.get("skipped"), time.perf_counter() - t0))
     if kmeans_hip.device_count() < 1:
         print("bench.py: no HIP device visible", file=sys.stderr)
         return 3
@@ -155,7 +242,8 @@ def main():
     t0 = time.perf_counter()
     X, k, _ = datasets.make(args.workload, args.scale, dtype)
     n, d = X.shape
-    C0 = datasets.seeded_row_init(X, k, datasets.SHAPES[args.workload][3])
+    seed = datasets.SHAPES[args.workload][3]
+    C0 = datasets.seeded_row_init(X, k, seed)
     log("generated %s: %d x %d %s, k=%d in %.1f s" % (args.workload, n, d, X.dtype, k,
                                                     time.perf_counter() - t0))
     s = X.dtype.itemsize
@@ -169,10 +257,15 @@ def main():
     t0 = time.perf_counter()
     h.set_data(X)
     h2d_s = time.perf_counter() - t0
+    if args.workload == "C4":  # the benchmark text starts this shape from k-means++
+        h.init_plusplus(seed)
+        C0 = h.centroids()
     h.set_centroids(C0)
     h.set_option("assign", args.assign)
     if args.no_fuse:
         h.set_option("fuse", 0)
+    if args.exact_argmin:
+        h.set_option("exact_argmin", 1)
     variant = h.assign_variant()
     log("upload %.3f s (%.1f GB/s incl. pageable staging; first call of the process %.3f s); "
         "assign variant %s" % (h2d_s, n * d * s / h2d_s / 1e9, h2d_first_s, variant))
@@ -202,9 +295,6 @@ def main():
     tflops = flops_per_iter / (assign_ms * 1e-3) / 1e12
     peak = PEAK_MFMA_TFLOPS[args.dtype]
     mfma_bound = variant != "valu"
-    traffic = None
-    if args.scale == 1.0:
-        traffic = MEASURED_TRAFFIC_BYTES.get((args.workload, args.dtype, dom))
     if mfma_bound:
         roofline = {"bound": "mfma", "kernel": "%s (%s)" % (dom, variant), "achieved": tflops,
                     "peak": peak, "unit": "TFLOP/s", "frac": tflops / peak, "traffic": traffic}
@@ -213,7 +303,7 @@ def main():
         gbps = float(n) * (d * s + s + 4 + s) / (assign_ms * 1e-3) / 1e9
         roofline = {"bound": "hbm", "kernel": "%s (valu)" % dom, "achieved": gbps,
                     "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": gbps / PEAK_HBM_GBPS,
-                    "traffic": None}
+                    "traffic": traffic}
     iter_gbps = bytes_per_iter / (ms_step * 1e-3) / 1e9
     copy_bytes = 1 << 30
     copy_ms = kmeans_hip.copy_probe(copy_bytes, 10)
@@ -242,10 +332,11 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic",
-        "config": {"workload": "%s: %d x %d %s Gaussian blobs, k=%d, seeded-random row init, "
-                               "one step = assign + centroid update" % (args.workload, n, d, args.dtype, k),
+        "config": {"workload": "%s: %d x %d %s, k=%d, %s; one step = assign + centroid update"
+                               % (args.workload, n, d, args.dtype, k, WORKLOAD_TEXT[args.workload]),
                    "rows": n, "cols": d, "k": k, "assign_variant": variant},
         "roofline": roofline,
+        "traffic_measurement": traffic_details,
         "iteration": {"algorithmic_bytes": bytes_per_iter, "algorithmic_flops": flops_per_iter,
                       "gbps": iter_gbps, "hbm_frac": iter_gbps / PEAK_HBM_GBPS,
                       "tflops": flops_per_iter / (ms_step * 1e-3) / 1e12,

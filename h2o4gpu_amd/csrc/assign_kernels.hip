@@ -1457,6 +1457,11 @@ static int launch_tiled_bcw(hipStream_t s, const T *X, const T *xnorm, const T *
     hipLaunchKernelGGL(kern, grid, dim3(Cfg::TPB), lds, s, X, xnorm, C, cnorm, labels,       \
                        mindist, D, n, ldn, d, k);                                            \
   } while (0)
+  // From 128 features on the float32 argmin compares the distances themselves: the
+  // epilogue is then about one per cent of the matrix work (2M x 256, k = 1024: 8.30 ->
+  // 8.37 ms; 500k x 784, k = 4096: 26.5 -> 26.9 ms), and on data whose distances are
+  // close to whole numbers the 16-ulp keys flipped four times as many near-tie rows.
+  if (d >= 128) exact = true;
 #define KM_TILED(VEC, TAIL)                                      \
   do {                                                           \
     if constexpr (MODE == 0 && sizeof(T) == 4) {                 \

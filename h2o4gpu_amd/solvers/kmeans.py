@@ -95,6 +95,14 @@ def assert_satisfies(value, cond, message):
         raise ValueError("%s (got %r)" % (message, value))
 
 
+def _clusterer_tags():
+    """scikit-learn's estimator tags (1.6 and later ask every estimator for them; the two
+    classes here do not inherit BaseEstimator, as in the reference)."""
+    from sklearn.utils import Tags, TargetTags, TransformerTags
+    return Tags(estimator_type="clusterer", target_tags=TargetTags(required=False),
+                transformer_tags=TransformerTags())
+
+
 class KMeansH2O:
     """K-Means on the GPU (reference class KMeansH2O, kmeans.py:18-588)."""
 
@@ -132,6 +140,9 @@ class KMeansH2O:
         self.n_iter_ = None
         self.sklearn_model = None
         self.double_precision = 0
+
+    def __sklearn_tags__(self):
+        return _clusterer_tags()
 
     _PARAMS = ["algorithm", "copy_x", "do_checks", "gpu_id", "init", "max_iter", "n_clusters", "n_gpus",
                "n_init", "n_jobs", "precompute_distances", "random_state", "tol", "verbose"]
@@ -197,7 +208,13 @@ class KMeansH2O:
                 inertia = h.inertia() if self._max_iter > 0 else None
                 if best is None or (inertia is not None and inertia < best[2]):
                     best = (h.centroids(), h.labels(), inertia, n_iter)
-        self.cluster_centers_, self.labels_, self.inertia_, self.n_iter_ = best
+        centers, self.labels_, self.inertia_, self.n_iter_ = best
+        if k < self._n_clusters:
+            # more clusters asked for than rows: the fit ran with k = rows (kmeans_h2o4gpu.cu:630-635);
+            # the result keeps n_clusters rows, the rest zero, exactly as the host path leaves its
+            # preallocated array, so predict / transform see one shape whichever path fitted
+            centers = np.concatenate([centers, np.zeros((self._n_clusters - k, dev.cols), centers.dtype)])
+        self.cluster_centers_ = centers
         return self.cluster_centers_, self.labels_
 
     def sklearn_fit(self, X, y=None):
@@ -227,8 +244,9 @@ class KMeansH2O:
         cluster_centers_ = self._toc(self.cluster_centers_, convert=False)
         c_res = np.zeros(rows, np.int32)
         c_kmeans = lib.make_ptr_float_kmeans if self.double_precision == 0 else lib.make_ptr_double_kmeans
+        k = int(self.cluster_centers_.shape[0])  # (== n_clusters after fit; the array decides)
         status = c_kmeans(1, self.verbose, self.random_state, self._gpu_id, self.n_gpus, rows, cols,
-                          self._n_clusters, self._max_iter, 0, self.tol, c_X_np, cluster_centers_,
+                          k, self._max_iter, 0, self.tol, c_X_np, cluster_centers_,
                           np.empty([], X_np.dtype), c_res)
         if status:
             raise RuntimeError("KMeans predict failed in the native library (status %d)" % status)
@@ -250,20 +268,21 @@ class KMeansH2O:
         X_np = _to_np(X)
         c_X_np = self._toc(X_np)
         cluster_centers_ = self._toc(self.cluster_centers_, convert=False)
+        k = int(self.cluster_centers_.shape[0])  # (== n_clusters after fit; the array decides)
         owned = getattr(lib, "kmeans_transform_owned", None)
         if owned is not None:  # adopt the library's buffer instead of zero-filling and copying
-            status, c_res = owned(self.verbose, self._gpu_id, self.n_gpus, rows, cols, self._n_clusters,
+            status, c_res = owned(self.verbose, self._gpu_id, self.n_gpus, rows, cols, k,
                                   c_X_np, cluster_centers_, X_np.dtype)
             if status != 0:
                 raise RuntimeError("KMeans transform failed in the native library (status %d)" % status)
-            return np.reshape(c_res, (rows, self._n_clusters), order='F')
-        c_res = np.zeros(rows * self._n_clusters, X_np.dtype)
+            return np.reshape(c_res, (rows, k), order='F')
+        c_res = np.zeros(rows * k, X_np.dtype)
         fn = lib.kmeans_transform_float if self.double_precision == 0 else lib.kmeans_transform_double
-        status = fn(self.verbose, self._gpu_id, self.n_gpus, rows, cols, self._n_clusters, c_X_np,
+        status = fn(self.verbose, self._gpu_id, self.n_gpus, rows, cols, k, c_X_np,
                     cluster_centers_, c_res)
         if status:
             raise RuntimeError("KMeans transform failed in the native library (status %d)" % status)
-        return np.reshape(c_res, (rows, self._n_clusters), order='F')
+        return np.reshape(c_res, (rows, k), order='F')
 
     def _transform_device(self, X, dev):
         """Distances of device rows, left on the device: a (rows, k) view of the engine's
@@ -358,7 +377,7 @@ class KMeansH2O:
         X_np = _to_np(X)
         dtype = np.float64 if X_np.dtype == np.float64 else np.float32
         X_np = np.ascontiguousarray(X_np, dtype=dtype)
-        with kmeans_hip.Handle(X_np.shape[0], X_np.shape[1], self._n_clusters, dtype,
+        with kmeans_hip.Handle(X_np.shape[0], X_np.shape[1], int(self.cluster_centers_.shape[0]), dtype,
                                gpu_id=self._gpu_id, verbose=self.verbose) as h:
             h.set_data(X_np)
             h.set_centroids(np.ascontiguousarray(self.cluster_centers_, dtype=dtype))
@@ -451,6 +470,14 @@ class KMeans:
         _backend = os.environ.get('H2O4GPU_BACKEND', None)
         if _backend is not None:
             backend = _backend
+        self._backend_arg = backend
+        # constructor arguments as given: what get_params reports, so that
+        # KMeans(**est.get_params()) rebuilds the same selection (sklearn.base.clone)
+        self._ctor_args = dict(n_clusters=n_clusters, init=init, n_init=n_init, max_iter=max_iter, tol=tol,
+                               precompute_distances=precompute_distances, verbose=verbose,
+                               random_state=random_state, copy_x=copy_x, n_jobs=n_jobs,
+                               algorithm=algorithm, gpu_id=gpu_id, n_gpus=n_gpus, do_checks=do_checks,
+                               backend=backend)
         self.do_sklearn = backend == 'sklearn'
         self.model_h2o4gpu = KMeansH2O(n_clusters=n_clusters, init=init, n_init=n_init, max_iter=max_iter,
                                        tol=tol, precompute_distances=precompute_distances,
@@ -505,7 +532,13 @@ class KMeans:
         return res
 
     def get_params(self, deep=True):
-        return self.model.get_params(deep)
+        # the selector's own constructor arguments, refreshed from the selected model for
+        # the ones it knows (set_params or attribute assignment may have changed them)
+        params = dict(self._ctor_args)
+        for key, value in self.model.get_params(deep).items():
+            if key in params and key not in ("n_gpus", "random_state", "tol"):
+                params[key] = value
+        return params
 
     def predict(self, X):
         res = self.model.predict(X)
@@ -517,9 +550,24 @@ class KMeans:
         return self.model.score(X, y)
 
     def set_params(self, **params):
-        res = self.model.set_params(**params)
+        params = dict(params)
+        if "backend" in params:
+            # the backend is chosen at construction; the same value is accepted silently
+            backend = params.pop("backend")
+            if backend != self._backend_arg:
+                raise ValueError("backend is fixed at construction (%r); build a new KMeans for %r"
+                                 % (self._backend_arg, backend))
+        known = self.model.get_params(deep=False)
+        unknown = [key for key in params if key not in self._ctor_args]
+        if unknown:
+            raise ValueError("Invalid parameter %s for estimator KMeans." % unknown[0])
+        self.model.set_params(**{key: value for key, value in params.items() if key in known})
+        self._ctor_args.update(params)
         self.set_attributes()
-        return res
+        return self
+
+    def __sklearn_tags__(self):
+        return _clusterer_tags()
 
     def transform(self, X):
         res = self.model.transform(X)

@@ -44,7 +44,8 @@ def label_report(oracle, X, C, got, want, gap_rtol=GAP_RTOL, noise_mult=NOISE_MU
     assert got.shape == want.shape
     bad = np.nonzero(got != want)[0]
     rep = {"rows": int(got.size), "mismatch": int(bad.size), "excused": 0,
-           "excused_by_gap": 0, "excused_by_noise_floor": 0, "worst_gap": 0.0}
+           "excused_by_gap": 0, "excused_by_noise_floor": 0, "worst_gap": 0.0,
+           "worst_floor_mult": 0.0}
     if bad.size == 0:
         return rep
     assert (got[bad] >= 0).all() and (got[bad] < C.shape[0]).all(), "label out of range"
@@ -60,6 +61,9 @@ def label_report(oracle, X, C, got, want, gap_rtol=GAP_RTOL, noise_mult=NOISE_MU
     by_gap = gap <= gap_rtol
     by_floor = ~by_gap & (diff <= floor)
     rep["worst_gap"] = float(gap.max())
+    # largest |da - db| of a mismatch in units of eps * (|x|^2 + |c|^2): how much of the
+    # noise-floor allowance (noise_mult of these units) is actually used
+    rep["worst_floor_mult"] = float((diff / (floor / noise_mult)).max())
     rep["excused_by_gap"] = int(by_gap.sum())
     rep["excused_by_noise_floor"] = int(by_floor.sum())
     rep["excused"] = rep["excused_by_gap"] + rep["excused_by_noise_floor"]
@@ -68,3 +72,17 @@ def label_report(oracle, X, C, got, want, gap_rtol=GAP_RTOL, noise_mult=NOISE_MU
         "%d of %d label mismatches are not near-ties (worst relative gap %.3e), first rows %s"
         % (real.size, bad.size, gap[~(by_gap | by_floor)].max(), real[:5]))
     return rep
+
+
+def record(entry):
+    """Appends one JSON line to gpurun_out/parity_report.jsonl (the per-configuration
+    parity table is assembled from these); never fails a test."""
+    import json
+    import os
+    try:
+        out = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out")
+        os.makedirs(out, exist_ok=True)
+        with open(os.path.join(out, "parity_report.jsonl"), "a") as f:
+            f.write(json.dumps(entry) + "\n")
+    except OSError:
+        pass

@@ -1,14 +1,16 @@
 """The five benchmark shapes on the GPU.
 
 Scaled-down rows (same d and k) are checked against the CPU oracle in lock-step and
-end-to-end; the full shapes are checked through size-independent properties plus an
-oracle check on a random sample of rows, so the CPU side stays within seconds.
+end-to-end over the full iteration count; the full shapes are checked in lock-step on ALL
+rows (one oracle assignment costs seconds at most), end to end for as many iterations as
+the CPU side affords, and through size-independent properties. Every full-size run
+appends its near-tie accounting to gpurun_out/parity_report.jsonl.
 """
 import numpy as np
 import pytest
 
 from h2o4gpu_amd import datasets
-from parity import assert_centroids_close, centroid_err, label_report
+from parity import assert_centroids_close, centroid_err, label_report, record
 
 pytestmark = pytest.mark.gpu
 
@@ -44,14 +46,18 @@ def test_scaled_shape_lockstep_and_end_to_end(hip, oracle, name, dtype, scale, i
         variant = h.assign_variant()
         # lock-step: both sides start every iteration from the oracle's centroids
         C = C0.copy()
-        excused = mism = 0
+        excused = mism = by_gap = by_floor = self_mism = 0
         for it in range(min(iters, 6)):
             h.set_centroids(C)
             h.iterate(1)
             labels = h.labels()
-            rep = label_report(oracle, X, C, labels, oracle.assign(X, C, threads=8))
+            want = oracle.assign(X, C, threads=8)
+            rep = label_report(oracle, X, C, labels, want)
             excused += rep["excused"]
             mism += rep["mismatch"]
+            by_gap += rep["excused_by_gap"]
+            by_floor += rep["excused_by_noise_floor"]
+            self_mism += int((_oracle_labels(oracle, X, C, descending=True)[0] != want).sum())
             wC, wcounts = oracle.update(X, labels, C)
             assert np.array_equal(h.counts(), wcounts)
             assert np.allclose(h.centroids(), wC, rtol=tol, atol=tol * np.abs(wC).max())
@@ -66,6 +72,14 @@ def test_scaled_shape_lockstep_and_end_to_end(hip, oracle, name, dtype, scale, i
     err = centroid_err(Cg, wC)
     rep = label_report(oracle, X, wC, Lg, wL, gap_rtol=1.0)   # report only, see below
     w_inertia = float(oracle.assign(X, wC, threads=8, return_mindist=True)[1].astype(np.float64).sum())
+    # near-tie flips stay of the order of the oracle's own sensitivity to summation order
+    assert mism <= 3 * self_mism + 20, (mism, self_mism)
+    record({"config": name + " scaled", "dtype": np.dtype(dtype).name, "n": n, "d": d, "k": k,
+            "variant": variant, "lockstep_iterations": min(iters, 6), "lockstep_mismatch": mism,
+            "excused_by_gap": by_gap, "excused_by_noise_floor": by_floor,
+            "oracle_desc_vs_asc_mismatch": self_mism, "end_to_end_iterations": iters,
+            "end_to_end_centroid_err": err, "end_to_end_label_diffs": rep["mismatch"],
+            "inertia_rel_diff": abs(inertia - w_inertia) / w_inertia})
     print("%s %s n=%d d=%d k=%d [%s]: lockstep mismatches %d (all excused near-ties: %d); "
           "end-to-end centroid error %.2e, label mismatches %d, inertia rel diff %.2e"
           % (name, np.dtype(dtype).name, n, d, k, variant, mism, excused, err, rep["mismatch"],
@@ -79,15 +93,143 @@ def test_scaled_shape_lockstep_and_end_to_end(hip, oracle, name, dtype, scale, i
     assert abs(inertia - w_inertia) <= 1e-4 * w_inertia
 
 
-def _full_shape_checks(hip, oracle, name, dtype, iters, extra=None):
+THREADS = 16
+
+
+def _oracle_labels(oracle, X, C, descending=False):
+    if descending:
+        oracle.set_dot_order(True)
+    try:
+        return oracle.assign(X, C, threads=THREADS, return_mindist=True)
+    finally:
+        oracle.set_dot_order(False)
+
+
+def _lockstep_all_rows(hip, oracle, h, X, C, dtype, where):
+    """One Lloyd step from the centroids C on ALL rows, engine and oracle side by side.
+    Every label mismatch is priced by label_report (near-tie by the 1e-5 gap rule or inside
+    the rounding floor of the expanded form, anything else fails). Three yardsticks are taken
+    with the same report: the oracle against itself with the features summed in descending
+    order (how many rows flip between two CORRECT evaluations), and, for float32 models on
+    the matrix cores, the engine's exact-compare epilogue (what the 16-ulp keys add)."""
+    tol = 1e-5 if dtype == np.float32 else 1e-12
+    h.set_option("exact_argmin", 0)
+    h.set_centroids(C)
+    h.iterate(1)
+    L, counts, C1 = h.labels(), h.counts(), h.centroids()
+    wL, wM = _oracle_labels(oracle, X, C)
+    rep = label_report(oracle, X, C, L, wL)
+    rL, _ = _oracle_labels(oracle, X, C, descending=True)
+    self_rep = label_report(oracle, X, C, rL, wL)
+    out = {"where": where, "rows": int(X.shape[0]), "mismatch": rep["mismatch"],
+           "excused_by_gap": rep["excused_by_gap"], "excused_by_noise_floor": rep["excused_by_noise_floor"],
+           "worst_gap": rep["worst_gap"], "worst_floor_mult": rep["worst_floor_mult"],
+           "oracle_desc_vs_asc_mismatch": self_rep["mismatch"],
+           "oracle_desc_vs_asc_worst_gap": self_rep["worst_gap"],
+           "oracle_desc_vs_asc_worst_floor_mult": self_rep["worst_floor_mult"]}
+    if dtype == np.float32 and h.assign_variant() != "valu":
+        h.set_option("exact_argmin", 1)
+        h.set_centroids(C)
+        h.assign()
+        Lx = h.labels()
+        h.set_option("exact_argmin", 0)
+        xrep = label_report(oracle, X, C, Lx, wL)
+        out["exact_compare_mismatch"] = xrep["mismatch"]
+        out["keys_vs_exact_compare_flips"] = int((L != Lx).sum())
+        # the keys may add flips to those of an exact float32 compare, never subtract the
+        # bound: both stay within a small multiple of the oracle's own order sensitivity
+        assert xrep["mismatch"] <= 3 * self_rep["mismatch"] + 20, out
+    # the engine's flips are of the order of the oracle's own sensitivity to summation order
+    assert rep["mismatch"] <= 3 * self_rep["mismatch"] + 20, out
+    # given its labels the engine's update is the oracle's
+    wC_own, wcounts = oracle.update(X, L, C, threads=THREADS)
+    assert np.array_equal(counts, wcounts), where
+    assert np.allclose(C1, wC_own, rtol=tol, atol=tol * np.abs(wC_own).max()), where
+    # against the pure oracle step (its own labels): what the excused rows move
+    wC1, _ = oracle.update(X, wL, C, threads=THREADS)
+    out["step_centroid_err"] = centroid_err(C1, wC1)
+    rC1, _ = oracle.update(X, rL, C, threads=THREADS)
+    out["oracle_desc_vs_asc_step_centroid_err"] = centroid_err(rC1, wC1)
+    if rep["mismatch"] == 0:
+        assert_centroids_close(C1, wC1, dtype)
+    return out
+
+
+def _end_to_end_all_rows(hip, oracle, h, X, C0, dtype, iters, where):
+    """Fixed iteration count from the same start on all rows: engine (keys), engine with the
+    exact-compare epilogue, and the oracle with descending summation, each against the oracle."""
+    wC, wL, _, _ = oracle.lloyd(X, C0, iters, 0.0, threads=THREADS)
+    w_inertia = float(_oracle_labels(oracle, X, wC)[1].astype(np.float64).sum())
+    out = {"where": where, "iterations": iters}
+
+    def run(exact):
+        h.set_option("exact_argmin", exact)
+        h.set_centroids(C0)
+        assert h.fit(iters, 0.0) == iters
+        C, L, inertia = h.centroids(), h.labels(), h.inertia()
+        h.set_option("exact_argmin", 0)
+        return centroid_err(C, wC), int((L != wL).sum()), abs(inertia - w_inertia) / w_inertia, C
+
+    err, diffs, din, Cg = run(0)
+    out.update({"centroid_err": err, "label_diffs": diffs, "inertia_rel_diff": din})
+    if dtype == np.float32 and h.assign_variant() != "valu":
+        xerr, xdiffs, xdin, Cx = run(1)
+        out.update({"exact_compare_centroid_err": xerr, "exact_compare_label_diffs": xdiffs,
+                    "keys_vs_exact_compare_centroid_err": centroid_err(Cg, Cx)})
+    oracle.set_dot_order(True)
+    try:
+        rC, rL, _, _ = oracle.lloyd(X, C0, iters, 0.0, threads=THREADS)
+    finally:
+        oracle.set_dot_order(False)
+    out["oracle_desc_vs_asc_centroid_err"] = centroid_err(rC, wC)
+    out["oracle_desc_vs_asc_label_diffs"] = int((rL != wL).sum())
+    r_inertia = float(_oracle_labels(oracle, X, rC)[1].astype(np.float64).sum())
+    out["oracle_desc_vs_asc_inertia_rel_diff"] = abs(r_inertia - w_inertia) / w_inertia
+    record(dict(out, kind="end_to_end"))
+    tol = 1e-4 if dtype == np.float32 else 1e-9
+    # the stated bar whenever the trajectory is not chaotic by itself: two correct
+    # evaluations (oracle, both summation orders) that stay within it bind the engine to it
+    if out["oracle_desc_vs_asc_centroid_err"] <= tol and diffs == 0:
+        assert err <= tol, out
+    # otherwise (a start that splits blobs, clusters of a few rows): flipped near-tie rows
+    # move small clusters visibly and the trajectories drift; the engine must stay within
+    # a small multiple of the drift between the oracle's own two summation orders
+    assert err <= max(tol, 6 * out["oracle_desc_vs_asc_centroid_err"]), out
+    assert diffs <= 6 * out["oracle_desc_vs_asc_label_diffs"] + 100, out
+    assert din <= max(1e-5, 6 * out["oracle_desc_vs_asc_inertia_rel_diff"]), out
+    return out
+
+
+# name, dtype, Lloyd iterations of the benchmark text, iterations of the full-size run
+# against the oracle (the CPU side costs 0.05 s per iteration at C2, 10 s at C5)
+FULL = [
+    ("C1", np.float32, 20, 20),
+    ("C2", np.float32, 50, 50),
+    ("C3", np.float32, 30, 12),
+    ("C4", np.float32, 20, 3),
+    ("C4", np.float64, 20, 2),
+    ("C5", np.float32, 15, 2),
+]
+
+
+@pytest.mark.timeout(900)
+@pytest.mark.parametrize("name,dtype,iters,e2e_iters", FULL)
+def test_full_shape(hip, oracle, name, dtype, iters, e2e_iters):
+    """A benchmark configuration at its full size: lock-step against the oracle on all rows
+    at the start and at the fitted centroids, end to end for a fixed number of iterations,
+    and the size-independent properties of a fit (monotone objective, predict reproduces
+    the labels, counts add up, centroids are means). C5 also transforms 100,000 held-out rows."""
     X, k, _ = datasets.make(name, 1.0, dtype)
     n, d = X.shape
+    tag = "%s %s" % (name, np.dtype(dtype).name)
     rng = np.random.default_rng(99)
     with hip.Handle(n, d, k, dtype) as h:
         h.set_data(X)
         C0 = _start(name, X, k, h)
-        h.set_centroids(C0)
+        variant = h.assign_variant()
+        start = _lockstep_all_rows(hip, oracle, h, X, C0, dtype, tag + " start")
         # monotone objective over the first iterations
+        h.set_centroids(C0)
         prev = None
         for _ in range(3):
             h.assign()
@@ -97,23 +239,23 @@ def _full_shape_checks(hip, oracle, name, dtype, iters, extra=None):
             prev = cur
             h.update(want_shift=False)
         h.set_centroids(C0)
-        done = h.fit(iters, 0.0)
-        assert done == iters
+        assert h.fit(iters, 0.0) == iters
         C, L, counts = h.centroids(), h.labels(), h.counts()
         # final relabel used the final centroids: predicting the same rows gives the labels
         sub = np.sort(rng.choice(n, size=min(n, 20000), replace=False))
         assert np.array_equal(h.predict(X[sub]), L[sub])
-        # oracle on a sample of rows (exact up to near-ties)
-        rep = label_report(oracle, X[sub], C, L[sub], oracle.assign(X[sub], C, threads=8))
-        if extra:
-            extra(h, X, C, L)
+        # all rows against the oracle at the fitted centroids, then one more step from there
+        final_rep = label_report(oracle, X, C, L, _oracle_labels(oracle, X, C)[0])
+        fitted = _lockstep_all_rows(hip, oracle, h, X, C, dtype, tag + " fitted")
+        e2e = _end_to_end_all_rows(hip, oracle, h, X, C0, dtype, e2e_iters, tag)
+        if name == "C5":
+            h.set_centroids(C)  # (the end-to-end runs above left their own centroids behind)
+            _transform_check(h, C)
     assert L.min() >= 0 and L.max() < k
     # the last update's counts describe the labelling before the final relabel; they sum to n
     assert int(counts.sum()) == n
     # centroids are means of their rows: check a handful of clusters directly
     final_counts = np.bincount(L, minlength=k)
-    tol = 5e-4 if dtype == np.float32 else 1e-8
-    h2 = None
     for c in rng.choice(k, size=4, replace=False):
         rows = np.nonzero(L == c)[0]
         if rows.size == 0:
@@ -123,79 +265,31 @@ def _full_shape_checks(hip, oracle, name, dtype, iters, extra=None):
         # the two differ by at most the last shift, checked loosely
         scale = np.abs(mean).max() + np.sqrt(np.mean(C.astype(np.float64) ** 2))
         assert np.max(np.abs(C[c] - mean)) <= 0.05 * scale
-    print("%s %s full shape: n=%d d=%d k=%d, sample label check %s, empty clusters %d"
-          % (name, np.dtype(dtype).name, n, d, k, rep, int((final_counts == 0).sum())))
+    entry = {"config": name, "dtype": np.dtype(dtype).name, "n": n, "d": d, "k": k, "variant": variant,
+             "fit_iterations": iters, "final_relabel_mismatch": final_rep["mismatch"],
+             "final_relabel_excused_by_gap": final_rep["excused_by_gap"],
+             "final_relabel_excused_by_noise_floor": final_rep["excused_by_noise_floor"],
+             "empty_clusters": int((final_counts == 0).sum()),
+             "lockstep_start": start, "lockstep_fitted": fitted, "end_to_end": e2e}
+    record(entry)
+    print("full shape %s" % entry)
 
 
-def test_full_shape_c3_headline(hip, oracle):
-    _full_shape_checks(hip, oracle, "C3", np.float32, 30)
-
-
-def test_full_shape_c3_end_to_end_against_oracle(hip, oracle):
-    """The headline shape, all 10M rows, fixed iterations on both sides.
-
-    A random-row start splits some blobs between two centroids; rows on such a boundary
-    are near-ties at the rounding level of the float32 expanded form, and a flipped row
-    moves the boundary a little in the next iteration. How far two CORRECT float32
-    evaluations drift apart after a fixed number of iterations is measured here with the
-    oracle itself (features summed ascending vs descending); the engine must stay within
-    the same order of magnitude of the oracle and agree on the objective."""
-    X, k, _ = datasets.make("C3", 1.0, np.float32)
-    n, d = X.shape
-    iters = 12
-    C0 = datasets.seeded_row_init(X, k, datasets.SHAPES["C3"][3])
-    with hip.Handle(n, d, k, np.float32) as h:
-        h.set_data(X)
-        h.set_centroids(C0)
-        assert h.fit(iters, 0.0) == iters
-        Cg, Lg = h.centroids(), h.labels()
-        inertia = h.inertia()
-    wC, wL, _, _ = oracle.lloyd(X, C0, iters, 0.0, threads=16)
-    oracle.set_dot_order(True)
-    try:
-        rC, rL, _, _ = oracle.lloyd(X, C0, iters, 0.0, threads=16)
-    finally:
-        oracle.set_dot_order(False)
-    err = centroid_err(Cg, wC)
-    self_err = centroid_err(rC, wC)
-    w_inertia = float(oracle.assign(X, wC, threads=16, return_mindist=True)[1].astype(np.float64).sum())
-    print("C3 full, %d iterations: engine vs oracle centroid error %.2e (label diffs %d); "
-          "oracle ascending vs descending order %.2e (label diffs %d); inertia rel diff %.2e"
-          % (iters, err, int((Lg != wL).sum()), self_err, int((rL != wL).sum()),
-             abs(inertia - w_inertia) / w_inertia))
-    assert err <= max(1e-4, 4 * self_err)
-    assert abs(inertia - w_inertia) <= 1e-5 * w_inertia
-
-
-def test_full_shape_c2_with_predict(hip, oracle):
-    _full_shape_checks(hip, oracle, "C2", np.float32, 50)
-
-
-def test_full_shape_c4_float32(hip, oracle):
-    _full_shape_checks(hip, oracle, "C4", np.float32, 20)
-
-
-def test_full_shape_c4_float64(hip, oracle):
-    _full_shape_checks(hip, oracle, "C4", np.float64, 20)
-
-
-def test_full_shape_c5_with_transform(hip, oracle):
-    def transform_check(h, X, C, L):
-        H = datasets.make_holdout("C5", 100_000)
-        D = h.transform(H)                      # [k][rows], squared distances
-        assert D.shape == (C.shape[0], H.shape[0])
-        rng = np.random.default_rng(5)
-        rows = rng.choice(H.shape[0], size=64, replace=False)
-        cols = rng.choice(C.shape[0], size=64, replace=False)
-        want = ((H[rows][:, None, :].astype(np.float64) - C[cols][None, :, :].astype(np.float64)) ** 2).sum(-1)
-        got = D[np.ix_(cols, rows)].T.astype(np.float64)
-        scale = (H[rows].astype(np.float64) ** 2).sum(1).max() * 2
-        assert np.max(np.abs(got - want)) <= 64 * np.finfo(np.float32).eps * scale
-        # labels of the held-out rows = column argmin of the transform (up to near-ties)
-        pl = h.predict(H[:5000])
-        am = np.argmin(D[:, :5000], axis=0)
-        bad = np.nonzero(pl != am)[0]
-        for i in bad:
-            a, b = D[pl[i], i], D[am[i], i]
-            assert abs(a - b) <= 1e-5 * max(a, b)
-    _full_shape_checks(hip, oracle, "C5", np.float32, 15, extra=transform_check)
+def _transform_check(h, C):
+    H = datasets.make_holdout("C5", 100_000)
+    D = h.transform(H)                      # [k][rows], squared distances
+    assert D.shape == (C.shape[0], H.shape[0])
+    rng = np.random.default_rng(5)
+    rows = rng.choice(H.shape[0], size=64, replace=False)
+    cols = rng.choice(C.shape[0], size=64, replace=False)
+    want = ((H[rows][:, None, :].astype(np.float64) - C[cols][None, :, :].astype(np.float64)) ** 2).sum(-1)
+    got = D[np.ix_(cols, rows)].T.astype(np.float64)
+    scale = (H[rows].astype(np.float64) ** 2).sum(1).max() * 2
+    assert np.max(np.abs(got - want)) <= 64 * np.finfo(np.float32).eps * scale
+    # labels of the held-out rows = column argmin of the transform (up to near-ties)
+    pl = h.predict(H[:5000])
+    am = np.argmin(D[:, :5000], axis=0)
+    bad = np.nonzero(pl != am)[0]
+    for i in bad:
+        a, b = D[pl[i], i], D[am[i], i]
+        assert abs(a - b) <= 1e-5 * max(a, b)

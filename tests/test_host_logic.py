@@ -176,3 +176,60 @@ def test_datasets_are_deterministic_and_shaped():
     assert H.shape == (100, 784) and not np.array_equal(H, X5[:100])
     C0 = datasets.seeded_row_init(X3, k3, 5)
     assert C0.shape == (256, 32) and len({r.tobytes() for r in C0}) == 256
+
+
+def test_more_clusters_than_rows_keeps_one_shape(model):
+    """n_clusters > rows: the library fits with k = rows (kmeans_h2o4gpu.cu:630-635) and the
+    estimator's centre array keeps n_clusters rows; predict and transform then hand the
+    library exactly as many centroids as that array holds."""
+    m, lib = model
+    m.n_clusters = 5
+    X = np.arange(6, dtype=np.float32).reshape(3, 2)            # 3 rows, 5 clusters asked for
+    m.fit(X)
+    assert m.cluster_centers_.shape == (5, 2)
+    m.predict(X)
+    name, a = lib.calls[-1]
+    assert a[7] == 5 and a[12].size == 5 * 2
+    D = m.transform(X)
+    name, a = lib.calls[-1]
+    assert a[5] == 5 and a[7].size == 5 * 2 and D.shape == (3, 5)
+    # a centre array shorter than n_clusters (set by hand, or left by an older fit) is
+    # never over-read: k follows the array
+    m.cluster_centers_ = np.zeros((3, 2), np.float32)
+    m.predict(X)
+    assert lib.calls[-1][1][7] == 3 and lib.calls[-1][1][12].size == 6
+    assert m.transform(X).shape == (3, 3)
+
+
+def test_cluster_namespace_clone_and_pipeline(monkeypatch):
+    """The scikit-learn-shaped surface (reference: scripts/prepare_sklearn.sh:65-66 puts the
+    estimator into the `cluster` namespace): importable from h2o4gpu_amd.cluster, accepted by
+    sklearn.base.clone and by a two-step Pipeline in both positions."""
+    from sklearn.base import clone
+    from sklearn.pipeline import Pipeline
+    from sklearn.preprocessing import StandardScaler
+    import sklearn.cluster
+    from h2o4gpu_amd import cluster
+    assert cluster.KMeans is km.KMeans and cluster.KMeansH2O is km.KMeansH2O
+    assert cluster.KMeansSklearn is sklearn.cluster.KMeans
+    monkeypatch.setattr("h2o4gpu_amd.util.gpu.device_count", lambda n_gpus=0: (1, 1))
+    lib = RecordingLib()
+    monkeypatch.setattr(km.KMeansH2O, "_load_lib", lambda self: lib)
+    est = cluster.KMeans(n_clusters=3, init="random", max_iter=7, tol=0.25, random_state=42,
+                         backend="h2o4gpu")
+    twin = clone(est)
+    assert twin is not est and twin.backend == "h2o4gpu"
+    assert twin.get_params() == est.get_params() and twin.get_params()["n_clusters"] == 3
+    inner = clone(est.model)
+    assert isinstance(inner, km.KMeansH2O) and inner.get_params() == est.model.get_params()
+    assert est.set_params(max_iter=9) is est and est.get_params()["max_iter"] == 9
+    with pytest.raises(ValueError):
+        est.set_params(backend="sklearn")
+    X = np.random.default_rng(0).standard_normal((20, 2)).astype(np.float32)
+    last = Pipeline([("scale", StandardScaler()), ("km", clone(est))]).fit(X)
+    assert last.predict(X).shape == (20,) and lib.calls[-1][0] == "make_ptr_float_kmeans"
+    first = Pipeline([("km", clone(est)), ("scale", StandardScaler())])
+    assert first.fit_transform(X).shape == (20, 3)
+    # the CPU backend clones into the CPU backend
+    cpu = clone(cluster.KMeans(n_clusters=2, n_gpus=0, random_state=1, n_init=1))
+    assert cpu.backend == "sklearn"
