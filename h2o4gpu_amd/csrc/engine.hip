@@ -493,8 +493,9 @@ struct Engine : h2o4gpu_kmeans_handle {
   int *pcounts = nullptr;
   T *shift_partials = nullptr;
   T *shift2 = nullptr;
-  int *order = nullptr, *order_label = nullptr, *bucket_offsets = nullptr, *bucket_cursor = nullptr;
-  int *bucket_counts = nullptr;
+  int *order = nullptr, *order_label = nullptr, *bucket_offsets = nullptr, *bucket_hist = nullptr;
+  int *bucket_seg = nullptr, *bucket_total = nullptr;
+  double *bucket_partials = nullptr;
   bool use_buckets = false;
   double *sum_partials = nullptr;  // [sum_partials_needed() + 1]
   double *kpp_bsums = nullptr;
@@ -553,8 +554,10 @@ struct Engine : h2o4gpu_kmeans_handle {
       KM_TRY(dalloc(&order, n));
       KM_TRY(dalloc(&order_label, n));
       KM_TRY(dalloc(&bucket_offsets, k));
-      KM_TRY(dalloc(&bucket_cursor, k));
-      KM_TRY(dalloc(&bucket_counts, k));
+      KM_TRY(dalloc(&bucket_hist, (size_t)bucket_blocks(n) * k));
+      KM_TRY(dalloc(&bucket_seg, (size_t)32 * k));
+      KM_TRY(dalloc(&bucket_total, 1));
+      KM_TRY(dalloc(&bucket_partials, bucket_partial_slots(n, k) * d));
     }
     KM_TRY(dalloc(&shift_partials, (size_t)max_shift_partials(d, k) + 1));
     KM_TRY(dalloc(&shift2, 1));
@@ -588,7 +591,7 @@ struct Engine : h2o4gpu_kmeans_handle {
     void *ptrs[] = {xnorm,  C[0],    C[1],           cnorm,  labels,       mindist,
                     counts, psums,   pcounts,        shift_partials, shift2,
                     sum_partials, kpp_bsums, kpp_rows, kpp_dcc, order, order_label, bucket_offsets,
-                    bucket_cursor, bucket_counts};
+                    bucket_hist, bucket_seg, bucket_total, bucket_partials};
     for (void *p : ptrs)
       if (p) (void)hipFree(p);
     if (stream) (void)hipStreamDestroy(stream);
@@ -762,8 +765,9 @@ struct Engine : h2o4gpu_kmeans_handle {
   int update_async() {
     if (use_buckets && opt_buckets) {
       PROFILED("accumulate", launch_bucketed_accumulate<T>(stream, X, labels, order, order_label,
-                                                           bucket_offsets, bucket_cursor,
-                                                           bucket_counts, psums, pcounts, n, d, k));
+                                                           bucket_offsets, bucket_hist, bucket_seg,
+                                                           bucket_total, bucket_partials, psums,
+                                                           pcounts, n, d, k));
       return finish_update(1, true);
     }
     PROFILED("accumulate", launch_accumulate<T>(stream, plan, X, labels, psums, pcounts, n, d, k));

@@ -116,15 +116,20 @@ template <typename T>
 int launch_accumulate(hipStream_t s, const UpdatePlan &p, const T *X,
                       const int *labels, double *psums, int *pcounts, int64_t n,
                       int d, int k);
-// Pass 1 for shapes whose sums need many LDS chunks: rows are bucketed by
-// label (order / order_label: [n] int32 each, offsets / cursor: [k] int32) and every
-// bucket is summed into gsum [k][d] double; counts receives the bucket sizes. The
-// result is consumed by launch_finalize with slots = 1.
+// Pass 1 for shapes whose sums need many LDS chunks: the rows are ordered by label with a
+// stable counting sort (order / order_label: [n] int32 each, offsets: [k] int32,
+// block_hist: [bucket_blocks(n)][k] int32, seg_hist: [32][k] int32) and summed in fixed
+// windows of the ordered rows (partials: [bucket_partial_slots(n, k)][d] double) into
+// gsum [k][d] double; counts receives the bucket sizes. Run-to-run reproducible for
+// both precisions. The result is consumed by launch_finalize with slots = 1.
 bool bucketed_update_applies(int k_chunks, int k, int d);
+int bucket_blocks(int64_t n);
+size_t bucket_partial_slots(int64_t n, int k);
 template <typename T>
 int launch_bucketed_accumulate(hipStream_t s, const T *X, const int *labels, int *order,
-                               int *order_label, int *offsets, int *cursor, int *total,
-                               double *gsum, int *counts, int64_t n, int d, int k);
+                               int *order_label, int *offsets, int *block_hist, int *seg_hist,
+                               int *total, double *partials, double *gsum, int *counts, int64_t n,
+                               int d, int k);
 
 // Pass 2: fixed-order reduction of the partials, empty clusters keep the old
 // centroid, mean = sum * (1/count), per-block partial of sum((old-new)^2).

@@ -422,40 +422,114 @@ int launch_accumulate<double>(hipStream_t s, const UpdatePlan &p, const double *
 // pass 1, large k*d: bucket rows by label, then sum each bucket.
 //
 // When the per-centroid sums do not fit in LDS the chunked kernel above has to
-// scan all labels once per centroid chunk. Instead the rows are bucketed by
-// label (counting sort: histogram, exclusive scan, scatter) and every wavefront
-// sums 64 consecutive rows of the bucketed order in registers, lanes across
-// features, flushing to the [k][d] double sums with a global atomic add only
-// when the label changes (about once per wavefront). The data set is read once,
-// in whole rows. Sums are double, so for float data the result does not depend
-// on the order inside a bucket (which the scatter does not fix).
+// scan all labels once per centroid chunk. Instead the rows are ordered by label
+// with a stable counting sort and the ordered rows are summed in fixed windows.
+// Nothing in it depends on the order in which workgroups or wavefronts run, so the
+// sums are the same bit for bit from run to run, in float64 too:
+//   histogram : rows per label of every block of rows               [blocks][k]
+//   scan      : per label, exclusive sum over the blocks (two levels), bucket
+//               sizes, and the exclusive sum of those over the labels
+//   scatter   : position of a row = start of its label's bucket + rows of that
+//               label in earlier blocks + rows of that label earlier in its own
+//               block (each wavefront walks a contiguous quarter of the block in
+//               row order and ranks 64 rows at a time with ballots)
+//   window sum: a wavefront sums WPOS consecutive positions of the ordered rows in
+//               registers, lanes across features, and stores the sum of every run
+//               of equal labels to a slot of its own (window + label: the index
+//               grows by at least one from each run to the next, so no two runs
+//               share a slot and nothing is added atomically)
+//   bucket sum: per label, the slots of its windows are added in window order by
+//               four strands with a fixed tree.
 // Replaces the reference's sort_by_key + calculate_centroids
-// (kmeans_centroids.h:40-75, 131).
+// (kmeans_centroids.h:40-75, 131), whose atomic adds arrive in no fixed order.
 // ---------------------------------------------------------------------------
-static constexpr int BUCKET_ROWS = 4096;  // rows per workgroup in count / scatter
+static constexpr int BUCKET_ROWS_MIN = 4096;  // rows per block of the histogram / scatter
+static constexpr int BUCKET_MAX_BLOCKS = 2048;
+static constexpr int BUCKET_SEGS = 32;        // block segments of the two-level scan
 
-__global__ __launch_bounds__(WG) void bucket_count_kernel(const int *__restrict__ labels,
-                                                         int *__restrict__ counts, int64_t n,
-                                                         int k) {
+int64_t bucket_rows_per_block(int64_t n) {
+  int64_t rpb = (n + BUCKET_MAX_BLOCKS - 1) / BUCKET_MAX_BLOCKS;
+  rpb = (rpb + 255) / 256 * 256;
+  return rpb < BUCKET_ROWS_MIN ? BUCKET_ROWS_MIN : rpb;
+}
+int bucket_blocks(int64_t n) { return (int)((n + bucket_rows_per_block(n) - 1) / bucket_rows_per_block(n)); }
+// wavefronts per scatter workgroup: each keeps its own [k] counters in LDS
+static int bucket_waves(int k) {
+  if ((size_t)4 * k * sizeof(int) <= 128 * 1024) return 4;
+  if ((size_t)2 * k * sizeof(int) <= 128 * 1024) return 2;
+  return 1;
+}
+// positions per window of the window sum: 128 once there are enough windows to fill the GPU
+int bucket_window(int64_t n) { return n >= (int64_t)1 << 20 ? 128 : 64; }
+size_t bucket_partial_slots(int64_t n, int k) { return (size_t)(n / bucket_window(n) + 2) + k; }
+
+__global__ __launch_bounds__(WG) void bucket_hist_kernel(const int *__restrict__ labels,
+                                                        int *__restrict__ bh, int64_t n, int k,
+                                                        int64_t rpb) {
   extern __shared__ int hist[];  // [k]
   const int tid = threadIdx.x;
   for (int c = tid; c < k; c += WG) hist[c] = 0;
   __syncthreads();
-  const int64_t r0 = (int64_t)blockIdx.x * BUCKET_ROWS;
-  const int64_t r1 = min(n, r0 + BUCKET_ROWS);
+  const int64_t r0 = (int64_t)blockIdx.x * rpb;
+  const int64_t r1 = min(n, r0 + rpb);
   for (int64_t i = r0 + tid; i < r1; i += WG) {
     const int l = labels[i];
-    if (l >= 0 && l < k) atomicAdd(&hist[l], 1);
+    if (l >= 0 && l < k) atomicAdd(&hist[l], 1);  // integer counts: order-independent
   }
   __syncthreads();
-  for (int c = tid; c < k; c += WG)
-    if (hist[c] > 0) atomicAdd(&counts[c], hist[c]);
+  int *dst = bh + (size_t)blockIdx.x * k;
+  for (int c = tid; c < k; c += WG) dst[c] = hist[c];
 }
 
-// offsets[c] = sum of counts[0..c), cursor = copy; single workgroup.
+// Level 1 of the scan over blocks: seg[s][c] = rows of label c in the blocks of segment s.
+__global__ __launch_bounds__(WG) void bucket_seg_kernel(const int *__restrict__ bh,
+                                                       int *__restrict__ seg, int nb, int k,
+                                                       int per_seg) {
+  const int c = blockIdx.x * WG + threadIdx.x;
+  if (c >= k) return;
+  const int b0 = blockIdx.y * per_seg, b1 = min(nb, b0 + per_seg);
+  int sum = 0;
+  int b = b0;
+  for (; b + 4 <= b1; b += 4) {
+    const int v0 = bh[(size_t)b * k + c], v1 = bh[(size_t)(b + 1) * k + c];
+    const int v2 = bh[(size_t)(b + 2) * k + c], v3 = bh[(size_t)(b + 3) * k + c];
+    sum += v0 + v1 + v2 + v3;
+  }
+  for (; b < b1; b++) sum += bh[(size_t)b * k + c];
+  seg[(size_t)blockIdx.y * k + c] = sum;
+}
+// Level 2: bh[b][c] <- rows of label c in blocks before b; the last segment also leaves the
+// bucket size in counts[c].
+__global__ __launch_bounds__(WG) void bucket_block_scan_kernel(int *__restrict__ bh,
+                                                              const int *__restrict__ seg,
+                                                              int *__restrict__ counts, int nb,
+                                                              int k, int per_seg) {
+  const int c = blockIdx.x * WG + threadIdx.x;
+  if (c >= k) return;
+  int run = 0;
+  for (int s = 0; s < (int)blockIdx.y; s++) run += seg[(size_t)s * k + c];
+  const int b0 = blockIdx.y * per_seg, b1 = min(nb, b0 + per_seg);
+  int b = b0;
+  for (; b + 4 <= b1; b += 4) {
+    const int v0 = bh[(size_t)b * k + c], v1 = bh[(size_t)(b + 1) * k + c];
+    const int v2 = bh[(size_t)(b + 2) * k + c], v3 = bh[(size_t)(b + 3) * k + c];
+    bh[(size_t)b * k + c] = run;
+    bh[(size_t)(b + 1) * k + c] = run + v0;
+    bh[(size_t)(b + 2) * k + c] = run + v0 + v1;
+    bh[(size_t)(b + 3) * k + c] = run + v0 + v1 + v2;
+    run += v0 + v1 + v2 + v3;
+  }
+  for (; b < b1; b++) {
+    const int v = bh[(size_t)b * k + c];
+    bh[(size_t)b * k + c] = run;
+    run += v;
+  }
+  if (blockIdx.y == gridDim.y - 1) counts[c] = run;
+}
+
+// offsets[c] = sum of counts[0..c), *total = sum of all; single workgroup.
 __global__ __launch_bounds__(WG) void bucket_scan_kernel(const int *__restrict__ counts,
                                                         int *__restrict__ offsets,
-                                                        int *__restrict__ cursor,
                                                         int *__restrict__ total, int k) {
   __shared__ int part[WG];
   const int tid = threadIdx.x;
@@ -478,59 +552,83 @@ __global__ __launch_bounds__(WG) void bucket_scan_kernel(const int *__restrict__
   int run = part[tid];
   for (int c = lo; c < hi; c++) {
     offsets[c] = run;
-    cursor[c] = run;
     run += counts[c];
   }
 }
 
-__global__ __launch_bounds__(WG) void bucket_scatter_kernel(const int *__restrict__ labels,
-                                                           int *__restrict__ cursor,
-                                                           int *__restrict__ order,
-                                                           int *__restrict__ order_label,
-                                                           int64_t n, int k) {
-  extern __shared__ int sm[];
-  int *hist = sm;      // [k] rows of this block per label, then running rank
-  int *base = sm + k;  // [k] start of this block's range inside the label's bucket
-  const int tid = threadIdx.x;
-  for (int c = tid; c < k; c += WG) hist[c] = 0;
+// Stable scatter. The workgroup has NWB wavefronts; wavefront w owns rows
+// [r0 + w*q, r0 + (w+1)*q) of the block, q = rpb / NWB, and its own counters wh[w][k].
+__global__ void bucket_scatter_kernel(const int *__restrict__ labels, const int *__restrict__ bh,
+                                      const int *__restrict__ offsets, int *__restrict__ order,
+                                      int *__restrict__ order_label, int64_t n, int k, int64_t rpb) {
+  extern __shared__ int wh[];  // [NWB][k]
+  const int tid = threadIdx.x, tpb = blockDim.x;
+  const int nwb = tpb >> 6, wave = tid >> 6, lane = tid & 63;
+  for (int e = tid; e < nwb * k; e += tpb) wh[e] = 0;
   __syncthreads();
-  const int64_t r0 = (int64_t)blockIdx.x * BUCKET_ROWS;
-  const int64_t r1 = min(n, r0 + BUCKET_ROWS);
-  for (int64_t i = r0 + tid; i < r1; i += WG) {
+  const int64_t r0 = (int64_t)blockIdx.x * rpb;
+  const int64_t q = rpb / nwb;  // rpb is a multiple of 256
+  const int64_t w0 = min(n, r0 + wave * q), w1 = min(n, w0 + q);
+  int *mine = wh + (size_t)wave * k;
+  for (int64_t i = w0 + lane; i < w1; i += 64) {
     const int l = labels[i];
-    if (l >= 0 && l < k) atomicAdd(&hist[l], 1);
+    if (l >= 0 && l < k) atomicAdd(&mine[l], 1);
   }
   __syncthreads();
-  for (int c = tid; c < k; c += WG) {
-    const int h = hist[c];
-    base[c] = h > 0 ? atomicAdd(&cursor[c], h) : 0;
-    hist[c] = 0;
+  // counters -> first position of (this wavefront, label): bucket start + earlier blocks +
+  // earlier wavefronts of this block
+  const int *bbase = bh + (size_t)blockIdx.x * k;
+  for (int c = tid; c < k; c += tpb) {
+    int run = offsets[c] + bbase[c];
+    for (int w = 0; w < nwb; w++) {
+      const int v = wh[(size_t)w * k + c];
+      wh[(size_t)w * k + c] = run;
+      run += v;
+    }
   }
   __syncthreads();
-  for (int64_t i = r0 + tid; i < r1; i += WG) {
-    const int l = labels[i];
-    if (l >= 0 && l < k) {
-      const int pos = base[l] + atomicAdd(&hist[l], 1);
+  // 64 rows at a time, in row order: every lane reads its label's counter, lanes with the
+  // same label rank themselves by lane number, the first of them advances the counter
+  for (int64_t i0 = w0; i0 < w1; i0 += 64) {
+    const int64_t i = i0 + lane;
+    const int l = i < w1 ? labels[i] : -1;
+    const bool valid = l >= 0 && l < k;
+    const int cur = valid ? mine[l] : 0;
+    unsigned long long todo = __ballot(valid);
+    int pos = -1, cnt = 0;
+    bool first = false;
+    while (todo) {
+      const int leader = __ffsll((long long)todo) - 1;
+      const int l0 = __shfl(l, leader, 64);
+      const unsigned long long same = __ballot(valid && l == l0);
+      if (valid && l == l0) {
+        pos = cur + __popcll(same & ((1ull << lane) - 1ull));
+        cnt = __popcll(same);
+        first = lane == leader;
+      }
+      todo &= ~same;
+    }
+    if (valid) {
       order[pos] = (int)i;
       order_label[pos] = l;
     }
+    if (first) mine[l] = cur + cnt;  // (one lane per label; read again only in the next round)
   }
 }
 
-// One wavefront per 64 bucketed rows; lanes across features (VEC each, NVEC
-// vectors per lane cover up to 64*VEC*NVEC features per pass over the rows).
+// One wavefront per window of WM*64 consecutive ordered positions; lanes across features
+// (VEC each, NVEC vectors per lane cover up to 64*VEC*NVEC features per pass over the rows).
+// The sum of every run of equal labels goes to slot (window + label) of P, [slots][d].
 template <typename T, int VEC, int NVEC>
-__global__ __launch_bounds__(WG) void segment_sum_kernel(
+__global__ __launch_bounds__(WG) void window_sum_kernel(
     const T *__restrict__ X, const int *__restrict__ order,
-    const int *__restrict__ order_label, double *__restrict__ gsum,
-    const int *__restrict__ total, int d) {
+    const int *__restrict__ order_label, double *__restrict__ P,
+    const int *__restrict__ total, int d, int wm) {
   const int64_t m = *total;
   const int lane = threadIdx.x & 63;
-  const int64_t pos0 = ((int64_t)blockIdx.x * (WG / 64) + (threadIdx.x >> 6)) * 64;
-  if (pos0 >= m) return;
-  const int cnt = (int)min<int64_t>(64, m - pos0);
-  const int my_row = lane < cnt ? order[pos0 + lane] : 0;
-  const int my_lab = lane < cnt ? order_label[pos0 + lane] : -1;
+  const int64_t win = (int64_t)blockIdx.x * (WG / 64) + (threadIdx.x >> 6);
+  const int64_t wpos0 = win * wm * 64;
+  if (wpos0 >= m) return;
   constexpr int SPAN = 64 * VEC * NVEC;
   for (int d0 = 0; d0 < d; d0 += SPAN) {
     double acc[NVEC][VEC];
@@ -538,7 +636,6 @@ __global__ __launch_bounds__(WG) void segment_sum_kernel(
     for (int q = 0; q < NVEC; q++)
 #pragma unroll
       for (int e = 0; e < VEC; e++) acc[q][e] = 0.0;
-    int cur = __shfl(my_lab, 0, 64);
     // Lane slot q covers features [j, j + VEC). When d is not a multiple of VEC the last
     // such vector would reach past the row: it is fetched from the row's last VEC values
     // instead (offset jc) and only its elements from `first` on belong to this lane.
@@ -552,44 +649,53 @@ __global__ __launch_bounds__(WG) void segment_sum_kernel(
       first[q] = active[q] ? j - jc[q] : 0;
     }
     auto flush = [&](int label) {
+      double *dst = P + (size_t)(win + label) * d;
 #pragma unroll
       for (int q = 0; q < NVEC; q++) {
 #pragma unroll
         for (int e = 0; e < VEC; e++) {
-          if (active[q] && e >= first[q])
-            unsafeAtomicAdd(gsum + (size_t)label * d + jc[q] + e, acc[q][e]);
+          if (active[q] && e >= first[q]) dst[jc[q] + e] = acc[q][e];
           acc[q][e] = 0.0;
         }
       }
     };
-    constexpr int U = 4;
-    for (int i0 = 0; i0 < cnt; i0 += U) {
-      typename RowVec<T, VEC>::type v[U][NVEC];
-      int lab[U];
+    int cur = -1;
+    for (int sub = 0; sub < wm; sub++) {
+      const int64_t pos0 = wpos0 + (int64_t)sub * 64;
+      if (pos0 >= m) break;
+      const int cnt = (int)min<int64_t>(64, m - pos0);
+      const int my_row = lane < cnt ? order[pos0 + lane] : 0;
+      const int my_lab = lane < cnt ? order_label[pos0 + lane] : -1;
+      if (sub == 0) cur = __shfl(my_lab, 0, 64);
+      constexpr int U = 4;
+      for (int i0 = 0; i0 < cnt; i0 += U) {
+        typename RowVec<T, VEC>::type v[U][NVEC];
+        int lab[U];
 #pragma unroll
-      for (int u = 0; u < U; u++) {
-        const int i = min(i0 + u, cnt - 1);
-        const int row = __shfl(my_row, i, 64);
-        lab[u] = __shfl(my_lab, i, 64);
-        const T *x = X + (int64_t)row * d;
+        for (int u = 0; u < U; u++) {
+          const int i = min(i0 + u, cnt - 1);
+          const int row = __shfl(my_row, i, 64);
+          lab[u] = __shfl(my_lab, i, 64);
+          const T *x = X + (int64_t)row * d;
 #pragma unroll
-        for (int q = 0; q < NVEC; q++) v[u][q] = load_vec<T, VEC>(x + jc[q]);  // inactive: masked below
-      }
-#pragma unroll
-      for (int u = 0; u < U; u++) {
-        if (i0 + u >= cnt) break;
-        if (lab[u] != cur) {
-          flush(cur);
-          cur = lab[u];
+          for (int q = 0; q < NVEC; q++) v[u][q] = load_vec<T, VEC>(x + jc[q]);  // inactive: masked below
         }
 #pragma unroll
-        for (int q = 0; q < NVEC; q++) {
-          if (active[q]) {
-            if constexpr (VEC == 1) {
-              acc[q][0] += (double)v[u][q];
-            } else {
+        for (int u = 0; u < U; u++) {
+          if (i0 + u >= cnt) break;
+          if (lab[u] != cur) {
+            flush(cur);
+            cur = lab[u];
+          }
 #pragma unroll
-              for (int e = 0; e < VEC; e++) acc[q][e] += (double)v[u][q][e];
+          for (int q = 0; q < NVEC; q++) {
+            if (active[q]) {
+              if constexpr (VEC == 1) {
+                acc[q][0] += (double)v[u][q];
+              } else {
+#pragma unroll
+                for (int e = 0; e < VEC; e++) acc[q][e] += (double)v[u][q][e];
+              }
             }
           }
         }
@@ -599,38 +705,80 @@ __global__ __launch_bounds__(WG) void segment_sum_kernel(
   }
 }
 
-size_t bucket_lds_bytes(int k) { return (size_t)2 * k * sizeof(int); }
+// gsum[c][j] = sum over the windows of label c's bucket of P[window + c][j], windows in
+// ascending order dealt to 4 strands (window w: strand (w - first) % 4), the four strand
+// sums then added as ((s0 + s1) + s2) + s3. grid (k, ceil(d / 64)).
+__global__ __launch_bounds__(WG) void bucket_sum_kernel(const double *__restrict__ P,
+                                                       const int *__restrict__ offsets,
+                                                       const int *__restrict__ counts,
+                                                       double *__restrict__ gsum, int d, int wpos) {
+  __shared__ double part[4][64];
+  const int c = blockIdx.x;
+  const int f = threadIdx.x & 63, strand = threadIdx.x >> 6;
+  const int j = blockIdx.y * 64 + f;
+  const int cnt = counts[c], off = offsets[c];
+  double s = 0.0;
+  if (cnt > 0 && j < d) {
+    const int w_first = off / wpos, w_last = (off + cnt - 1) / wpos;
+    const double *src = P + (size_t)c * d + j;
+    int w = w_first + strand;
+    for (; w + 12 <= w_last; w += 16) {
+      const double a0 = src[(size_t)w * d], a1 = src[(size_t)(w + 4) * d];
+      const double a2 = src[(size_t)(w + 8) * d], a3 = src[(size_t)(w + 12) * d];
+      s = s + a0;
+      s = s + a1;
+      s = s + a2;
+      s = s + a3;
+    }
+    for (; w <= w_last; w += 4) s = s + src[(size_t)w * d];
+  }
+  part[strand][f] = s;
+  __syncthreads();
+  if (strand == 0 && j < d) gsum[(size_t)c * d + j] = ((part[0][f] + part[1][f]) + part[2][f]) + part[3][f];
+}
+
+size_t bucket_lds_bytes(int k) { return (size_t)bucket_waves(k) * k * sizeof(int); }
 bool bucketed_update_applies(int k_chunks, int k, int d) {
   // Measured: up to 8 chunks the LDS kernel is ahead (10M x 32, k = 4096: 0.61 vs 0.83 ms;
   // 8M x 16, k = 8192: 0.40 vs 0.66), from 11 chunks on bucketing is (2M x 256, k = 1024:
-  // 0.49 vs 0.62; 500k x 784, k = 256: 0.36 vs 0.52). With a handful of centroids the
-  // scatter's few cursors serialise, so bucketing is never used while the sums fit LDS.
+  // 0.49 vs 0.62; 500k x 784, k = 256: 0.36 vs 0.52). With a handful of centroids a bucket
+  // spans thousands of windows and the per-label sum has no parallelism left, so bucketing
+  // is never used while the sums fit LDS.
   (void)d;
-  return k_chunks > KM_MAX_LDS_CHUNKS && bucket_lds_bytes(k) <= 128 * 1024;
+  return k_chunks > KM_MAX_LDS_CHUNKS && (size_t)k * sizeof(int) <= 128 * 1024;
 }
 
 template <typename T>
 int launch_bucketed_accumulate(hipStream_t s, const T *X, const int *labels, int *order,
-                               int *order_label, int *offsets, int *cursor, int *total,
-                               double *gsum, int *counts, int64_t n, int d, int k) {
-  KM_HIP_TRY(hipMemsetAsync(counts, 0, (size_t)k * sizeof(int), s));
-  KM_HIP_TRY(hipMemsetAsync(gsum, 0, (size_t)k * d * sizeof(double), s));
-  const unsigned blocks = (unsigned)((n + BUCKET_ROWS - 1) / BUCKET_ROWS);
+                               int *order_label, int *offsets, int *block_hist, int *seg_hist,
+                               int *total, double *partials, double *gsum, int *counts, int64_t n,
+                               int d, int k) {
+  const int64_t rpb = bucket_rows_per_block(n);
+  const int nb = bucket_blocks(n);
+  const int per_seg = (nb + BUCKET_SEGS - 1) / BUCKET_SEGS;
+  const int segs = (nb + per_seg - 1) / per_seg;
   const size_t lds1 = (size_t)k * sizeof(int), lds2 = bucket_lds_bytes(k);
+  KM_TRY(ensure_dynamic_lds(reinterpret_cast<const void *>(bucket_hist_kernel), lds1));
   KM_TRY(ensure_dynamic_lds(reinterpret_cast<const void *>(bucket_scatter_kernel), lds2));
-  KM_TRY(ensure_dynamic_lds(reinterpret_cast<const void *>(bucket_count_kernel), lds2));
-  hipLaunchKernelGGL(bucket_count_kernel, dim3(blocks), dim3(WG), lds1, s, labels, counts, n, k);
-  hipLaunchKernelGGL(bucket_scan_kernel, dim3(1), dim3(WG), 0, s, counts, offsets, cursor, total, k);
-  hipLaunchKernelGGL(bucket_scatter_kernel, dim3(blocks), dim3(WG), lds2, s, labels, cursor, order,
-                     order_label, n, k);
-  // rows with a label outside [0, k) are not bucketed, so the bucketed order may be
-  // shorter than n: the grid covers n positions and every wavefront bounds itself by
-  // the device-side total
-  const unsigned sblocks = (unsigned)((n + 255) / 256);
+  const unsigned kblocks = (unsigned)((k + WG - 1) / WG);
+  hipLaunchKernelGGL(bucket_hist_kernel, dim3(nb), dim3(WG), lds1, s, labels, block_hist, n, k, rpb);
+  hipLaunchKernelGGL(bucket_seg_kernel, dim3(kblocks, segs), dim3(WG), 0, s, block_hist, seg_hist, nb, k,
+                     per_seg);
+  hipLaunchKernelGGL(bucket_block_scan_kernel, dim3(kblocks, segs), dim3(WG), 0, s, block_hist, seg_hist,
+                     counts, nb, k, per_seg);
+  hipLaunchKernelGGL(bucket_scan_kernel, dim3(1), dim3(WG), 0, s, counts, offsets, total, k);
+  hipLaunchKernelGGL(bucket_scatter_kernel, dim3(nb), dim3(bucket_waves(k) * 64), lds2, s, labels,
+                     block_hist, offsets, order, order_label, n, k, rpb);
+  // rows with a label outside [0, k) are not bucketed, so the ordered rows may be fewer
+  // than n: the grid covers n positions and every wavefront bounds itself by the
+  // device-side total
+  const int wm = bucket_window(n) / 64;
+  const int64_t windows = (n + (int64_t)wm * 64 - 1) / ((int64_t)wm * 64);
+  const unsigned sblocks = (unsigned)((windows + WG / 64 - 1) / (WG / 64));
   // 16-byte loads for any d that holds a whole vector (rows need element alignment only)
-#define KM_SEG(VEC, NVEC)                                                                   \
-  hipLaunchKernelGGL((segment_sum_kernel<T, VEC, NVEC>), dim3(sblocks), dim3(WG), 0, s, X, \
-                     order, order_label, gsum, total, d)
+#define KM_SEG(VEC, NVEC)                                                                  \
+  hipLaunchKernelGGL((window_sum_kernel<T, VEC, NVEC>), dim3(sblocks), dim3(WG), 0, s, X, \
+                     order, order_label, partials, total, d, wm)
   if constexpr (sizeof(T) == 4) {
     if (d >= 4) {
       if (d <= 256) KM_SEG(4, 1);
@@ -649,6 +797,8 @@ int launch_bucketed_accumulate(hipStream_t s, const T *X, const int *labels, int
     }
   }
 #undef KM_SEG
+  hipLaunchKernelGGL(bucket_sum_kernel, dim3((unsigned)k, (unsigned)((d + 63) / 64)), dim3(WG), 0, s,
+                     partials, offsets, counts, gsum, d, wm * 64);
   KM_HIP_TRY(hipGetLastError());
   return 0;
 }
@@ -882,11 +1032,11 @@ int launch_gather_rows(hipStream_t s, const T *X, const int *idx, T *C, int k, i
 }
 
 template int launch_bucketed_accumulate<float>(hipStream_t, const float *, const int *, int *, int *,
-                                               int *, int *, int *, double *, int *, int64_t, int,
-                                               int);
-template int launch_bucketed_accumulate<double>(hipStream_t, const double *, const int *, int *,
-                                                int *, int *, int *, int *, double *, int *, int64_t,
-                                                int, int);
+                                               int *, int *, int *, int *, double *, double *, int *,
+                                               int64_t, int, int);
+template int launch_bucketed_accumulate<double>(hipStream_t, const double *, const int *, int *, int *,
+                                                int *, int *, int *, int *, double *, double *, int *,
+                                                int64_t, int, int);
 
 #define KM_INSTANTIATE(T)                                                            \
   template int launch_row_norms<T>(hipStream_t, const T *, T *, int64_t, int);       \

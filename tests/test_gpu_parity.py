@@ -138,6 +138,40 @@ def test_duplicate_centroids_lowest_index_wins(hip, oracle, variant, k, pairs, e
             assert np.array_equal(C1[hi], C0[hi]) and not np.array_equal(C1[lo], C0[lo])
 
 
+@pytest.mark.parametrize("n,d,k,dtype,exact", [
+    # float32 rows are summed in double, which is exact whatever the order: every path repeats
+    (200000, 16, 8, np.float32, True), (150000, 32, 256, np.float32, True),
+    (100000, 64, 64, np.float32, True), (80000, 40, 600, np.float32, True),
+    # sums that do not fit LDS: rows ordered by label with a stable sort, fixed windows and
+    # a fixed tree, so float64 repeats bit for bit as well
+    (60000, 256, 700, np.float64, True), (60000, 256, 700, np.float32, True),
+    (30000, 784, 1100, np.float32, True), (50000, 130, 1500, np.float64, True),
+    # float64 rows through the LDS-privatised sums are added in arrival order inside a
+    # workgroup: repeatable to rounding only
+    (100000, 32, 64, np.float64, False),
+])
+def test_two_identical_fits_repeat(hip, n, d, k, dtype, exact):
+    """The same fit twice in one process and once more on a fresh handle: labels always
+    identical; centroids bit-identical wherever the sums are order-independent (float32
+    rows) or taken in a fixed order (the bucketed update of large models)."""
+    X = blobs(n, d, min(k, 64), dtype, spread=6.0, sigma=2.0, seed=n + d)
+    C0 = np.ascontiguousarray(X[np.random.default_rng(k).choice(n, size=k, replace=False)])
+    runs = []
+    for fresh in range(2):
+        with hip.Handle(n, d, k, dtype) as h:
+            h.set_data(X)
+            for _ in range(2 - fresh):
+                h.set_centroids(C0)
+                assert h.fit(4, 0.0) == 4
+                runs.append((h.centroids(), h.labels(), h.inertia()))
+    C, L, inertia = runs[0]
+    for Cr, Lr, ir in runs[1:]:
+        if exact:
+            assert np.array_equal(Cr, C) and np.array_equal(Lr, L) and ir == inertia
+        else:
+            assert np.allclose(Cr, C, rtol=1e-12, atol=1e-12 * np.abs(C).max())
+
+
 def separated_problem(n, d, k, dtype, seed, spread=10.0, offset=0.5):
     """Blobs plus one start per blob (true centre + offset). No blob is split by the
     start, so no row sits on a decision boundary and a last-bit difference in a
