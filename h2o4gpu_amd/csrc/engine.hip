@@ -8,6 +8,7 @@
 // are independent.
 #include <algorithm>
 #include <atomic>
+#include <cmath>
 #include <csignal>
 #include <cstdarg>
 #include <cstdlib>
@@ -195,7 +196,18 @@ struct h2o4gpu_kmeans_handle {
   virtual int init_random_rows(int seed) = 0;
   virtual int start_from_rows(const int *rows) = 0;  // centroids = the given k rows of the data
   virtual int init_plusplus(int seed) = 0;
+  virtual int init_parallel(int seed) = 0;
   std::vector<int> last_seed_rows;
+  // what the last k-means|| run found: data row of every candidate in the order found,
+  // candidates added and sum of minimum costs per round, rows per nearest candidate (empty
+  // when there were at most k candidates), candidate index of each final centre (-1: zero row)
+  struct ParallelSeedInfo {
+    std::vector<int> cand_rows;
+    int round_count[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    double phi[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    std::vector<double> weights;
+    std::vector<int> chosen;
+  } seed_info;
   virtual int fit(int max_iterations, double threshold, int *iters) = 0;
   virtual int assign() = 0;
   virtual int update(double *shift2) = 0;
@@ -740,6 +752,181 @@ struct Engine : h2o4gpu_kmeans_handle {
     return init_from_rows(idx.data());
   }
 
+  // k-means|| followed by the reference's host k-means++ over the weighted candidates
+  // (kmeans_parallel, kmeans_h2o4gpu.cu:331-563, one device; kmeans_plus_plus :201-279;
+  // pick_point_idx_weighted :154-199). Kept as the reference has them: the first centre
+  // from mt19937(seed); min(8, (int)(2 + log(k))) rounds; a round measures the rows against
+  // the candidates of the previous round only and keeps a running minimum; a row becomes
+  // a candidate when T(2.0 * k * cost / total) exceeds its threshold, which depends on
+  // (seed, row) alone; a potential of 0 skips the selection; more than k candidates are
+  // weighted by the rows nearest to each and reduced on the host with the re-seeded
+  // sampler; at most k candidates become the first centres followed by zero rows. The
+  // seed is used as given, negative or not (:339-342 re-declares the variable it means to
+  // replace). Not the reference's: the order of the sums (distances come from these
+  // kernels instead of cuBLAS, the sum of the costs is a fixed tree in double, rounded to T).
+  int init_parallel(int seed) override {
+    KM_HIP_TRY(hipSetDevice(dev));
+    if (!have_data) return H2O4GPU_KMEANS_ESTATE;
+    if ((int64_t)k > n) return H2O4GPU_KMEANS_EARG;
+    seed_info = ParallelSeedInfo();
+    std::mt19937 gen(seed);
+    std::uniform_int_distribution<> dis(0, (int)(n - 1));
+    std::vector<int> all(1, dis(gen));
+    std::vector<int> recent = all;
+    T *cost = nullptr, *Cc = nullptr, *ccn = nullptr, *best = nullptr;
+    int *list = nullptr, *didx = nullptr, *dcount = nullptr;
+    int rc = parallel_rounds(seed, all, recent, &cost, &Cc, &ccn, &best, &list, &didx, &dcount);
+    (void)hipStreamSynchronize(stream);
+    void *ptrs[] = {cost, Cc, ccn, best, list, didx, dcount};
+    for (void *p : ptrs)
+      if (p) (void)hipFree(p);
+    have_mindist = false;  // mindist served as scratch
+    return rc;
+  }
+  // (re)allocates a device buffer of at least `count` elements
+  template <typename U>
+  int regrow(U **p, size_t *have, size_t count) {
+    if (*p && *have >= count) return 0;
+    if (*p) (void)hipFree(*p);
+    *p = nullptr;
+    *have = 0;
+    KM_TRY(dalloc(p, count));
+    *have = count;
+    return 0;
+  }
+  int parallel_rounds(int seed, std::vector<int> &all, std::vector<int> &recent, T **cost, T **Cc,
+                      T **ccn, T **best, int **list, int **didx, int **dcount) {
+    const int64_t nb = (n + KPP_BLOCK - 1) / KPP_BLOCK;
+    size_t cap_model = 0, cap_norm = 0, cap_idx = 0, cap_best = 0;
+    const int list_cap = (int)n;
+    KM_TRY(dalloc(cost, n));
+    KM_TRY(dalloc(list, list_cap));
+    KM_TRY(dalloc(dcount, 1));
+    std::vector<double> bs((size_t)nb);
+    // stage m candidate rows as a padded model
+    auto stage = [&](const std::vector<int> &rows) -> int {
+      const size_t m = rows.size();
+      const size_t mpad = (m + CENTROID_PAD - 1) / CENTROID_PAD * CENTROID_PAD;
+      KM_TRY(regrow(Cc, &cap_model, mpad * d));
+      KM_TRY(regrow(ccn, &cap_norm, mpad));
+      KM_TRY(regrow(didx, &cap_idx, m));
+      KM_HIP_TRY(hipMemcpyAsync(*didx, rows.data(), m * sizeof(int), hipMemcpyHostToDevice, stream));
+      return launch_gather_model<T>(stream, X, xnorm, *didx, (int)m, (int)mpad, *Cc, *ccn, d);
+    };
+    uint32_t state0 = (uint32_t)seed % 2147483647u;  // thrust seeds minstd_rand like this
+    if (state0 == 0) state0 = 1;
+    const int rounds = std::min(8, (int)(2 + std::log((double)k)));
+    for (int counter = 0; counter < rounds; counter++) {
+      log_msg(verbose, LOG_VERBOSE, "KMeans|| - Iteration %d.", counter);
+      KM_TRY(stage(recent));
+      // minimum distance to this round's candidates, compared as floats (no integer keys)
+      PROFILED("seed_assign", launch_assign<T>(stream, opt_assign, X, xnorm, *Cc, *ccn, labels, mindist,
+                                               n, d, (int)recent.size(), num_cu, nullptr, true));
+      PROFILED("seed_fold", launch_fold_min<T>(stream, mindist, *cost, kpp_bsums, n, counter == 0));
+      KM_HIP_TRY(hipMemcpyAsync(bs.data(), kpp_bsums, (size_t)nb * sizeof(double), hipMemcpyDeviceToHost,
+                                stream));
+      KM_HIP_TRY(hipStreamSynchronize(stream));
+      double sum = 0;
+      for (int64_t b = 0; b < nb; b++) sum += bs[(size_t)b];
+      const T total = (T)sum;
+      seed_info.phi[counter] = (double)total;
+      log_msg(verbose, LOG_VERBOSE, "KMeans|| - Total min cost from centers %g.", (double)total);
+      if (total == (T)0) continue;
+      KM_HIP_TRY(hipMemsetAsync(*dcount, 0, sizeof(int), stream));
+      PROFILED("seed_select", launch_select_rows<T>(stream, *cost, total, state0, k, *list, *dcount,
+                                                    list_cap, n));
+      int count = 0;
+      KM_HIP_TRY(hipMemcpyAsync(&count, *dcount, sizeof(int), hipMemcpyDeviceToHost, stream));
+      KM_HIP_TRY(hipStreamSynchronize(stream));
+      if (count > list_cap) count = list_cap;  // (cannot happen: one entry per row at most)
+      seed_info.round_count[counter] = count;
+      log_msg(verbose, LOG_VERBOSE, "KMeans|| - New potential centroids %d.", count);
+      if (count > 0) {
+        recent.resize((size_t)count);
+        KM_HIP_TRY(hipMemcpyAsync(recent.data(), *list, (size_t)count * sizeof(int), hipMemcpyDeviceToHost,
+                                  stream));
+        KM_HIP_TRY(hipStreamSynchronize(stream));
+        std::sort(recent.begin(), recent.end());  // the reference's copy_if keeps row order
+        all.insert(all.end(), recent.begin(), recent.end());
+      }
+    }
+    seed_info.cand_rows = all;
+    const int M = (int)all.size();
+    seed_info.chosen.assign((size_t)k, -1);
+    if (M <= k) {  // kmeans_h2o4gpu.cu:536-540: the candidates, then zero rows
+      for (int c = 0; c < M; c++) seed_info.chosen[(size_t)c] = c;
+      KM_HIP_TRY(hipMemsetAsync(C[cur], 0, (size_t)k * d * sizeof(T), stream));
+      KM_TRY(regrow(didx, &cap_idx, (size_t)M));
+      KM_HIP_TRY(hipMemcpyAsync(*didx, all.data(), (size_t)M * sizeof(int), hipMemcpyHostToDevice, stream));
+      KM_TRY(launch_gather_rows<T>(stream, X, *didx, C[cur], M, d));
+      last_seed_rows.assign((size_t)k, -1);
+      std::copy(all.begin(), all.end(), last_seed_rows.begin());
+      KM_TRY(centroids_changed());
+      KM_HIP_TRY(hipStreamSynchronize(stream));
+      return 0;
+    }
+    // weights: rows per nearest candidate (count_pts_per_centroid, kmeans_h2o4gpu.h:90-126)
+    KM_TRY(stage(all));
+    PROFILED("seed_weights", launch_assign<T>(stream, opt_assign, X, xnorm, *Cc, *ccn, labels, mindist, n, d,
+                                              M, num_cu, nullptr, true));
+    int *dhist = nullptr;
+    size_t cap_hist = 0;
+    KM_TRY(regrow(&dhist, &cap_hist, (size_t)M));
+    std::vector<int> hist((size_t)M);
+    int rc = hipMemsetAsync(dhist, 0, (size_t)M * sizeof(int), stream) == hipSuccess ? 0 : H2O4GPU_KMEANS_EDEVICE;
+    if (rc == 0) rc = launch_label_histogram(stream, labels, dhist, n);
+    if (rc == 0 && hipMemcpyAsync(hist.data(), dhist, (size_t)M * sizeof(int), hipMemcpyDeviceToHost, stream) != hipSuccess)
+      rc = H2O4GPU_KMEANS_EDEVICE;
+    if (rc == 0 && hipStreamSynchronize(stream) != hipSuccess) rc = H2O4GPU_KMEANS_EDEVICE;
+    (void)hipFree(dhist);
+    KM_TRY(rc);
+    std::vector<T> w((size_t)M);
+    seed_info.weights.resize((size_t)M);
+    for (int c = 0; c < M; c++) {
+      w[(size_t)c] = (T)hist[(size_t)c];
+      seed_info.weights[(size_t)c] = (double)hist[(size_t)c];
+    }
+    // the host k-means++ (kmeans_h2o4gpu.cu:201-279); its distances run on the device
+    KM_TRY(regrow(best, &cap_best, (size_t)M));
+    std::vector<T> thr((size_t)M), hbest((size_t)M);
+    {
+      std::mt19937 mt(seed);  // the sampler makes a fresh one on every call: same draws
+      std::uniform_real_distribution<> dist(0.0, 1.0);
+      for (int i = 0; i < M; i++) thr[(size_t)i] = (T)dist(mt);
+    }
+    auto pick = [&](const T *data) -> int {  // pick_point_idx_weighted
+      T weighted_sum = 0;
+      for (int i = 0; i < M; i++) weighted_sum += data ? data[i] * w[(size_t)i] : w[(size_t)i];
+      T best_prob = 0;
+      int best_idx = 0;
+      for (int i = 0; i < M; i++) {
+        T val = w[(size_t)i];
+        if (data) val *= data[i];
+        const T share = val / weighted_sum;
+        if (share > thr[(size_t)i]) return i;
+        if (share >= best_prob) {
+          best_prob = share;
+          best_idx = i;
+        }
+      }
+      return best_idx;
+    };
+    int idx = pick(nullptr);
+    for (int c = 0; c < k; c++) {
+      seed_info.chosen[(size_t)c] = idx;
+      w[(size_t)idx] = 0;
+      if (c == k - 1) break;
+      PROFILED("seed_pick", launch_candidate_dists<T>(stream, *Cc, *ccn, idx, *best, M, d, c == 0));
+      KM_HIP_TRY(hipMemcpyAsync(hbest.data(), *best, (size_t)M * sizeof(T), hipMemcpyDeviceToHost, stream));
+      KM_HIP_TRY(hipStreamSynchronize(stream));
+      idx = pick(hbest.data());
+    }
+    std::vector<int> rows((size_t)k);
+    for (int c = 0; c < k; c++) rows[(size_t)c] = all[(size_t)seed_info.chosen[(size_t)c]];
+    last_seed_rows = rows;
+    return init_from_rows(rows.data());
+  }
+
   // The fused kernels compute the centroid norms themselves, so a Lloyd loop that needs no
   // convergence scalar skips the post-update launch and leaves cnorm behind the current
   // centroids; every other consumer of cnorm refreshes it first.
@@ -1106,9 +1293,11 @@ static int fit_entry(int verbose, int seed, int gpu_id, size_t rows, size_t cols
     if (init_from_data == 0) {
       rc = start_rows.empty() ? h->init_random_rows(seed) : h->start_from_rows(start_rows.data());
     } else if (init_from_data == 1) {
-      rc = h->init_plusplus(seed);
+      rc = h->init_parallel(seed);  // k-means||, as the reference (kmeans_h2o4gpu.cu:733-737)
     } else if (init_from_data == 2) {
       rc = centroids ? h->set_centroids_host(centroids) : H2O4GPU_KMEANS_EARG;
+    } else if (init_from_data == 3) {
+      rc = h->init_plusplus(seed);  // extension: k-means++ (D^2 sampling)
     } else {
       // the reference has no branch for other values and runs from all-zero
       // centroids (kmeans_h2o4gpu.cu:684-740); same here
@@ -1334,6 +1523,30 @@ KM_API int h2o4gpu_kmeans_init_random_rows(h2o4gpu_kmeans_handle *h, int seed) {
 KM_API int h2o4gpu_kmeans_init_plusplus(h2o4gpu_kmeans_handle *h, int seed) {
   KM_CHECK_HANDLE(h);
   return h->init_plusplus(seed);
+}
+KM_API int h2o4gpu_kmeans_init_parallel(h2o4gpu_kmeans_handle *h, int seed) {
+  KM_CHECK_HANDLE(h);
+  return h->init_parallel(seed);
+}
+KM_API int h2o4gpu_kmeans_parallel_seed_info(h2o4gpu_kmeans_handle *h, int cap, int *cand_rows,
+                                             int *n_candidates, int *round_count, double *phi,
+                                             double *weights, int *chosen) {
+  KM_CHECK_HANDLE(h);
+  const auto &si = h->seed_info;
+  if (si.cand_rows.empty()) return H2O4GPU_KMEANS_ESTATE;
+  const int m = (int)si.cand_rows.size();
+  if (n_candidates) *n_candidates = m;
+  if (round_count) memcpy(round_count, si.round_count, sizeof(si.round_count));
+  if (phi) memcpy(phi, si.phi, sizeof(si.phi));
+  if (chosen) memcpy(chosen, si.chosen.data(), si.chosen.size() * sizeof(int));
+  if (cand_rows || weights) {
+    if (cap < m) return H2O4GPU_KMEANS_EARG;
+    if (cand_rows) memcpy(cand_rows, si.cand_rows.data(), (size_t)m * sizeof(int));
+    if (weights) {
+      for (int c = 0; c < m; c++) weights[c] = si.weights.empty() ? 0.0 : si.weights[(size_t)c];
+    }
+  }
+  return 0;
 }
 KM_API int h2o4gpu_kmeans_get_seed_rows(h2o4gpu_kmeans_handle *h, int *rows) {
   KM_CHECK_HANDLE(h);

@@ -168,6 +168,24 @@ int launch_min_dist_update(hipStream_t s, const T *X, const T *xnorm, int64_t ce
                            T *mind, int *nearest, int *rows, T *dcc, int t, double *bsums,
                            int64_t n, int d);
 
+// k-means|| building blocks (kmeans_h2o4gpu.cu:331-563): a padded model of candidate rows
+// for the assign kernels; running minimum cost + its fixed-order block sums
+// (bsums: [ceil(n / KPP_BLOCK)]); the reference's per-row acceptance test, rows taken
+// appended to list (arrival order, *count may exceed cap); rows per nearest candidate;
+// one distance step of the host k-means++ over the candidates.
+template <typename T>
+int launch_gather_model(hipStream_t s, const T *X, const T *xnorm, const int *idx, int m, int mpad,
+                        T *Cc, T *ccn, int d);
+template <typename T>
+int launch_fold_min(hipStream_t s, const T *cur, T *cost, double *bsums, int64_t n, int init);
+template <typename T>
+int launch_select_rows(hipStream_t s, const T *cost, T total, uint32_t state0, int k, int *list,
+                       int *count, int cap, int64_t n);
+int launch_label_histogram(hipStream_t s, const int *labels, int *counts, int64_t n);
+template <typename T>
+int launch_candidate_dists(hipStream_t s, const T *Cc, const T *ccn, int centre, T *best, int m,
+                           int d, int first);
+
 // Copy rows idx[0..k-1] of X into C ([k][d]).
 template <typename T>
 int launch_gather_rows(hipStream_t s, const T *X, const int *idx, T *C, int k,

@@ -8,6 +8,9 @@
 // for plain k-means++: one kernel updates the running minimum against the
 // newest centre and emits fixed-order block sums; the host draws the next
 // centre from the block sums and one block of minima.
+#include <algorithm>
+#include <limits>
+
 #include "kmeans_common.h"
 
 namespace kmhip {
@@ -203,6 +206,194 @@ int launch_min_dist_update(hipStream_t s, const T *X, const T *xnorm, int64_t ce
   KM_HIP_TRY(hipGetLastError());
   return 0;
 }
+
+// ---------------------------------------------------------------------------
+// k-means|| (the reference's init_from_data == 1, kmeans_h2o4gpu.cu:331-563).
+// A round measures every row against the candidates of the previous round with the
+// assign kernels (their minimum distance is min_calc_functor's inner minimum, :281-304);
+// the kernels below fold that into the running cost, sum it, and apply the reference's
+// acceptance test to every row.
+// ---------------------------------------------------------------------------
+
+// Model of m candidate rows for the assign kernels: Cc [mpad][d] = rows idx[0..m-1] of X
+// followed by zero rows, ccn [mpad] = their squared norms (taken from xnorm: the same
+// value row_norms would compute) followed by +inf.
+template <typename T>
+__global__ __launch_bounds__(WG) void gather_model_kernel(const T *__restrict__ X,
+                                                         const T *__restrict__ xnorm,
+                                                         const int *__restrict__ idx, int m, int mpad,
+                                                         T *__restrict__ Cc, T *__restrict__ ccn,
+                                                         int d) {
+  const int64_t total = (int64_t)mpad * d;
+  const int64_t stride = (int64_t)gridDim.x * WG;
+  const int64_t t0 = (int64_t)blockIdx.x * WG + threadIdx.x;
+  for (int64_t e = t0; e < total; e += stride) {
+    const int c = (int)(e / d), j = (int)(e - (int64_t)c * d);
+    Cc[e] = c < m ? X[(int64_t)idx[c] * d + j] : (T)0;
+  }
+  for (int64_t c = t0; c < mpad; c += stride)
+    ccn[c] = c < m ? xnorm[idx[c]] : (T)__builtin_huge_val();
+}
+template <typename T>
+int launch_gather_model(hipStream_t s, const T *X, const T *xnorm, const int *idx, int m, int mpad,
+                        T *Cc, T *ccn, int d) {
+  const int64_t total = (int64_t)mpad * d;
+  const unsigned blocks = (unsigned)std::min<int64_t>((total + WG - 1) / WG, 4096);
+  hipLaunchKernelGGL((gather_model_kernel<T>), dim3(blocks), dim3(WG), 0, s, X, xnorm, idx, m, mpad,
+                     Cc, ccn, d);
+  KM_HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+// cost[i] = min(cost[i], cur[i]) (init != 0: cost[i] = min(max(T), cur[i])), then the block
+// sums of cost in double with the fixed tree of block_sum. One workgroup per KPP_BLOCK rows.
+template <typename T>
+__global__ __launch_bounds__(WG) void fold_min_kernel(const T *__restrict__ cur, T *__restrict__ cost,
+                                                     double *__restrict__ bsums, int64_t n,
+                                                     int init) {
+  __shared__ double red[WG];
+  const int64_t b0 = (int64_t)blockIdx.x * KPP_BLOCK;
+#pragma unroll
+  for (int q = 0; q < KPP_BLOCK / WG; q++) {
+    const int64_t row = b0 + threadIdx.x + q * WG;
+    if (row < n) {
+      const T prev = init ? std::numeric_limits<T>::max() : cost[row];
+      const T c = cur[row];
+      cost[row] = c < prev ? c : prev;
+    }
+  }
+  __syncthreads();  // (each thread re-reads only what it wrote; the barrier orders the LDS use)
+  block_sum<T>(cost, bsums, blockIdx.x, n, red);
+}
+template <typename T>
+int launch_fold_min(hipStream_t s, const T *cur, T *cost, double *bsums, int64_t n, int init) {
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL((fold_min_kernel<T>), dim3((unsigned)((n + KPP_BLOCK - 1) / KPP_BLOCK)),
+                     dim3(WG), 0, s, cur, cost, bsums, n, init);
+  KM_HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+// a * b mod (2^31 - 1) for a, b below the modulus
+__device__ __forceinline__ uint32_t mulmod_m31(uint32_t a, uint32_t b) {
+  const uint64_t p = (uint64_t)a * b;
+  uint64_t r = (p & 0x7FFFFFFFull) + (p >> 31);
+  r = (r & 0x7FFFFFFFull) + (r >> 31);
+  return (uint32_t)(r >= 0x7FFFFFFFull ? r - 0x7FFFFFFFull : r);
+}
+
+// The acceptance test of kmeans_h2o4gpu.cu:436-456 for every row:
+//   thrust::default_random_engine rng(seed); rng.discard(row);
+//   T threshold = (T)thrust::uniform_real_distribution<>(0, 1)(rng);     (a float)
+//   T prob = (2.0 * k * cost[row]) / total;                               (formed in double)
+//   take the row when prob > threshold.
+// The engine is minstd_rand (x <- 48271 x mod 2^31 - 1), so the value row `row` draws is
+// state0 * 48271^(row+1); the distribution maps x to float(x - 1) / (1.0f + float(m - 2)).
+// Rows taken are appended to list in arrival order (the host sorts them); *count may
+// exceed cap, in which case only cap entries were written.
+template <typename T>
+__global__ __launch_bounds__(WG) void select_rows_kernel(const T *__restrict__ cost, T total,
+                                                        uint32_t state0, int k,
+                                                        int *__restrict__ list,
+                                                        int *__restrict__ count, int cap,
+                                                        int64_t n) {
+  const int64_t row = (int64_t)blockIdx.x * WG + threadIdx.x;
+  if (row >= n) return;
+  uint32_t acc = state0, base = 48271u;
+  for (uint64_t e = (uint64_t)row + 1; e != 0; e >>= 1) {
+    if (e & 1) acc = mulmod_m31(acc, base);
+    base = mulmod_m31(base, base);
+  }
+  float u = static_cast<float>(acc - 1u);
+  u /= (1.0f + static_cast<float>(2147483645u));
+  const T threshold = (T)u;
+  const T prob = (T)((2.0 * k * (double)cost[row]) / (double)total);
+  if (prob > threshold) {
+    const int pos = atomicAdd(count, 1);
+    if (pos < cap) list[pos] = (int)row;
+  }
+}
+template <typename T>
+int launch_select_rows(hipStream_t s, const T *cost, T total, uint32_t state0, int k, int *list,
+                       int *count, int cap, int64_t n) {
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL((select_rows_kernel<T>), dim3((unsigned)((n + WG - 1) / WG)), dim3(WG), 0, s,
+                     cost, total, state0, k, list, count, cap, n);
+  KM_HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+// counts[label]++ over all rows (count_functor, kmeans_h2o4gpu.h:44-72, whose argmin starts
+// at candidate 0: a row no distance could be compared for counts there). Integer atomics:
+// the result does not depend on their order.
+__global__ __launch_bounds__(WG) void label_histogram_kernel(const int *__restrict__ labels,
+                                                            int *__restrict__ counts, int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * WG;
+  for (int64_t i = (int64_t)blockIdx.x * WG + threadIdx.x; i < n; i += stride) {
+    const int l = labels[i];
+    atomicAdd(&counts[l < 0 ? 0 : l], 1);
+  }
+}
+int launch_label_histogram(hipStream_t s, const int *labels, int *counts, int64_t n) {
+  if (n <= 0) return 0;
+  const unsigned blocks = (unsigned)std::min<int64_t>((n + WG - 1) / WG, 2048);
+  hipLaunchKernelGGL(label_histogram_kernel, dim3(blocks), dim3(WG), 0, s, labels, counts, n);
+  KM_HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+// One step of the host k-means++ over the candidates (kmeans_h2o4gpu.cu:226-271), the part
+// that touches every candidate: v = (xx + cc) - 2 x.c against candidate `centre` (the
+// expanded form of src/common/utils.cpp:34-57, no absolute value), best = v at the first
+// step, min(v, best) afterwards with best[centre] taken as 0. lpr lanes share a row.
+template <typename T>
+__global__ __launch_bounds__(WG) void candidate_dists_kernel(const T *__restrict__ Cc,
+                                                            const T *__restrict__ ccn, int centre,
+                                                            T *__restrict__ best, int m, int d,
+                                                            int first, int lpr) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int rps = 64 / lpr;
+  const int i = (blockIdx.x * (WG / 64) + wave) * rps + lane / lpr;
+  const int col = lane % lpr;
+  const T *x = Cc + (size_t)(i < m ? i : m - 1) * d;
+  const T *c = Cc + (size_t)centre * d;
+  T dot = 0;
+  for (int j = col; j < d; j += lpr) dot += x[j] * c[j];
+  for (int off = 1; off < lpr; off <<= 1) dot += __shfl_xor(dot, off, 64);
+  if (col == 0 && i < m) {
+    const T t = ccn[i] + ccn[centre];
+    const T v = (T)-2 * dot + t;
+    if (first) {
+      best[i] = v;
+    } else {
+      const T prev = i == centre ? (T)0 : best[i];
+      best[i] = v < prev ? v : prev;
+    }
+  }
+}
+template <typename T>
+int launch_candidate_dists(hipStream_t s, const T *Cc, const T *ccn, int centre, T *best, int m,
+                           int d, int first) {
+  if (m <= 0) return 0;
+  int lpr = 1;
+  while (lpr < d && lpr < 64) lpr <<= 1;
+  const int rows_per_block = (WG / 64) * (64 / lpr);
+  hipLaunchKernelGGL((candidate_dists_kernel<T>), dim3((unsigned)((m + rows_per_block - 1) / rows_per_block)),
+                     dim3(WG), 0, s, Cc, ccn, centre, best, m, d, first, lpr);
+  KM_HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+#define KM_SEED_INSTANTIATE(T)                                                                  \
+  template int launch_gather_model<T>(hipStream_t, const T *, const T *, const int *, int, int, \
+                                      T *, T *, int);                                           \
+  template int launch_fold_min<T>(hipStream_t, const T *, T *, double *, int64_t, int);         \
+  template int launch_select_rows<T>(hipStream_t, const T *, T, uint32_t, int, int *, int *,    \
+                                     int, int64_t);                                             \
+  template int launch_candidate_dists<T>(hipStream_t, const T *, const T *, int, T *, int, int, \
+                                         int);
+KM_SEED_INSTANTIATE(float)
+KM_SEED_INSTANTIATE(double)
 
 template int launch_min_dist_update<float>(hipStream_t, const float *, const float *, int64_t,
                                            float *, int *, int *, float *, int, double *, int64_t,

@@ -49,6 +49,9 @@ PROTOTYPES = {
     "h2o4gpu_kmeans_set_centroids_host": (c_int, [c_void_p, c_void_p]),
     "h2o4gpu_kmeans_init_random_rows": (c_int, [c_void_p, c_int]),
     "h2o4gpu_kmeans_init_plusplus": (c_int, [c_void_p, c_int]),
+    "h2o4gpu_kmeans_init_parallel": (c_int, [c_void_p, c_int]),
+    "h2o4gpu_kmeans_parallel_seed_info": (c_int, [c_void_p, c_int, c_void_p, P(c_int), c_void_p, c_void_p,
+                                                  c_void_p, c_void_p]),
     "h2o4gpu_kmeans_get_seed_rows": (c_int, [c_void_p, c_void_p]),
     "h2o4gpu_kmeans_fit": (c_int, [c_void_p, c_int, c_double, P(c_int)]),
     "h2o4gpu_kmeans_assign": (c_int, [c_void_p]),
@@ -181,6 +184,26 @@ class Handle:
 
     def init_plusplus(self, seed):
         _check("init_plusplus", lib().h2o4gpu_kmeans_init_plusplus(self._h, seed))
+
+    def init_parallel(self, seed):
+        """k-means|| as the reference runs it (its init_from_data == 1)."""
+        _check("init_parallel", lib().h2o4gpu_kmeans_init_parallel(self._h, seed))
+
+    def parallel_seed_info(self):
+        """What the last init_parallel found: dict with cand_rows, round_count [8], phi [8],
+        weights (None when there were at most k candidates) and chosen [k]."""
+        m = c_int(0)
+        rc = np.zeros(8, np.int32)
+        phi = np.zeros(8, np.float64)
+        chosen = np.empty(self.k, np.int32)
+        _check("parallel_seed_info", lib().h2o4gpu_kmeans_parallel_seed_info(
+            self._h, 0, None, ctypes.byref(m), _vp(rc), _vp(phi), None, _vp(chosen)))
+        cand = np.empty(m.value, np.int32)
+        w = np.empty(m.value, np.float64)
+        _check("parallel_seed_info", lib().h2o4gpu_kmeans_parallel_seed_info(
+            self._h, m.value, _vp(cand), None, None, None, _vp(w), None))
+        return {"cand_rows": cand, "round_count": rc, "phi": phi,
+                "weights": w if m.value > self.k else None, "chosen": chosen}
 
     def seed_rows(self):
         out = np.empty(self.k, np.int32)

@@ -10,6 +10,10 @@ on top of the gfx950 engine. Differences, all additive:
   * `inertia_` is filled after fit (the reference leaves it None, :187);
   * when scikit-learn is chosen as backend it is the installed scikit-learn (the
     reference uses its own renamed copy);
+  * `init='k-means++'` runs k-means|| as in the reference (whose native side does so for
+    that name); `'k-means||'` is accepted as a second name for it and `'d2-sampling'`
+    selects textbook k-means++ (one centre per pass, drawn proportionally to the squared
+    distance to the nearest chosen centre);
   * `n_init` restarts, `n_iter_` and a native `score`;
   * fit / predict / score / transform accept rows that already live on the GPU (any
     object with `__cuda_array_interface__`, e.g. a PyTorch-ROCm tensor): the engine adopts
@@ -111,7 +115,7 @@ class KMeansH2O:
                  algorithm='auto', gpu_id=0, n_gpus=-1, do_checks=1):
         if isinstance(tol, np.floating):
             tol = tol.item()
-        if isinstance(init, str) and init not in ['random', 'k-means++']:
+        if isinstance(init, str) and init not in ['random', 'k-means++', 'k-means||', 'd2-sampling']:
             raise ValueError("Invalid initialization method. Should be 'k-means++' or 'random' "
                              "but got '%s'." % init)
         self.init = init
@@ -200,7 +204,9 @@ class KMeansH2O:
             for r in range(restarts):
                 if start is not None:
                     h.set_centroids(start)
-                elif self.init == "k-means++":
+                elif self.init in ("k-means++", "k-means||"):
+                    h.init_parallel(self.random_state + r)
+                elif self.init == "d2-sampling":
                     h.init_plusplus(self.random_state + r)
                 else:
                     h.init_random_rows(self.random_state + r)
@@ -323,8 +329,10 @@ class KMeansH2O:
                 "init must have shape (n_clusters, n_features)"
             c_init = 2
             centroids = np.ascontiguousarray(init_arr, dtype=data.dtype).flatten()
-        elif self.init == "k-means++":
-            c_init = 1
+        elif self.init in ("k-means++", "k-means||"):
+            c_init = 1  # kmeans.py:472-475; the native side runs k-means|| for it, as the reference
+        elif self.init == "d2-sampling":
+            c_init = 3
         else:
             c_init = 0
         fn = lib.make_ptr_float_kmeans if self.double_precision == 0 else lib.make_ptr_double_kmeans
@@ -484,7 +492,9 @@ class KMeans:
                                        verbose=verbose, random_state=random_state, copy_x=copy_x,
                                        n_jobs=n_jobs, algorithm=algorithm, gpu_id=gpu_id, n_gpus=n_gpus,
                                        do_checks=do_checks)
-        self._sk_args = dict(n_clusters=n_clusters, init=init, n_init=n_init, max_iter=max_iter, tol=tol,
+        # (scikit-learn knows the engine's two extra seeding names only as 'k-means++')
+        sk_init = 'k-means++' if isinstance(init, str) and init in ('k-means||', 'd2-sampling') else init
+        self._sk_args = dict(n_clusters=n_clusters, init=sk_init, n_init=n_init, max_iter=max_iter, tol=tol,
                              verbose=verbose, random_state=random_state, copy_x=copy_x)
         self.model_sklearn = None
         # scikit-learn is used only when asked for (backend='sklearn' or n_gpus=0). The

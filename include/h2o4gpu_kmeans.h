@@ -37,9 +37,12 @@ extern "C" {
  *   with malloc() and handed to the caller through *pred_centroids ([k][n])
  *   and *pred_labels ([mTrain] int32); the caller owns them.
  *   init_from_data: 0 = seeded random distinct rows (std::shuffle with
- *   std::default_random_engine(seed), as the reference), 1 = k-means++
- *   seeding on the device, 2 = start from `centroids` ([k][n], extension:
- *   the reference ignores `centroids` when fitting).
+ *   std::default_random_engine(seed), as the reference), 1 = k-means|| with
+ *   the reference's rounds, acceptance test and host k-means++ over the
+ *   candidates (kmeans_h2o4gpu.cu:331-563; the estimator's 'k-means++'),
+ *   2 = start from `centroids` ([k][n], extension: the reference ignores
+ *   `centroids` when fitting), 3 = k-means++ by D^2 sampling on the device
+ *   (extension).
  *   threshold: absolute bound on sum((C_old - C_new)^2); the loop stops when
  *   the sum is below it. Exactly as the reference, a run of N iterations
  *   makes N centroid updates and N+1 assignment passes, the last one with the
@@ -148,12 +151,25 @@ int h2o4gpu_kmeans_set_data_host(h2o4gpu_kmeans_handle *h, const void *X);
 int h2o4gpu_kmeans_set_data_device(h2o4gpu_kmeans_handle *h, const void *d_X);
 
 /* Initial centroids: given ([k][cols] host), seeded random distinct rows
- * (the reference's std::shuffle rule), or k-means++ on the device. */
+ * (the reference's std::shuffle rule), k-means++ (D^2 sampling) on the device, or
+ * k-means|| as the reference runs it for init_from_data == 1 (kmeans_parallel,
+ * src/gpu/kmeans/kmeans_h2o4gpu.cu:331-563, with its host k-means++ over the
+ * weighted candidates, :154-279). */
 int h2o4gpu_kmeans_set_centroids_host(h2o4gpu_kmeans_handle *h, const void *C);
 int h2o4gpu_kmeans_init_random_rows(h2o4gpu_kmeans_handle *h, int seed);
 int h2o4gpu_kmeans_init_plusplus(h2o4gpu_kmeans_handle *h, int seed);
-/* Row indices the last init_random_rows / init_plusplus call chose ([k] int32). */
+int h2o4gpu_kmeans_init_parallel(h2o4gpu_kmeans_handle *h, int seed);
+/* Data rows the last init_* call chose ([k] int32; -1 where k-means|| found fewer than k
+ * candidates and left a zero row, as the reference does). */
 int h2o4gpu_kmeans_get_seed_rows(h2o4gpu_kmeans_handle *h, int *rows);
+/* What the last init_parallel call found: *n_candidates; round_count[8] and phi[8]
+ * (candidates added and sum of the minimum costs per round); with cap >= *n_candidates
+ * also cand_rows (data row of every candidate, in the order found) and weights (rows per
+ * nearest candidate; zeros when there were at most k candidates); chosen[k] = candidate
+ * index of every final centre (-1: zero row). Any pointer may be NULL. */
+int h2o4gpu_kmeans_parallel_seed_info(h2o4gpu_kmeans_handle *h, int cap, int *cand_rows,
+                                      int *n_candidates, int *round_count, double *phi,
+                                      double *weights, int *chosen);
 
 /* The reference's loop (kmeans_impl.h:109-232): up to max_iterations of
  * assign + update, stop when shift^2 < threshold, final assignment with the
@@ -206,7 +222,8 @@ int h2o4gpu_kmeans_set_option(h2o4gpu_kmeans_handle *h, const char *name,
  * is bracketed by its own event pair and kernel_time() returns the launch count
  * and summed milliseconds since profiling was switched on, by kernel name
  * ("assign", "accumulate", "assign_accumulate", "finalize", "post_update",
- * "row_norms", "transform", "min_dist_update", "inertia_sum"). */
+ * "row_norms", "transform", "min_dist_update", "inertia_sum", "seed_assign",
+ * "seed_fold", "seed_select", "seed_weights", "seed_pick"). */
 int h2o4gpu_kmeans_timer_start(h2o4gpu_kmeans_handle *h);
 int h2o4gpu_kmeans_timer_stop(h2o4gpu_kmeans_handle *h, float *milliseconds);
 int h2o4gpu_kmeans_profile(h2o4gpu_kmeans_handle *h, int on);

@@ -171,6 +171,56 @@ class Oracle:
                                       _ptr(mind))
         return rows, mind
 
+    def minstd_nth(self, seed, nth):
+        """Value of the nth call (nth >= 1) of thrust's default_random_engine seeded with seed."""
+        self.lib.oracle_minstd_nth.restype = ctypes.c_uint
+        return int(self.lib.oracle_minstd_nth(_int(seed), _i64(nth)))
+
+    def row_threshold(self, seed, row):
+        """The k-means|| acceptance threshold of a data row (float)."""
+        self.lib.oracle_kmeans_parallel_row_threshold.restype = ctypes.c_float
+        return float(self.lib.oracle_kmeans_parallel_row_threshold(_int(seed), _i64(row)))
+
+    def pick_point_idx_weighted(self, seed, weights, data=None):
+        weights = np.ascontiguousarray(weights)
+        if data is not None:
+            data = np.ascontiguousarray(data, weights.dtype)
+        fn = self._fn("pick_point_idx_weighted", weights.dtype)
+        fn.restype = _int
+        return int(fn(_int(seed), _int(weights.shape[0]), _ptr(data), _ptr(weights)))
+
+    def weighted_kmeanspp(self, seed, data, weights, k):
+        """Candidate indices chosen by the reference's host k-means++ over weighted candidates."""
+        data = np.ascontiguousarray(data)
+        weights = np.ascontiguousarray(weights, data.dtype)
+        m, d = data.shape
+        chosen = np.empty(k, np.int32)
+        self._fn("weighted_kmeanspp", data.dtype)(_int(seed), _int(m), _int(d), _int(k), _ptr(data),
+                                                  _ptr(weights), _ptr(chosen))
+        return chosen
+
+    def kmeans_parallel(self, X, k, seed, threads=1, cap=None):
+        """k-means|| as the reference runs it. Returns a dict: cand_rows (data row of every
+        candidate, in the order found), round_count [8], phi [8], weights (None when there
+        were at most k candidates), chosen [k] (candidate index, -1 = zero row), centroids."""
+        X, _ = self._prep(X)
+        n, d = X.shape
+        cap = int(cap if cap is not None else min(n * 8 + 1, max(64 * k + 64, 4096)))
+        cand = np.empty(cap, np.int32)
+        rc = np.zeros(8, np.int32)
+        phi = np.zeros(8, np.float64)
+        weights = np.zeros(cap, X.dtype)
+        chosen = np.empty(k, np.int32)
+        C = np.empty((k, d), X.dtype)
+        fn = self._fn("kmeans_parallel", X.dtype)
+        fn.restype = _int
+        m = int(fn(_i64(n), _int(d), _int(k), _ptr(X), _int(seed), _int(cap), _ptr(cand), _ptr(rc),
+                   _ptr(phi), _ptr(weights), _ptr(chosen), _ptr(C), _int(threads)))
+        if m < 0:
+            raise RuntimeError("k-means||: more than %d candidates" % cap)
+        return {"cand_rows": cand[:m].copy(), "round_count": rc, "phi": phi,
+                "weights": weights[:m].copy() if m > k else None, "chosen": chosen, "centroids": C}
+
     def kmeanspp_first(self, seed, n):
         self.lib.oracle_kmeanspp_first.restype = _int
         return int(self.lib.oracle_kmeanspp_first(_int(seed), _i64(n)))

@@ -25,9 +25,17 @@
 //       centroid pairs chosen asymmetrically (an a/b swap fails).
 //   descending dot order          : bit-equal to a numpy evaluation that adds the
 //       products of the column-reversed arrays in ascending order, norms untouched.
-//   kmeanspp_*                    : parity unpinned against the reference (the
-//       reference seeds with k-means|| whose candidate stream needs a CUDA
-//       build); pinned only against the textbook D^2-sampling definition.
+//   kmeanspp_*                    : not part of the reference (which seeds with
+//       k-means||); pinned against the textbook D^2-sampling definition.
+//   kmeans_parallel, weighted_kmeanspp, pick_point_idx_weighted, row thresholds:
+//       the two generators by their published 10000th values, the row thresholds
+//       bit for bit by rocThrust's host code, the host sampler's draws by numpy's
+//       MT19937, the sampler on cases worked from the draws alone, every round's
+//       candidates by float64 brute force over the thresholds, the weights by
+//       brute-force nearest-candidate cells. Parity unpinned against a run of the
+//       reference itself: its distances come out of cuBLAS / cblas and its sum of
+//       costs out of thrust::reduce, both in an unspecified order (j ascending
+//       and a fixed tree in double here).
 //
 // Build: make -C oracle   (g++ -O3 -fopenmp -ffp-contract=off)
 
@@ -408,6 +416,254 @@ void kmeanspp(int64_t n, int d, int k, const T *X, int seed, int *rows_out, T *m
   if (mind_out) std::copy(mind.begin(), mind.end(), mind_out);
 }
 
+
+// ---------------------------------------------------------------------------
+// k-means|| seeding, the reference's init_from_data == 1
+// (kmeans_parallel, kmeans_h2o4gpu.cu:331-563) followed by its host-side weighted
+// k-means++ over the candidates (:154-279).
+// ---------------------------------------------------------------------------
+
+// thrust::default_random_engine is minstd_rand: x <- 48271 x mod (2^31 - 1), state seeded
+// with seed mod m, or 1 when that is 0. The value the engine returns is the new state.
+static const uint32_t MINSTD_M = 2147483647u;
+static inline uint32_t minstd_seed(int seed) {
+  const uint32_t s = (uint32_t)seed % MINSTD_M;  // int -> result_type (uint32) first
+  return s == 0 ? 1u : s;
+}
+static inline uint32_t minstd_next(uint32_t x) {
+  return (uint32_t)(((uint64_t)x * 48271u) % MINSTD_M);
+}
+// thrust::uniform_real_distribution<> has RealType float and maps one engine value x to
+//   float(x - min) / (1.0f + float(max - min)) * (b - a) + a,   min = 1, max = m - 1,
+// all in float (thrust/random/detail/uniform_real_distribution.inl). With a = 0, b = 1.
+static inline float thrust_uniform01(uint32_t x) {
+  float result = static_cast<float>(x - 1u);
+  result /= (1.0f + static_cast<float>((MINSTD_M - 1u) - 1u));
+  return (result * (1.0f - 0.0f)) + 0.0f;
+}
+// The threshold of a row: rng(seed); rng.discard(row); dist(rng)  (:444-449). It does not
+// depend on the round.
+static float row_threshold(int seed, int64_t row) {
+  uint32_t x = minstd_seed(seed);
+  for (int64_t i = 0; i <= row; i++) x = minstd_next(x);
+  return thrust_uniform01(x);
+}
+
+// Sum of n values in double: blocks of 1024 rows, each formed from 256 partial sums (rows
+// t, t+256, t+512, t+768) combined by a halving tree, the block sums then added in block
+// order. The reference calls thrust::reduce in T, whose order is unspecified; this is the
+// order the GPU engine uses, so that both sides agree to the bit.
+template <typename T>
+double blocked_sum(int64_t n, const T *v) {
+  const int BLOCK = 1024, W = 256;
+  double total = 0;
+  for (int64_t b0 = 0; b0 < n; b0 += BLOCK) {
+    double part[W];
+    for (int t = 0; t < W; t++) {
+      double acc = 0;
+      for (int q = 0; q < BLOCK / W; q++) {
+        const int64_t row = b0 + t + q * W;
+        if (row < n) acc += (double)v[row];
+      }
+      part[t] = acc;
+    }
+    for (int off = W / 2; off > 0; off >>= 1)
+      for (int t = 0; t < off; t++) part[t] += part[t + off];
+    total += part[0];
+  }
+  return total;
+}
+
+// pick_point_idx_weighted (:154-199). weighted_sum is a sequential sum in T of weights[i]
+// (data == null) or data[i]*weights[i]. A fresh mt19937(seed) is made on every call; entry
+// i is taken as soon as its share of the sum exceeds the i-th draw of
+// std::uniform_real_distribution<double>(0,1) cast to T. When no entry is taken the result
+// is the last entry whose share reached the running maximum (start 0, updated on >=).
+template <typename T>
+int pick_point_idx_weighted(int seed, const T *data, const T *weights, int m) {
+  T weighted_sum = 0;
+  for (int i = 0; i < m; i++) weighted_sum += data ? data[i] * weights[i] : weights[i];
+  T best_prob = 0;
+  int best_idx = 0;
+  std::mt19937 mt(seed);
+  std::uniform_real_distribution<> dist(0.0, 1.0);
+  for (int i = 0; i < m; i++) {
+    const T threshold = (T)dist(mt);
+    T val = weights[i];
+    if (data) val *= data[i];
+    const T share = val / weighted_sum;
+    if (share > threshold) return i;
+    if (share >= best_prob) {
+      best_prob = share;
+      best_idx = i;
+    }
+  }
+  return best_idx;
+}
+
+// compute_distances for one centroid (src/common/utils.cpp:7-57): xx + cc formed first,
+// then the GEMM adds -2 * dot to it; no absolute value. The order inside the reference's
+// cblas GEMM is not specified; j ascending here.
+template <typename T>
+void host_dists_to_one(int m, int d, const T *data, const T *centre, T *out) {
+  T cc = 0;
+  for (int j = 0; j < d; j++) cc += centre[j] * centre[j];
+  for (int i = 0; i < m; i++) {
+    const T *x = data + (size_t)i * d;
+    T xx = 0, dot = 0;
+    for (int j = 0; j < d; j++) xx += x[j] * x[j];
+    for (int j = 0; j < d; j++) dot += x[j] * centre[j];
+    const T t = xx + cc;
+    out[i] = (T)-2 * dot + t;
+  }
+}
+
+// kmeans_plus_plus over the candidates (:201-279): first entry drawn from the weights
+// alone; every chosen entry gets weight 0; the running minimum of a chosen entry is set
+// to 0 before the distances to it are folded in. chosen receives k candidate indices.
+template <typename T>
+void weighted_kmeanspp(int seed, int m, int d, int k, const T *data, T *weights, int *chosen) {
+  std::vector<T> best((size_t)m), curr((size_t)m);
+  int idx = pick_point_idx_weighted<T>(seed, nullptr, weights, m);
+  chosen[0] = idx;
+  weights[idx] = 0;
+  host_dists_to_one<T>(m, d, data, data + (size_t)idx * d, best.data());
+  for (int it = 0; it < k - 1; it++) {
+    idx = pick_point_idx_weighted<T>(seed, best.data(), weights, m);
+    chosen[it + 1] = idx;
+    weights[idx] = 0;
+    best[idx] = 0;
+    host_dists_to_one<T>(m, d, data, data + (size_t)idx * d, curr.data());
+    for (int i = 0; i < m; i++) best[i] = std::min(curr[i], best[i]);
+  }
+}
+
+// kmeans_parallel (:331-563), one device.
+//   first centre: mt19937(seed), uniform_int_distribution<>(0, rows-1)   (:343-347)
+//   min_costs start at numeric_limits<T>::max()                          (:372-377)
+//   rounds: min(8, (int)(2 + log(k)))                                    (:382)
+//   a round measures every row against the candidates the PREVIOUS round added
+//     (|xx + cc - 2 x.c|, running minimum: min_calc_functor :281-304), sums the minima,
+//     and, unless the sum is 0, takes every row with
+//     T(2.0 * k * min_cost / total) > T(threshold(row)) as a new candidate, in row order
+//     (:436-476). A round that adds nothing leaves the previous candidate list in place.
+//   more than k candidates: weights = rows per nearest candidate (count_functor,
+//     kmeans_h2o4gpu.h:44-72: first index wins, start value the distance to candidate 0),
+//     then weighted_kmeanspp; otherwise the candidates followed by zero rows (:536-540).
+// cand_rows receives the data row of every candidate in the order found (capacity cap),
+// round_count[r] the number added by round r (r < 8; the first centre is not counted),
+// phi[r] the sum of minima of round r, weights the per-candidate counts (when computed),
+// chosen the k candidate indices of the final centres (-1: zero row). Returns the number
+// of candidates, or -1 when cap is too small.
+template <typename T>
+int kmeans_parallel(int64_t n, int d, int k, const T *X, int seed, int cap, int *cand_rows,
+                    int *round_count, double *phi, T *weights, int *chosen, T *C_out,
+                    int threads) {
+  std::mt19937 gen(seed);
+  std::uniform_int_distribution<> dis(0, (int)(n - 1));
+  std::vector<int> all;
+  all.push_back(dis(gen));
+  std::vector<int> recent = all;
+  std::vector<T> min_costs((size_t)n, std::numeric_limits<T>::max());
+  std::vector<T> xx((size_t)n);
+  row_norms<T>(n, d, X, xx.data(), threads);
+  std::vector<float> thr((size_t)n);
+  {
+    uint32_t x = minstd_seed(seed);
+    for (int64_t i = 0; i < n; i++) {
+      x = minstd_next(x);
+      thr[(size_t)i] = thrust_uniform01(x);
+    }
+  }
+  auto gather = [&](const std::vector<int> &rows) {
+    std::vector<T> c(rows.size() * (size_t)d);
+    for (size_t r = 0; r < rows.size(); r++)
+      std::copy(X + (int64_t)rows[r] * d, X + ((int64_t)rows[r] + 1) * d, c.begin() + r * d);
+    return c;
+  };
+  const int max_iter = std::min(8, (int)(2 + std::log((double)k)));
+  for (int r = 0; r < 8; r++) {
+    round_count[r] = 0;
+    phi[r] = 0;
+  }
+  for (int counter = 0; counter < max_iter; counter++) {
+    const int m = (int)recent.size();
+    std::vector<T> Cc = gather(recent);
+    std::vector<T> Ct = transpose_centroids(d, m, Cc.data());
+    std::vector<T> cc(m);
+    row_norms<T>(m, d, Cc.data(), cc.data(), 1);
+#pragma omp parallel num_threads(threads)
+    {
+      std::vector<T> acc(m);
+#pragma omp for schedule(static)
+      for (int64_t i = 0; i < n; i++) {
+        dist_row<T>(d, m, X + i * (int64_t)d, xx[(size_t)i], Ct.data(), cc.data(), acc.data());
+        T best = std::numeric_limits<T>::max();
+        for (int c = 0; c < m; c++) best = std::min(best, acc[c]);
+        min_costs[(size_t)i] = std::min(min_costs[(size_t)i], best);
+      }
+    }
+    const T total = (T)blocked_sum<T>(n, min_costs.data());
+    phi[counter] = (double)total;
+    if (total == (T)0) continue;
+    std::vector<int> fresh;
+    for (int64_t i = 0; i < n; i++) {
+      const T threshold = (T)thr[(size_t)i];
+      const T prob = (T)((2.0 * k * min_costs[(size_t)i]) / total);
+      if (prob > threshold) fresh.push_back((int)i);
+    }
+    round_count[counter] = (int)fresh.size();
+    if (!fresh.empty()) {
+      recent = fresh;
+      all.insert(all.end(), fresh.begin(), fresh.end());
+    }
+  }
+  const int M = (int)all.size();
+  if (M > cap) return -1;
+  std::copy(all.begin(), all.end(), cand_rows);
+  std::fill(C_out, C_out + (size_t)k * d, (T)0);
+  if (M <= k) {
+    for (int c = 0; c < k; c++) chosen[c] = c < M ? c : -1;
+    for (int c = 0; c < M; c++)
+      std::copy(X + (int64_t)all[c] * d, X + ((int64_t)all[c] + 1) * d, C_out + (size_t)c * d);
+    return M;
+  }
+  std::vector<T> Call = gather(all);
+  {
+    std::vector<T> Ct = transpose_centroids(d, M, Call.data());
+    std::vector<T> cc(M);
+    row_norms<T>(M, d, Call.data(), cc.data(), 1);
+    std::vector<int64_t> counts((size_t)M, 0);
+#pragma omp parallel num_threads(threads)
+    {
+      std::vector<T> acc(M);
+      std::vector<int64_t> local((size_t)M, 0);
+#pragma omp for schedule(static)
+      for (int64_t i = 0; i < n; i++) {
+        dist_row<T>(d, M, X + i * (int64_t)d, xx[(size_t)i], Ct.data(), cc.data(), acc.data());
+        int closest = 0;
+        T best = acc[0];
+        for (int c = 1; c < M; c++) {
+          if (acc[c] < best) {
+            best = acc[c];
+            closest = c;
+          }
+        }
+        local[(size_t)closest]++;
+      }
+#pragma omp critical
+      for (int c = 0; c < M; c++) counts[(size_t)c] += local[(size_t)c];
+    }
+    for (int c = 0; c < M; c++) weights[c] = (T)counts[(size_t)c];
+  }
+  std::vector<T> w(weights, weights + M);
+  weighted_kmeanspp<T>(seed, M, d, k, Call.data(), w.data(), chosen);
+  for (int c = 0; c < k; c++)
+    std::copy(Call.begin() + (size_t)chosen[c] * d, Call.begin() + ((size_t)chosen[c] + 1) * d,
+              C_out + (size_t)c * d);
+  return M;
+}
+
 }  // namespace
 
 extern "C" {
@@ -483,6 +739,35 @@ ORACLE_EXPORT void oracle_kmeanspp_f64(int64_t n, int d, int k, const double *X,
                                        int *rows_out, double *mind_out) {
   kmeanspp<double>(n, d, k, X, seed, rows_out, mind_out);
 }
+
+ORACLE_EXPORT float oracle_kmeans_parallel_row_threshold(int seed, int64_t row) {
+  return row_threshold(seed, row);
+}
+ORACLE_EXPORT unsigned oracle_minstd_nth(int seed, int64_t nth) {  // value of the nth call, nth >= 1
+  uint32_t x = minstd_seed(seed);
+  for (int64_t i = 0; i < nth; i++) x = minstd_next(x);
+  return x;
+}
+#define DEFINE_SEED_FOR(T, SUF)                                                              \
+  ORACLE_EXPORT int oracle_pick_point_idx_weighted_##SUF(int seed, int m, const T *data,    \
+                                                         const T *weights) {                \
+    return pick_point_idx_weighted<T>(seed, data, weights, m);                              \
+  }                                                                                         \
+  ORACLE_EXPORT void oracle_weighted_kmeanspp_##SUF(int seed, int m, int d, int k,           \
+                                                    const T *data, const T *weights,        \
+                                                    int *chosen) {                          \
+    std::vector<T> w(weights, weights + m);                                                 \
+    weighted_kmeanspp<T>(seed, m, d, k, data, w.data(), chosen);                            \
+  }                                                                                         \
+  ORACLE_EXPORT int oracle_kmeans_parallel_##SUF(int64_t n, int d, int k, const T *X,       \
+                                                 int seed, int cap, int *cand_rows,         \
+                                                 int *round_count, double *phi, T *weights, \
+                                                 int *chosen, T *C_out, int threads) {      \
+    return kmeans_parallel<T>(n, d, k, X, seed, cap, cand_rows, round_count, phi, weights,  \
+                              chosen, C_out, threads);                                      \
+  }
+DEFINE_SEED_FOR(float, f32)
+DEFINE_SEED_FOR(double, f64)
 
 // Seeded random-row initialisation: a permutation of 0..n-1 by
 // std::shuffle(v.begin(), v.end(), std::default_random_engine(seed)); the

@@ -75,14 +75,17 @@ def label_report(oracle, X, C, got, want, gap_rtol=GAP_RTOL, noise_mult=NOISE_MU
 
 
 def record(entry):
-    """Appends one JSON line to gpurun_out/parity_report.jsonl (the per-configuration
-    parity table is assembled from these); never fails a test."""
+    """Appends one JSON line to the file named by the environment variable
+    H2O4GPU_PARITY_REPORT (the per-configuration parity table is assembled from these);
+    without the variable nothing is written. Never fails a test."""
     import json
     import os
+    path = os.environ.get("H2O4GPU_PARITY_REPORT")
+    if not path:
+        return
     try:
-        out = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out")
-        os.makedirs(out, exist_ok=True)
-        with open(os.path.join(out, "parity_report.jsonl"), "a") as f:
+        os.makedirs(os.path.dirname(os.path.abspath(path)), exist_ok=True)
+        with open(path, "a") as f:
             f.write(json.dumps(entry) + "\n")
     except OSError:
         pass

@@ -4,7 +4,7 @@ Scaled-down rows (same d and k) are checked against the CPU oracle in lock-step 
 end-to-end over the full iteration count; the full shapes are checked in lock-step on ALL
 rows (one oracle assignment costs seconds at most), end to end for as many iterations as
 the CPU side affords, and through size-independent properties. Every full-size run
-appends its near-tie accounting to gpurun_out/parity_report.jsonl.
+appends its near-tie accounting to the file named by H2O4GPU_PARITY_REPORT, when set.
 """
 import numpy as np
 import pytest
