@@ -495,7 +495,8 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
     const T *__restrict__ X, const T *__restrict__ xnorm,
     const T *__restrict__ C, const T *__restrict__ cnorm,
     int *__restrict__ labels, T *__restrict__ mindist, int64_t n, int d, int k,
-    int kp, double *__restrict__ psums, int *__restrict__ pcounts, int c_off, int merge) {
+    int kp, double *__restrict__ psums, int *__restrict__ pcounts, int c_off, int merge,
+    int sets, int kps, int kset) {
   constexpr int TPB = NW * 64;
   typedef Mfma<T> M;
   constexpr int MT = M::MT, KL = M::KL, NACC = M::NACC, VW = M::VW;
@@ -573,7 +574,11 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
       Cs[cs_slot(c, j)] = v;
     }
   }
-  for (int c = tid; c < kp; c += TPB) ccs[c] = (c < k && cnorm) ? cnorm[c] : pos_inf<T>();
+  // Stacked model (sets > 1): `sets` independent centroid sets laid end to end, each padded
+  // to kps rows (a multiple of the tile height) of which the first kset are centroids; a
+  // padding row's norm is +inf, so it can never win. One set: kps = kp, kset = k.
+  for (int c = tid; c < kp; c += TPB)
+    ccs[c] = (c < k && (c % kps) < kset && cnorm) ? cnorm[c] : pos_inf<T>();
   __syncthreads();
   if (cnorm == nullptr) {
     // No norm buffer given: take the norms from the staged centroids. A staged value is
@@ -581,6 +586,7 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
     // separately) is bit for bit what row_norms / post_update would have stored.
 #pragma clang fp contract(off)
     for (int c = tid; c < k; c += TPB) {
+      if ((c % kps) >= kset) continue;
       T acc = 0;
       for (int j = 0; j < d; j++) {
         const T v = (T)-0.5 * Cs[cs_slot(c, j)];
@@ -679,13 +685,6 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
     int bidx[ROWT];
     unsigned bkey[ROWT];  // float32 path: running minimum key and its tile
     int btile[ROWT];
-#pragma unroll
-    for (int rt = 0; rt < ROWT; rt++) {
-      best[rt] = argmin_start<T>();
-      bidx[rt] = -1;
-      bkey[rt] = 0x7F7FFFF0u;  // FLT_MAX with the index bits cleared
-      btile[rt] = -1;
-    }
     auto tile_mma = [&](acc_t (&acc)[ROWT], int t) {
 #pragma unroll
       for (int v = 0; v < NACC; v++) {
@@ -753,53 +752,64 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
     // (Software-pipelining tile t's matrix work against tile t-1's argmin with a second
     // accumulator set measured no faster: the two do not overlap on this hardware, and
     // the extra registers cost occupancy.)
-    for (int t = 0; t < KT; t++) {
-      acc_t acc[ROWT];
-      tile_mma(acc, t);
-      tile_argmin(acc, t);
-    }
-    if constexpr (KEYS) {
+    const int tps = KT / sets;  // tiles per centroid set
+    for (int set = 0; set < sets; set++) {
 #pragma unroll
       for (int rt = 0; rt < ROWT; rt++) {
-        best[rt] = __uint_as_float(bkey[rt] & 0xFFFFFFF0u);
-        bidx[rt] = btile[rt] < 0 ? -1 : btile[rt] * MT + key_row(bkey[rt] & 15u, g);
+        best[rt] = argmin_start<T>();
+        bidx[rt] = -1;
+        bkey[rt] = 0x7F7FFFF0u;  // FLT_MAX with the index bits cleared
+        btile[rt] = -1;
       }
-    }
-#pragma unroll
-    for (int rt = 0; rt < ROWT; rt++) {
-#pragma unroll
-      for (int off = MT; off < 64; off <<= 1) {
-        const T ob = __shfl_xor(best[rt], off, 64);
-        const int oi = __shfl_xor(bidx[rt], off, 64);
-        argmin_merge(best[rt], bidx[rt], ob, oi);
+      for (int t = set * tps; t < (set + 1) * tps; t++) {
+        acc_t acc[ROWT];
+        tile_mma(acc, t);
+        tile_argmin(acc, t);
       }
-      const int64_t row = wrow0 + rt * MT + r;
-      if (g == 0 && row < n) {
-        // A model too large for LDS is swept in chunks of centroids, one launch each:
-        // C and cnorm then point at the chunk, c_off is its first centroid, and from the
-        // second chunk on (merge) the row's result so far is read back and kept unless
-        // this chunk is strictly closer (earlier chunks hold the lower indices).
-        T bv = best[rt];
-        int bi = bidx[rt] < 0 ? -1 : bidx[rt] + c_off;
-        if (!FUSE && merge) argmin_merge(bv, bi, pm[rt], pl[rt]);  // (a fused step is never chunked)
-        labels[row] = bi;
-        if (mindist) mindist[row] = bv;
+      if constexpr (KEYS) {
+#pragma unroll
+        for (int rt = 0; rt < ROWT; rt++) {
+          best[rt] = __uint_as_float(bkey[rt] & 0xFFFFFFF0u);
+          bidx[rt] = btile[rt] < 0 ? -1 : btile[rt] * MT + key_row(bkey[rt] & 15u, g);
+        }
       }
-      if (FUSE && row < n && bidx[rt] >= 0) {
-        double *srow = sums + (size_t)bidx[rt] * SD;
 #pragma unroll
-        for (int q = 0; q < NV; q++) {
-          if (LOAD == 1 || q < nq) {
+      for (int rt = 0; rt < ROWT; rt++) {
 #pragma unroll
-            for (int e = 0; e < VW; e++) {
-              const int f = (q * KL + g) * VW + e;  // the feature this register holds
-              if (LOAD == 1 || f < d) unsafeAtomicAdd(srow + f, (double)x[rt][q * VW + e]);
+        for (int off = MT; off < 64; off <<= 1) {
+          const T ob = __shfl_xor(best[rt], off, 64);
+          const int oi = __shfl_xor(bidx[rt], off, 64);
+          argmin_merge(best[rt], bidx[rt], ob, oi);
+        }
+        const int64_t row = wrow0 + rt * MT + r;
+        if (g == 0 && row < n) {
+          // A model too large for LDS is swept in chunks of centroids, one launch each:
+          // C and cnorm then point at the chunk, c_off is its first centroid, and from the
+          // second chunk on (merge) the row's result so far is read back and kept unless
+          // this chunk is strictly closer (earlier chunks hold the lower indices).
+          // (a set's labels count from its own first centroid and go to its own [n] block)
+          T bv = best[rt];
+          int bi = bidx[rt] < 0 ? -1 : bidx[rt] + c_off - set * kps;
+          if (!FUSE && merge) argmin_merge(bv, bi, pm[rt], pl[rt]);  // (a fused step is never chunked)
+          labels[(int64_t)set * n + row] = bi;
+          if (mindist) mindist[(int64_t)set * n + row] = bv;
+        }
+        if (FUSE && row < n && bidx[rt] >= 0) {
+          double *srow = sums + (size_t)bidx[rt] * SD;
+#pragma unroll
+          for (int q = 0; q < NV; q++) {
+            if (LOAD == 1 || q < nq) {
+#pragma unroll
+              for (int e = 0; e < VW; e++) {
+                const int f = (q * KL + g) * VW + e;  // the feature this register holds
+                if (LOAD == 1 || f < d) unsafeAtomicAdd(srow + f, (double)x[rt][q * VW + e]);
+              }
             }
           }
+          if (g == 0) atomicAdd(&cnt[bidx[rt]], 1);
         }
-        if (g == 0) atomicAdd(&cnt[bidx[rt]], 1);
       }
-    }
+    }  // centroid sets
   }
   if (FUSE) {
     __syncthreads();
@@ -1233,9 +1243,13 @@ template <typename T, int DP, int ROWT, bool FUSE, int NW>
 static int launch_rowstat_nw(hipStream_t s, const T *X, const T *xnorm, const T *C,
                              const T *cnorm, int *labels, T *mindist, int64_t n, int d,
                              int k, int num_cu, double *psums, int *pcounts, int *slots,
-                             size_t lds, int c_off, int merge, bool exact) {
+                             size_t lds, int c_off, int merge, bool exact, const StackShape &st) {
   const int MT = Mfma<T>::MT;
   const int kp = (k + MT - 1) / MT * MT;
+  const int sets = st.sets > 1 ? st.sets : 1;
+  const int kps = sets > 1 ? st.kps : kp, kset = sets > 1 ? st.kset : k;
+  if (sets > 1 && (kps % MT != 0 || (int64_t)sets * kps != k || kset > kps || c_off != 0 || merge))
+    return H2O4GPU_KMEANS_EARG;
   // (row tiles go round the workgroups before a second wavefront of any gets one, so a
   // small data set spreads over as many CUs as it has tiles)
   const int rows_per_wave = ROWT * MT;
@@ -1252,7 +1266,8 @@ static int launch_rowstat_nw(hipStream_t s, const T *X, const T *xnorm, const T 
     auto kern = assign_rowstat_kernel<T, DP, ROWT, LOAD, FUSE, NW, EXACT>;                    \
     KM_TRY(ensure_dynamic_lds(reinterpret_cast<const void *>(kern), lds));                    \
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), lds, s, X, xnorm, C, cnorm, \
-                       labels, mindist, n, d, k, kp, psums, pcounts, c_off, merge);           \
+                       labels, mindist, n, d, k, kp, psums, pcounts, c_off, merge, sets, kps, \
+                       kset);                                                                 \
   } while (0)
   // the exact-compare form exists for the float32 assignment-only kernels
 #define KM_RS_LAUNCH(LOAD)                                       \
@@ -1278,7 +1293,7 @@ static int launch_rowstat_dp(hipStream_t s, const T *X, const T *xnorm,
                              const T *C, const T *cnorm, int *labels,
                              T *mindist, int64_t n, int d, int k, int num_cu,
                              double *psums, int *pcounts, int *slots, int c_off, int merge,
-                             bool exact) {
+                             bool exact, const StackShape &st) {
   const size_t lds = FUSE ? rowstat_fused_lds<T>(d, k) : rowstat_lds<T>(d, k);
   // Shapes whose register use fits 128 VGPRs run one 16-wavefront workgroup per CU, which
   // measured ahead of two 4-wave workgroups everywhere it applies (float32 10M x 32 and
@@ -1287,14 +1302,14 @@ static int launch_rowstat_dp(hipStream_t s, const T *X, const T *xnorm,
                         (sizeof(T) == 8 && ((DP <= 32 && ROWT <= 2) || (DP == 64 && ROWT == 1)));
   if (!wide && rowstat_two_per_cu(lds))
     return launch_rowstat_nw<T, DP, ROWT, FUSE, 4>(s, X, xnorm, C, cnorm, labels, mindist, n, d,
-                                                   k, num_cu, psums, pcounts, slots, lds, c_off, merge, exact);
+                                                   k, num_cu, psums, pcounts, slots, lds, c_off, merge, exact, st);
   // one workgroup per CU: as many wavefronts as the register budget allows
   if constexpr (wide)
     return launch_rowstat_nw<T, DP, ROWT, FUSE, 16>(s, X, xnorm, C, cnorm, labels, mindist, n, d,
-                                                    k, num_cu, psums, pcounts, slots, lds, c_off, merge, exact);
+                                                    k, num_cu, psums, pcounts, slots, lds, c_off, merge, exact, st);
   else
     return launch_rowstat_nw<T, DP, ROWT, FUSE, 8>(s, X, xnorm, C, cnorm, labels, mindist, n, d,
-                                                   k, num_cu, psums, pcounts, slots, lds, c_off, merge, exact);
+                                                   k, num_cu, psums, pcounts, slots, lds, c_off, merge, exact, st);
 }
 
 template <typename T, bool FUSE>
@@ -1302,13 +1317,13 @@ struct RowstatDispatch;
 #define KM_ROWSTAT_CASE(T, DP, ROWT)                                                  \
   case DP:                                                                            \
     return launch_rowstat_dp<T, DP, ROWT, FUSE>(s, X, xnorm, C, cnorm, labels, mindist, \
-                                                n, d, k, num_cu, psums, pcounts, slots, c_off, merge, exact)
+                                                n, d, k, num_cu, psums, pcounts, slots, c_off, merge, exact, st)
 template <bool FUSE>
 struct RowstatDispatch<float, FUSE> {
   static int run(hipStream_t s, const float *X, const float *xnorm, const float *C,
                  const float *cnorm, int *labels, float *mindist, int64_t n, int d,
                  int k, int num_cu, double *psums, int *pcounts, int *slots, int c_off = 0,
-                 int merge = 0, bool exact = false) {
+                 int merge = 0, bool exact = false, const StackShape &st = StackShape()) {
     switch (rowstat_dp<float>(d)) {
       KM_ROWSTAT_CASE(float, 8, 2);
       KM_ROWSTAT_CASE(float, 16, 2);
@@ -1324,7 +1339,7 @@ struct RowstatDispatch<double, FUSE> {
   static int run(hipStream_t s, const double *X, const double *xnorm, const double *C,
                  const double *cnorm, int *labels, double *mindist, int64_t n, int d,
                  int k, int num_cu, double *psums, int *pcounts, int *slots, int c_off = 0,
-                 int merge = 0, bool exact = false) {
+                 int merge = 0, bool exact = false, const StackShape &st = StackShape()) {
     switch (rowstat_dp<double>(d)) {
       // two row tiles keep these within 128 registers, i.e. 16 wavefronts per CU
       KM_ROWSTAT_CASE(double, 8, 2);
@@ -1427,17 +1442,18 @@ template <typename T>
 int launch_assign_accumulate(hipStream_t s, int variant, const T *X, const T *xnorm, const T *C,
                              const T *cnorm, int *labels, T *mindist, int64_t n, int d,
                              int k, int num_cu, double *psums, int *pcounts, int *slots,
-                             int *used) {
+                             int *used, StackShape st) {
   // cnorm == nullptr: the kernel computes the centroid norms from C itself
   if (n <= 0 || d < 1 || k < 1) return H2O4GPU_KMEANS_EARG;
   const int v = pick_assign_variant<T>(variant, n, d, k);
   if (used) *used = v;
+  if (st.sets > 1 && v != ASSIGN_ROWSTAT) return H2O4GPU_KMEANS_EARG;
   if (v == ASSIGN_VALU && valu_fused_applies(d, k))
     return launch_valu_fused<T, true>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu,
                                       psums, pcounts, slots);
   if (v != ASSIGN_ROWSTAT) return H2O4GPU_KMEANS_EARG;
   return RowstatDispatch<T, true>::run(s, X, xnorm, C, cnorm, labels, mindist, n, d, k,
-                                       num_cu, psums, pcounts, slots);
+                                       num_cu, psums, pcounts, slots, 0, 0, false, st);
 }
 
 template <typename T, int MODE, int BCW>
@@ -1496,12 +1512,17 @@ static int launch_tiled(hipStream_t s, const T *X, const T *xnorm, const T *C,
 template <typename T>
 int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
                   const T *C, const T *cnorm, int *labels, T *mindist, int64_t n,
-                  int d, int k, int num_cu, int *used, bool exact) {
+                  int d, int k, int num_cu, int *used, bool exact, StackShape st) {
   if (n <= 0) return 0;
   if (d < 1 || k < 1) return H2O4GPU_KMEANS_EARG;
   const int v = pick_assign_variant<T>(variant, n, d, k);
   if (v < 0) return H2O4GPU_KMEANS_EARG;
   if (used) *used = v;
+  if (st.sets > 1) {  // stacked sets: the row-stationary kernel with the whole model in LDS
+    if (v != ASSIGN_ROWSTAT || rowstat_chunk<T>(d, k) < k || !mindist) return H2O4GPU_KMEANS_EARG;
+    return RowstatDispatch<T, false>::run(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu,
+                                          nullptr, nullptr, nullptr, 0, 0, exact, st);
+  }
   switch (v) {
     case ASSIGN_VALU:
       // The staged kernels of the fused step, minus the sums: the one-thread-per-row
@@ -1546,19 +1567,19 @@ template int fused_slots<double>(int, int64_t, int, int, int);
 template int launch_assign_accumulate<float>(hipStream_t, int, const float *, const float *,
                                              const float *, const float *, int *, float *,
                                              int64_t, int, int, int, double *, int *, int *,
-                                             int *);
+                                             int *, StackShape);
 template int launch_assign_accumulate<double>(hipStream_t, int, const double *, const double *,
                                               const double *, const double *, int *, double *,
                                               int64_t, int, int, int, double *, int *, int *,
-                                              int *);
+                                              int *, StackShape);
 template int pick_assign_variant<float>(int, int64_t, int, int);
 template int pick_assign_variant<double>(int, int64_t, int, int);
 template int launch_assign<float>(hipStream_t, int, const float *, const float *,
                                   const float *, const float *, int *, float *,
-                                  int64_t, int, int, int, int *, bool);
+                                  int64_t, int, int, int, int *, bool, StackShape);
 template int launch_assign<double>(hipStream_t, int, const double *, const double *,
                                    const double *, const double *, int *, double *,
-                                   int64_t, int, int, int, int *, bool);
+                                   int64_t, int, int, int, int *, bool, StackShape);
 template int launch_transform<float>(hipStream_t, const float *, const float *,
                                      const float *, const float *, float *, int64_t,
                                      int64_t, int, int, int);

@@ -167,7 +167,11 @@ struct h2o4gpu_kmeans_handle {
   int elem_size = 0;
   int64_t n = 0;
   int d = 0;
-  int k = 0;
+  int k = 0;  // rows of the model; a stacked handle holds sets * kps of them
+  // stacked restarts: `sets` independent centroid sets of kset centroids each, every set
+  // padded to kps model rows; cur_set is the set the per-set calls address
+  int sets = 1, kset = 0, kps = 0, cur_set = 0;
+  std::vector<int> set_iterations;
   int dev = 0;
   int verbose = 0;
   int num_cu = 0;
@@ -222,6 +226,7 @@ struct h2o4gpu_kmeans_handle {
   virtual int transform_host(size_t rows, const void *X, void *dist) = 0;
   virtual int transform_resident(void *d_dist) = 0;
   virtual int release() = 0;
+  int kk() const { return sets > 1 ? kset : k; }  // centroids of one set
 
   hipEvent_t get_event() {
     if (!pool.empty()) {
@@ -514,6 +519,16 @@ struct Engine : h2o4gpu_kmeans_handle {
   int *kpp_rows = nullptr;  // [k] rows chosen so far by k-means++
   T *kpp_dcc = nullptr;     // [k] distances newest centre -> earlier centres
   bool have_data = false, have_centroids = false, have_mindist = false;
+  int *d_frozen = nullptr;  // [sets] flags of a stacked handle's sets that have converged
+  StackShape shape() const {
+    StackShape st;
+    st.sets = sets;
+    st.kps = kps;
+    st.kset = kset;
+    return st;
+  }
+  size_t set_off() const { return sets > 1 ? (size_t)cur_set * kps : 0; }  // first model row of the set
+  size_t row_off() const { return sets > 1 ? (size_t)cur_set * (size_t)n : 0; }  // its block of labels
 
   template <typename U>
   int dalloc(U **p, size_t count) {
@@ -552,10 +567,18 @@ struct Engine : h2o4gpu_kmeans_handle {
       KM_HIP_TRY(hipMemcpyAsync(cnorm, inf.data(), kpad * sizeof(T), hipMemcpyHostToDevice, stream));
       KM_HIP_TRY(hipStreamSynchronize(stream));
     }
+    if (sets > 1) {
+      // every step of a stacked handle is the fused row-stationary kernel over the whole model
+      if (pick_assign_variant<T>(ASSIGN_AUTO, n, d, k) != ASSIGN_ROWSTAT ||
+          fused_slots<T>(ASSIGN_AUTO, n, d, k, num_cu) <= 0)
+        return H2O4GPU_KMEANS_EARG;
+      KM_TRY(dalloc(&d_frozen, sets));
+      KM_HIP_TRY(hipMemsetAsync(d_frozen, 0, (size_t)sets * sizeof(int), stream));
+    }
     KM_TRY(dalloc(&counts, k));
-    KM_TRY(dalloc(&labels, n));
+    KM_TRY(dalloc(&labels, (size_t)n * sets));
     KM_TRY(dalloc(&xnorm, n));
-    KM_TRY(dalloc(&mindist, n));
+    KM_TRY(dalloc(&mindist, (size_t)n * sets));
     int slots = plan.row_blocks;
     const int fs = fused_slots<T>(ASSIGN_AUTO, n, d, k, num_cu);
     if (fs > slots) slots = fs;
@@ -572,13 +595,13 @@ struct Engine : h2o4gpu_kmeans_handle {
       KM_TRY(dalloc(&bucket_partials, bucket_partial_slots(n, k) * d));
     }
     KM_TRY(dalloc(&shift_partials, (size_t)max_shift_partials(d, k) + 1));
-    KM_TRY(dalloc(&shift2, 1));
+    KM_TRY(dalloc(&shift2, (size_t)sets));
     KM_TRY(dalloc(&sum_partials, sum_partials_needed() + 1));
     KM_TRY(dalloc(&kpp_bsums, (n + KPP_BLOCK - 1) / KPP_BLOCK + 1));
     KM_TRY(dalloc(&kpp_rows, (size_t)k + 1));
     KM_TRY(dalloc(&kpp_dcc, (size_t)k + 1));
     // the reference's label vector starts zeroed (thrust::device_vector<int>)
-    KM_HIP_TRY(hipMemsetAsync(labels, 0, (size_t)n * sizeof(int), stream));
+    KM_HIP_TRY(hipMemsetAsync(labels, 0, (size_t)n * sets * sizeof(int), stream));
     KM_HIP_TRY(hipMemsetAsync(counts, 0, (size_t)k * sizeof(int), stream));
     KM_HIP_TRY(hipStreamSynchronize(stream));
     log_msg(verbose, LOG_DEBUG,
@@ -603,7 +626,7 @@ struct Engine : h2o4gpu_kmeans_handle {
     void *ptrs[] = {xnorm,  C[0],    C[1],           cnorm,  labels,       mindist,
                     counts, psums,   pcounts,        shift_partials, shift2,
                     sum_partials, kpp_bsums, kpp_rows, kpp_dcc, order, order_label, bucket_offsets,
-                    bucket_hist, bucket_seg, bucket_total, bucket_partials};
+                    bucket_hist, bucket_seg, bucket_total, bucket_partials, d_frozen};
     for (void *p : ptrs)
       if (p) (void)hipFree(p);
     if (stream) (void)hipStreamDestroy(stream);
@@ -648,7 +671,8 @@ struct Engine : h2o4gpu_kmeans_handle {
   int set_centroids_host(const void *hC) override {
     KM_HIP_TRY(hipSetDevice(dev));
     if (!hC) return H2O4GPU_KMEANS_EARG;
-    KM_HIP_TRY(hipMemcpyAsync(C[cur], hC, (size_t)k * d * sizeof(T), hipMemcpyHostToDevice, stream));
+    KM_HIP_TRY(hipMemcpyAsync(C[cur] + set_off() * d, hC, (size_t)kk() * d * sizeof(T),
+                              hipMemcpyHostToDevice, stream));
     KM_TRY(centroids_changed());
     KM_HIP_TRY(hipStreamSynchronize(stream));
     return 0;
@@ -659,6 +683,7 @@ struct Engine : h2o4gpu_kmeans_handle {
   int init_random_rows(int seed) override {
     KM_HIP_TRY(hipSetDevice(dev));
     if (!have_data) return H2O4GPU_KMEANS_ESTATE;
+    const int k = kk();
     if ((int64_t)k > n) return H2O4GPU_KMEANS_EARG;
     unsigned useed = (unsigned)seed;
     if (seed < 0) {
@@ -674,15 +699,16 @@ struct Engine : h2o4gpu_kmeans_handle {
   int start_from_rows(const int *rows) override {
     KM_HIP_TRY(hipSetDevice(dev));
     if (!have_data || !rows) return H2O4GPU_KMEANS_ESTATE;
-    last_seed_rows.assign(rows, rows + k);
+    last_seed_rows.assign(rows, rows + kk());
     return init_from_rows(rows);
   }
 
   int init_from_rows(const int *idx_host) {
+    const int k = kk();
     int *didx = nullptr;
     KM_TRY(dalloc(&didx, k));
     hipError_t e = hipMemcpyAsync(didx, idx_host, (size_t)k * sizeof(int), hipMemcpyHostToDevice, stream);
-    int rc = e == hipSuccess ? launch_gather_rows<T>(stream, X, didx, C[cur], k, d)
+    int rc = e == hipSuccess ? launch_gather_rows<T>(stream, X, didx, C[cur] + set_off() * d, k, d)
                              : H2O4GPU_KMEANS_EDEVICE;
     if (rc == 0) rc = centroids_changed();
     (void)hipStreamSynchronize(stream);
@@ -699,6 +725,7 @@ struct Engine : h2o4gpu_kmeans_handle {
   int init_plusplus(int seed) override {
     KM_HIP_TRY(hipSetDevice(dev));
     if (!have_data) return H2O4GPU_KMEANS_ESTATE;
+    const int k = kk();
     if ((int64_t)k > n) return H2O4GPU_KMEANS_EARG;
     std::mt19937 gen(seed >= 0 ? (unsigned)seed : std::random_device{}());
     std::uniform_int_distribution<> first(0, (int)(n - 1));
@@ -747,7 +774,7 @@ struct Engine : h2o4gpu_kmeans_handle {
       }
       idx[c] = (int)pick;
     }
-    have_mindist = true;  // minimum distance of every row to the k chosen centres
+    have_mindist = sets == 1;  // minimum distance of every row to the k chosen centres
     last_seed_rows = idx;
     return init_from_rows(idx.data());
   }
@@ -767,7 +794,7 @@ struct Engine : h2o4gpu_kmeans_handle {
   int init_parallel(int seed) override {
     KM_HIP_TRY(hipSetDevice(dev));
     if (!have_data) return H2O4GPU_KMEANS_ESTATE;
-    if ((int64_t)k > n) return H2O4GPU_KMEANS_EARG;
+    if ((int64_t)kk() > n) return H2O4GPU_KMEANS_EARG;
     seed_info = ParallelSeedInfo();
     std::mt19937 gen(seed);
     std::uniform_int_distribution<> dis(0, (int)(n - 1));
@@ -796,6 +823,7 @@ struct Engine : h2o4gpu_kmeans_handle {
   }
   int parallel_rounds(int seed, std::vector<int> &all, std::vector<int> &recent, T **cost, T **Cc,
                       T **ccn, T **best, int **list, int **didx, int **dcount) {
+    const int k = kk();
     const int64_t nb = (n + KPP_BLOCK - 1) / KPP_BLOCK;
     size_t cap_model = 0, cap_norm = 0, cap_idx = 0, cap_best = 0;
     const int list_cap = (int)n;
@@ -855,10 +883,10 @@ struct Engine : h2o4gpu_kmeans_handle {
     seed_info.chosen.assign((size_t)k, -1);
     if (M <= k) {  // kmeans_h2o4gpu.cu:536-540: the candidates, then zero rows
       for (int c = 0; c < M; c++) seed_info.chosen[(size_t)c] = c;
-      KM_HIP_TRY(hipMemsetAsync(C[cur], 0, (size_t)k * d * sizeof(T), stream));
+      KM_HIP_TRY(hipMemsetAsync(C[cur] + set_off() * d, 0, (size_t)k * d * sizeof(T), stream));
       KM_TRY(regrow(didx, &cap_idx, (size_t)M));
       KM_HIP_TRY(hipMemcpyAsync(*didx, all.data(), (size_t)M * sizeof(int), hipMemcpyHostToDevice, stream));
-      KM_TRY(launch_gather_rows<T>(stream, X, *didx, C[cur], M, d));
+      KM_TRY(launch_gather_rows<T>(stream, X, *didx, C[cur] + set_off() * d, M, d));
       last_seed_rows.assign((size_t)k, -1);
       std::copy(all.begin(), all.end(), last_seed_rows.begin());
       KM_TRY(centroids_changed());
@@ -944,7 +972,7 @@ struct Engine : h2o4gpu_kmeans_handle {
     KM_TRY(ensure_cnorm());
     PROFILED("assign", launch_assign<T>(stream, opt_assign, X, xnorm, C[cur], cnorm,
                                         labels, mindist, n, d, k, num_cu, &last_variant,
-                                        opt_exact != 0));
+                                        opt_exact != 0, shape()));
     have_mindist = true;
     return 0;
   }
@@ -967,15 +995,16 @@ struct Engine : h2o4gpu_kmeans_handle {
     // (the exact-compare argmin exists in the assignment-only kernels)
     const bool exact_mfma = opt_exact && sizeof(T) == 4 &&
                             pick_assign_variant<T>(opt_assign, n, d, k) != ASSIGN_VALU;
-    if (opt_fuse && !exact_mfma && fused_slots<T>(opt_assign, n, d, k, num_cu) > 0) {
+    if ((opt_fuse || sets > 1) && !exact_mfma && fused_slots<T>(opt_assign, n, d, k, num_cu) > 0) {
       int slots = 0;
       PROFILED("assign_accumulate",
                launch_assign_accumulate<T>(stream, opt_assign, X, xnorm, C[cur], (const T *)nullptr,
                                            labels, mindist, n, d, k, num_cu, psums, pcounts, &slots,
-                                           &last_variant));
+                                           &last_variant, shape()));
       have_mindist = true;
       return finish_update(slots, want_shift);
     }
+    if (sets > 1) return H2O4GPU_KMEANS_ESTATE;  // a stacked handle has no other step
     KM_TRY(assign());
     return update_async();
   }
@@ -984,6 +1013,20 @@ struct Engine : h2o4gpu_kmeans_handle {
   // norms are marked stale and the scalar of this step does not exist.
   int finish_update(int slots, bool post) {
     int nsp = 0;
+    if (sets > 1 && post) {
+      // per-set convergence: frozen sets keep their centroids; every set's squared shift is
+      // the ordered sum of its own partials
+      PROFILED("finalize", launch_finalize<T>(stream, slots, psums, pcounts, C[cur], C[cur ^ 1],
+                                              counts, shift_partials, &nsp, d, k, d_frozen, kps));
+      const int per = nsp / sets;
+      for (int s = 0; s < sets; s++)
+        PROFILED("post_update",
+                 launch_post_update<T>(stream, C[cur ^ 1] + (size_t)s * kps * d, cnorm + (size_t)s * kps,
+                                       shift_partials + (size_t)s * per, per, shift2 + s, d, kps));
+      cnorm_stale = false;
+      cur ^= 1;
+      return 0;
+    }
     PROFILED("finalize", launch_finalize<T>(stream, slots, psums, pcounts, C[cur], C[cur ^ 1],
                                             counts, shift_partials, &nsp, d, k));
     if (post)
@@ -1004,7 +1047,7 @@ struct Engine : h2o4gpu_kmeans_handle {
 
   int update(double *s2) override {
     KM_HIP_TRY(hipSetDevice(dev));
-    if (!have_data || !have_centroids) return H2O4GPU_KMEANS_ESTATE;
+    if (!have_data || !have_centroids || sets > 1) return H2O4GPU_KMEANS_ESTATE;
     KM_TRY(update_async());
     if (s2) KM_TRY(read_shift2(s2));
     return 0;
@@ -1018,7 +1061,9 @@ struct Engine : h2o4gpu_kmeans_handle {
     if (!have_data || !have_centroids) return H2O4GPU_KMEANS_ESTATE;
     maybe_install_signal_handlers();
     int updates = 0;
-    if (threshold > 0 && max_iterations > 0) {
+    if (sets > 1) {
+      KM_TRY(fit_stacked(max_iterations, threshold, &updates));
+    } else if (threshold > 0 && max_iterations > 0) {
       KM_TRY(fit_with_threshold(max_iterations, threshold, &updates));
     } else {
       for (int i = 0; i < max_iterations; i++) {
@@ -1039,6 +1084,50 @@ struct Engine : h2o4gpu_kmeans_handle {
     }
     KM_HIP_TRY(hipStreamSynchronize(stream));
     if (iters) *iters = updates;
+    return 0;
+  }
+
+  // Every set of a stacked handle runs the loop of kmeans_impl.h:109-232 on its own: the
+  // same kernel labels the rows against all sets and sums them per set; with a threshold,
+  // a set whose squared shift falls below it keeps its centroids from then on (its labels
+  // are still refreshed, and stay what its final relabel would give) while the others go
+  // on. The scalars of an iteration are read before the next one is queued: unlike the
+  // single-set loop this one waits for the host once per iteration.
+  int fit_stacked(int max_iterations, double threshold, int *updates_out) {
+    const bool test = threshold > 0;
+    std::vector<int> frozen((size_t)sets, 0);
+    std::vector<T> sh((size_t)sets);
+    set_iterations.assign((size_t)sets, 0);
+    KM_HIP_TRY(hipMemsetAsync(d_frozen, 0, (size_t)sets * sizeof(int), stream));
+    int updates = 0, live = sets;
+    for (int i = 0; i < max_iterations && live > 0; i++) {
+      KM_TRY(step_async(test));
+      updates = i + 1;
+      for (int s = 0; s < sets; s++)
+        if (!frozen[(size_t)s]) set_iterations[(size_t)s] = i + 1;
+      if (test) {
+        KM_HIP_TRY(hipMemcpyAsync(sh.data(), shift2, (size_t)sets * sizeof(T), hipMemcpyDeviceToHost, stream));
+        KM_HIP_TRY(hipStreamSynchronize(stream));
+        bool changed = false;
+        for (int s = 0; s < sets; s++) {
+          if (!frozen[(size_t)s] && (double)sh[(size_t)s] < threshold) {
+            frozen[(size_t)s] = 1;
+            changed = true;
+            live--;
+          }
+        }
+        if (changed)
+          KM_HIP_TRY(hipMemcpyAsync(d_frozen, frozen.data(), (size_t)sets * sizeof(int), hipMemcpyHostToDevice,
+                                    stream));
+      }
+      if (g_stop_flag) {
+        fprintf(stderr, "Signal caught. Terminated early.\n");
+        g_stop_flag = 0;
+        break;
+      }
+    }
+    if (max_iterations > 0) KM_TRY(assign());  // final relabel of every set with its final centroids
+    *updates_out = updates;
     return 0;
   }
 
@@ -1101,6 +1190,7 @@ struct Engine : h2o4gpu_kmeans_handle {
   }
 
   int set_labels_host(const int *h) override {
+    if (sets > 1) return H2O4GPU_KMEANS_ESTATE;
     KM_HIP_TRY(hipSetDevice(dev));
     KM_HIP_TRY(hipMemcpyAsync(labels, h, (size_t)n * sizeof(int), hipMemcpyHostToDevice, stream));
     KM_HIP_TRY(hipStreamSynchronize(stream));
@@ -1112,24 +1202,26 @@ struct Engine : h2o4gpu_kmeans_handle {
     KM_HIP_TRY(hipStreamSynchronize(stream));
     return 0;
   }
-  int get_centroids(void *out) override { return d2h(out, C[cur], (size_t)k * d * sizeof(T)); }
-  int get_labels(int *out) override { return d2h(out, labels, (size_t)n * sizeof(int)); }
-  int get_counts(int *out) override { return d2h(out, counts, (size_t)k * sizeof(int)); }
+  int get_centroids(void *out) override {
+    return d2h(out, C[cur] + set_off() * d, (size_t)kk() * d * sizeof(T));
+  }
+  int get_labels(int *out) override { return d2h(out, labels + row_off(), (size_t)n * sizeof(int)); }
+  int get_counts(int *out) override { return d2h(out, counts + set_off(), (size_t)kk() * sizeof(int)); }
   int get_min_distances(void *out) override {
     if (!have_mindist) return H2O4GPU_KMEANS_ESTATE;
-    return d2h(out, mindist, (size_t)n * sizeof(T));
+    return d2h(out, mindist + row_off(), (size_t)n * sizeof(T));
   }
   int inertia(double *out) override {
     KM_HIP_TRY(hipSetDevice(dev));
     if (!have_mindist) return H2O4GPU_KMEANS_ESTATE;
     const int np = sum_partials_needed();
-    PROFILED("inertia_sum", launch_sum<T>(stream, mindist, n, sum_partials, np, sum_partials + np));
+    PROFILED("inertia_sum", launch_sum<T>(stream, mindist + row_off(), n, sum_partials, np, sum_partials + np));
     return d2h(out, sum_partials + np, sizeof(double));
   }
 
   int predict_host(size_t rows, const void *hX, int *out) override {
     KM_HIP_TRY(hipSetDevice(dev));
-    if (!have_centroids) return H2O4GPU_KMEANS_ESTATE;
+    if (!have_centroids || sets > 1) return H2O4GPU_KMEANS_ESTATE;
     if (rows == 0) return 0;
     T *dX = nullptr, *dxn = nullptr, *dmin = nullptr;
     int *dl = nullptr;
@@ -1163,7 +1255,7 @@ struct Engine : h2o4gpu_kmeans_handle {
   // this", kmeans_h2o4gpu.cu:936).
   int transform_host(size_t rows, const void *hX, void *hD) override {
     KM_HIP_TRY(hipSetDevice(dev));
-    if (!have_centroids) return H2O4GPU_KMEANS_ESTATE;
+    if (!have_centroids || sets > 1) return H2O4GPU_KMEANS_ESTATE;
     if (rows == 0) return 0;
     size_t batch = ((size_t)4 << 30) / ((size_t)k * sizeof(T));
     batch = batch / 128 * 128;
@@ -1202,7 +1294,7 @@ struct Engine : h2o4gpu_kmeans_handle {
   }
   int transform_resident(void *d_dist) override {
     KM_HIP_TRY(hipSetDevice(dev));
-    if (!have_data || !have_centroids || !d_dist) return H2O4GPU_KMEANS_ESTATE;
+    if (!have_data || !have_centroids || !d_dist || sets > 1) return H2O4GPU_KMEANS_ESTATE;
     KM_TRY(ensure_cnorm());
     PROFILED("transform", launch_transform<T>(stream, X, xnorm, C[cur], cnorm,
                                               static_cast<T *>(d_dist), n, n, d, k, num_cu));
@@ -1213,7 +1305,7 @@ struct Engine : h2o4gpu_kmeans_handle {
 
 template <typename T>
 static int create_engine(h2o4gpu_kmeans_handle **out, size_t rows, size_t cols, int k,
-                         int gpu_id, int verbose) {
+                         int gpu_id, int verbose, int sets = 1) {
   const int nvis = visible_devices();
   if (nvis < 1) {
     log_msg(verbose ? verbose : LOG_ERROR, LOG_ERROR, "no HIP device visible");
@@ -1225,6 +1317,12 @@ static int create_engine(h2o4gpu_kmeans_handle **out, size_t rows, size_t cols, 
   e->n = (int64_t)rows;
   e->d = (int)cols;
   e->k = k;
+  if (sets > 1) {
+    e->sets = sets;
+    e->kset = k;
+    e->kps = (k + 31) / 32 * 32;
+    e->k = sets * e->kps;
+  }
   e->verbose = verbose;
   if (gpu_id < 0) gpu_id = 0;
   e->dev = gpu_id % nvis;  // kmeans_init: gpu_id = gpu_idtry % n_gpuvis
@@ -1476,6 +1574,23 @@ static int predict_device_noalloc(size_t rows, size_t cols, int k, const T *dX, 
                           k, nd.num_cu, nullptr);
 }
 
+// Largest number of centroid sets (at most max_sets) of k centroids each that one stacked
+// handle can hold for rows of `cols` values: the stacked model and its per-centroid sums
+// must fit one CU's LDS beside each other. 1: no stacking for this shape.
+template <typename T>
+static int stack_width(size_t rows, size_t cols, int k, int max_sets) {
+  const int kps = (k + 31) / 32 * 32;
+  int best = 1;
+  for (int s = 2; s <= max_sets; s++) {
+    const int64_t K = (int64_t)s * kps;
+    if (K > 65536) break;
+    if (pick_assign_variant<T>(ASSIGN_AUTO, (int64_t)rows, (int)cols, (int)K) != ASSIGN_ROWSTAT) break;
+    if (fused_slots<T>(ASSIGN_AUTO, (int64_t)rows, (int)cols, (int)K, 1) <= 0) break;
+    best = s;
+  }
+  return best;
+}
+
 // ---------------------------------------------------------------------------
 // C ABI, part 3
 // ---------------------------------------------------------------------------
@@ -1497,6 +1612,36 @@ KM_API int h2o4gpu_kmeans_create(h2o4gpu_kmeans_handle **out, int elem_size, siz
   if (elem_size == 4) return create_engine<float>(out, rows, cols, k, gpu_id, verbose);
   if (elem_size == 8) return create_engine<double>(out, rows, cols, k, gpu_id, verbose);
   return H2O4GPU_KMEANS_EARG;
+}
+KM_API int h2o4gpu_kmeans_stack_width(int elem_size, size_t rows, size_t cols, int k, int max_sets) {
+  if (rows < 1 || cols < 1 || k < 1 || cols > 1000000ull || rows > 2147483647ull) return 1;
+  if (elem_size == 4) return stack_width<float>(rows, cols, k, max_sets);
+  if (elem_size == 8) return stack_width<double>(rows, cols, k, max_sets);
+  return 1;
+}
+KM_API int h2o4gpu_kmeans_create_stacked(h2o4gpu_kmeans_handle **out, int elem_size, size_t rows,
+                                         size_t cols, int k, int sets, int gpu_id, int verbose) {
+  if (!out) return H2O4GPU_KMEANS_EARG;
+  *out = nullptr;
+  if (sets < 2) return h2o4gpu_kmeans_create(out, elem_size, rows, cols, k, gpu_id, verbose);
+  if (rows < 1 || cols < 1 || k < 1 || rows > 2147483647ull || cols > 1000000ull ||
+      sets > h2o4gpu_kmeans_stack_width(elem_size, rows, cols, k, sets))
+    return H2O4GPU_KMEANS_EARG;
+  if (elem_size == 4) return create_engine<float>(out, rows, cols, k, gpu_id, verbose, sets);
+  if (elem_size == 8) return create_engine<double>(out, rows, cols, k, gpu_id, verbose, sets);
+  return H2O4GPU_KMEANS_EARG;
+}
+KM_API int h2o4gpu_kmeans_select_set(h2o4gpu_kmeans_handle *h, int set) {
+  KM_CHECK_HANDLE(h);
+  if (set < 0 || set >= h->sets) return H2O4GPU_KMEANS_EARG;
+  h->cur_set = set;
+  return 0;
+}
+KM_API int h2o4gpu_kmeans_set_iterations(h2o4gpu_kmeans_handle *h, int *iterations) {
+  KM_CHECK_HANDLE(h);
+  if (!iterations || (int)h->set_iterations.size() != h->sets) return H2O4GPU_KMEANS_ESTATE;
+  memcpy(iterations, h->set_iterations.data(), (size_t)h->sets * sizeof(int));
+  return 0;
 }
 KM_API int h2o4gpu_kmeans_destroy(h2o4gpu_kmeans_handle *h) {
   KM_CHECK_HANDLE(h);
@@ -1550,8 +1695,8 @@ KM_API int h2o4gpu_kmeans_parallel_seed_info(h2o4gpu_kmeans_handle *h, int cap, 
 }
 KM_API int h2o4gpu_kmeans_get_seed_rows(h2o4gpu_kmeans_handle *h, int *rows) {
   KM_CHECK_HANDLE(h);
-  if (!rows || (int)h->last_seed_rows.size() != h->k) return H2O4GPU_KMEANS_ESTATE;
-  memcpy(rows, h->last_seed_rows.data(), (size_t)h->k * sizeof(int));
+  if (!rows || (int)h->last_seed_rows.size() != h->kk()) return H2O4GPU_KMEANS_ESTATE;
+  memcpy(rows, h->last_seed_rows.data(), (size_t)h->kk() * sizeof(int));
   return 0;
 }
 KM_API int h2o4gpu_kmeans_fit(h2o4gpu_kmeans_handle *h, int max_iterations, double threshold,

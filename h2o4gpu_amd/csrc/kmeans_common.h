@@ -61,6 +61,18 @@ enum AssignVariant {
 // be padded to: launch_assign / launch_transform may read that far.
 static const int CENTROID_PAD = 256;
 
+// Several independent centroid sets (restarts of one fit) laid end to end as one model:
+// `sets` sets, each padded to kps rows (a multiple of 32; padding rows are zero) of which
+// the first kset are centroids. Labels and minimum distances then hold one [n] block per
+// set, the labels counting from the set's own first centroid; partial sums and counts are
+// those of the whole stacked model. sets <= 1: an ordinary model. Only the row-stationary
+// kernels with the whole model in LDS take a stacked model.
+struct StackShape {
+  int sets = 1;
+  int kps = 0;
+  int kset = 0;
+};
+
 // Fused distance + argmin. labels[i] = argmin_c |(xx_i + cc_c) - 2 x_i.c_c|,
 // strict '<', lowest index wins, -1 when no distance is below FLT_MAX.
 // mindist (nullable) receives the minimum. Returns the variant actually used
@@ -70,7 +82,8 @@ static const int CENTROID_PAD = 256;
 template <typename T>
 int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
                   const T *C, const T *cnorm, int *labels, T *mindist,
-                  int64_t n, int d, int k, int num_cu, int *used, bool exact = false);
+                  int64_t n, int d, int k, int num_cu, int *used, bool exact = false,
+                  StackShape st = StackShape());
 template <typename T>
 int pick_assign_variant(int requested, int64_t n, int d, int k);
 const char *assign_variant_name(int variant);
@@ -88,7 +101,7 @@ template <typename T>
 int launch_assign_accumulate(hipStream_t s, int variant, const T *X, const T *xnorm, const T *C,
                              const T *cnorm, int *labels, T *mindist, int64_t n, int d,
                              int k, int num_cu, double *psums, int *pcounts, int *slots,
-                             int *used);
+                             int *used, StackShape st = StackShape());
 
 // Full squared-distance matrix, centroid-major: D[c * ldn + i], i < n.
 template <typename T>
@@ -133,7 +146,10 @@ int launch_bucketed_accumulate(hipStream_t s, const T *X, const int *labels, int
 
 // Pass 2: fixed-order reduction of the partials, empty clusters keep the old
 // centroid, mean = sum * (1/count), per-block partial of sum((old-new)^2).
-// shift_partials must hold max_shift_partials(d, k) entries.
+// shift_partials must hold max_shift_partials(d, k) entries. frozen (nullable, device,
+// [k / kps] flags): centroids of a set of a stacked model whose flag is set stay as they
+// are; each block of 32 coordinates then lies inside one set (kps is a multiple of 32), so
+// a set's squared shift is the sum of its own partials.
 static const int64_t FINALIZE_NARROW_KD = 4096;
 static inline int max_shift_partials(int d, int k) {
   const int64_t kd = (int64_t)k * d;
@@ -142,7 +158,8 @@ static inline int max_shift_partials(int d, int k) {
 template <typename T>
 int launch_finalize(hipStream_t s, int slots, const double *psums,
                     const int *pcounts, const T *c_old, T *c_new, int *counts,
-                    T *shift_partials, int *n_shift_partials, int d, int k);
+                    T *shift_partials, int *n_shift_partials, int d, int k,
+                    const int *frozen = nullptr, int kps = 1);
 // Pass 3: cnorm of the new centroids and the fixed-order sum of the shift
 // partials into *shift2.
 template <typename T>

@@ -815,7 +815,7 @@ template <typename T, int EPW>
 __global__ __launch_bounds__(WG) void finalize_kernel(
     const double *__restrict__ psums, const int *__restrict__ pcounts, int row_blocks,
     const T *__restrict__ c_old, T *__restrict__ c_new, int *__restrict__ counts,
-    T *__restrict__ shift_partials, int d, int k) {
+    T *__restrict__ shift_partials, int d, int k, const int *__restrict__ frozen, int kps) {
 #pragma clang fp contract(off)
   constexpr int RS = WG / EPW;
   __shared__ double part[RS][EPW];
@@ -863,7 +863,8 @@ __global__ __launch_bounds__(WG) void finalize_kernel(
     }
     const T oldv = c_old[e];
     T newv;
-    if (ctot < 1) {
+    // (frozen: a stacked model's set that has met its convergence test keeps its centroids)
+    if (ctot < 1 || (frozen != nullptr && frozen[c / kps] != 0)) {
       newv = oldv;  // revert_zeroed_centroids, kmeans_centroids.h:77-88
     } else {
       const T scale = (T)1.0 / (T)ctot;  // scale_centroids, kmeans_centroids.h:90-105
@@ -886,16 +887,18 @@ __global__ __launch_bounds__(WG) void finalize_kernel(
 template <typename T>
 int launch_finalize(hipStream_t s, int slots, const double *psums,
                     const int *pcounts, const T *c_old, T *c_new, int *counts,
-                    T *shift_partials, int *n_shift_partials, int d, int k) {
+                    T *shift_partials, int *n_shift_partials, int d, int k, const int *frozen,
+                    int kps) {
   const int64_t kd = (int64_t)k * d;
-  const bool narrow = kd <= FINALIZE_NARROW_KD && slots >= 256;
+  // (a stacked model always takes the wide form: its sets' partials must not share a block)
+  const bool narrow = kd <= FINALIZE_NARROW_KD && slots >= 256 && frozen == nullptr;
   const int blocks = narrow ? (int)((kd + 3) / 4) : (int)((kd + 31) / 32);
   if (narrow)
     hipLaunchKernelGGL((finalize_kernel<T, 4>), dim3(blocks), dim3(WG), 0, s, psums, pcounts,
-                       slots, c_old, c_new, counts, shift_partials, d, k);
+                       slots, c_old, c_new, counts, shift_partials, d, k, frozen, kps);
   else
     hipLaunchKernelGGL((finalize_kernel<T, 32>), dim3(blocks), dim3(WG), 0, s, psums, pcounts,
-                       slots, c_old, c_new, counts, shift_partials, d, k);
+                       slots, c_old, c_new, counts, shift_partials, d, k, frozen, kps);
   KM_HIP_TRY(hipGetLastError());
   *n_shift_partials = blocks;
   return 0;
@@ -1043,7 +1046,7 @@ template int launch_bucketed_accumulate<double>(hipStream_t, const double *, con
   template UpdatePlan plan_update<T>(int64_t, int, int, int);                        \
   template int launch_finalize<T>(hipStream_t, int, const double *,                  \
                                   const int *, const T *, T *, int *, T *, int *,    \
-                                  int, int);                                         \
+                                  int, int, const int *, int);                       \
   template int launch_post_update<T>(hipStream_t, const T *, T *, const T *, int,    \
                                      T *, int, int);                                 \
   template int launch_sum<T>(hipStream_t, const T *, int64_t, double *, int,         \

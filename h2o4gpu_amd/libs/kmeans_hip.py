@@ -44,6 +44,11 @@ PROTOTYPES = {
     "h2o4gpu_kmeans_random_start_rows": (c_int, [c_int, c_size_t, c_int, c_void_p]),
     "h2o4gpu_kmeans_create": (c_int, [P(c_void_p), c_int, c_size_t, c_size_t, c_int, c_int, c_int]),
     "h2o4gpu_kmeans_destroy": (c_int, [c_void_p]),
+    "h2o4gpu_kmeans_stack_width": (c_int, [c_int, c_size_t, c_size_t, c_int, c_int]),
+    "h2o4gpu_kmeans_create_stacked": (c_int, [P(c_void_p), c_int, c_size_t, c_size_t, c_int, c_int, c_int,
+                                              c_int]),
+    "h2o4gpu_kmeans_select_set": (c_int, [c_void_p, c_int]),
+    "h2o4gpu_kmeans_set_iterations": (c_int, [c_void_p, c_void_p]),
     "h2o4gpu_kmeans_set_data_host": (c_int, [c_void_p, c_void_p]),
     "h2o4gpu_kmeans_set_data_device": (c_int, [c_void_p, c_void_p]),
     "h2o4gpu_kmeans_set_centroids_host": (c_int, [c_void_p, c_void_p]),
@@ -128,21 +133,42 @@ def _vp(a):
     return a.ctypes.data_as(c_void_p)
 
 
+def stack_width(rows, cols, k, dtype, max_sets):
+    """How many restarts of a k-cluster fit one stacked handle can run at once for this shape."""
+    return int(lib().h2o4gpu_kmeans_stack_width(np.dtype(dtype).itemsize, int(rows), int(cols), int(k),
+                                                int(max_sets)))
+
+
 ASSIGN_VARIANTS = {"auto": 0, "valu": 1, "mfma_rowstat": 2, "mfma_tiled": 3}
 
 
 class Handle:
     """Resident data set + model working set on one GPU (part 3 of the C ABI)."""
 
-    def __init__(self, rows, cols, k, dtype=np.float32, gpu_id=0, verbose=0):
+    def __init__(self, rows, cols, k, dtype=np.float32, gpu_id=0, verbose=0, sets=1):
+        """sets > 1: a stacked handle holding that many independent centroid sets (restarts)
+        over the same rows; see stack_width() for how many a shape allows."""
         self.dtype = np.dtype(dtype)
         if self.dtype not in (np.dtype(np.float32), np.dtype(np.float64)):
             raise TypeError("float32 or float64 only")
         self.rows, self.cols, self.k = int(rows), int(cols), int(k)
+        self.sets = int(sets)
         self._h = c_void_p()
         self._keep = None
-        _check("create", lib().h2o4gpu_kmeans_create(ctypes.byref(self._h), self.dtype.itemsize,
-                                                     self.rows, self.cols, self.k, gpu_id, verbose))
+        _check("create", lib().h2o4gpu_kmeans_create_stacked(ctypes.byref(self._h), self.dtype.itemsize,
+                                                             self.rows, self.cols, self.k, self.sets,
+                                                             gpu_id, verbose))
+
+    def select_set(self, s):
+        """Stacked handle: the set that set_centroids, init_*, centroids, labels, counts,
+        min_distances, seed_rows and inertia address."""
+        _check("select_set", lib().h2o4gpu_kmeans_select_set(self._h, int(s)))
+
+    def set_iterations(self):
+        """Stacked handle: centroid updates each set made in the last fit."""
+        out = np.empty(self.sets, np.int32)
+        _check("set_iterations", lib().h2o4gpu_kmeans_set_iterations(self._h, _vp(out)))
+        return out
 
     def close(self):
         if self._h:

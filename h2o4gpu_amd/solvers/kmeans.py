@@ -179,14 +179,66 @@ class KMeansH2O:
         self._did_sklearn_fit = 0
         return self
 
-    def _device_handle(self, dev, k):
+    def _device_handle(self, dev, k, sets=1):
         """A handle that adopts the device rows (no copy)."""
         if self._load_lib() is None:
             raise RuntimeError("device input needs a usable GPU")
         from ..libs import kmeans_hip
-        h = kmeans_hip.Handle(dev.rows, dev.cols, k, dev.dtype, gpu_id=self._gpu_id, verbose=self.verbose)
+        h = kmeans_hip.Handle(dev.rows, dev.cols, k, dev.dtype, gpu_id=self._gpu_id, verbose=self.verbose,
+                              sets=sets)
         h.set_data_device(dev.ptr, keepalive=dev.owner)
         return h
+
+    def _seed_handle(self, h, start, seed):
+        """Initial centroids of the handle's selected set."""
+        if start is not None:
+            h.set_centroids(start)
+        elif self.init in ("k-means++", "k-means||"):
+            h.init_parallel(seed)
+        elif self.init == "d2-sampling":
+            h.init_plusplus(seed)
+        else:
+            h.init_random_rows(seed)
+
+    def _fit_on_handle(self, make_handle, rows, cols, dtype, k, start):
+        """Runs the restarts (seeds random_state, random_state + 1, ...) on rows that stay on
+        the device, keeps the one with the lowest inertia, and sets the fitted attributes.
+        As many restarts as the shape allows run stacked: their centroid sets form one model,
+        one kernel labels every row against all of them and sums the rows per set, so every
+        iteration reads the rows once for the whole group (the reference documents n_init > 1
+        as unsupported, kmeans.py:722-725). make_handle(sets) returns a handle that holds
+        the rows."""
+        from ..libs import kmeans_hip
+        restarts = 1 if start is not None else max(1, int(self.n_init or 1))
+        width = kmeans_hip.stack_width(rows, cols, k, dtype, restarts) if restarts > 1 else 1
+        groups = -(-restarts // width)
+        sets = -(-restarts // groups)  # balanced groups; a spare set repeats the group's first start
+        best = None
+        with make_handle(sets) as h:
+            for g in range(groups):
+                members = [g * sets + s for s in range(sets)]
+                for s, r in enumerate(members):
+                    if sets > 1:
+                        h.select_set(s)
+                    self._seed_handle(h, start, self.random_state + (r if r < restarts else members[0]))
+                n_iter = h.fit(self._max_iter, self.tol)
+                iters = h.set_iterations() if sets > 1 else [n_iter]
+                for s, r in enumerate(members):
+                    if r >= restarts:
+                        continue
+                    if sets > 1:
+                        h.select_set(s)
+                    inertia = h.inertia() if self._max_iter > 0 else None
+                    if best is None or (inertia is not None and inertia < best[2]):
+                        best = (h.centroids(), h.labels(), inertia, int(iters[s]))
+        centers, self.labels_, self.inertia_, self.n_iter_ = best
+        if k < self._n_clusters:
+            # more clusters asked for than rows: the fit ran with k = rows (kmeans_h2o4gpu.cu:630-635);
+            # the result keeps n_clusters rows, the rest zero, exactly as the host-pointer entry point
+            # leaves its preallocated array, so predict / transform see one shape whichever path fitted
+            centers = np.concatenate([centers, np.zeros((self._n_clusters - k, cols), centers.dtype)])
+        self.cluster_centers_ = centers
+        return self.cluster_centers_, self.labels_
 
     def _fit_device(self, dev):
         """fit on rows resident in device memory, through the handle entry points: same
@@ -198,30 +250,8 @@ class KMeansH2O:
             assert self.init.shape == (self._n_clusters, dev.cols), \
                 "init must have shape (n_clusters, n_features)"
             start = np.ascontiguousarray(self.init[:k], dtype=dev.dtype)
-        restarts = 1 if start is not None else max(1, int(self.n_init or 1))
-        best = None
-        with self._device_handle(dev, k) as h:
-            for r in range(restarts):
-                if start is not None:
-                    h.set_centroids(start)
-                elif self.init in ("k-means++", "k-means||"):
-                    h.init_parallel(self.random_state + r)
-                elif self.init == "d2-sampling":
-                    h.init_plusplus(self.random_state + r)
-                else:
-                    h.init_random_rows(self.random_state + r)
-                n_iter = h.fit(self._max_iter, self.tol)
-                inertia = h.inertia() if self._max_iter > 0 else None
-                if best is None or (inertia is not None and inertia < best[2]):
-                    best = (h.centroids(), h.labels(), inertia, n_iter)
-        centers, self.labels_, self.inertia_, self.n_iter_ = best
-        if k < self._n_clusters:
-            # more clusters asked for than rows: the fit ran with k = rows (kmeans_h2o4gpu.cu:630-635);
-            # the result keeps n_clusters rows, the rest zero, exactly as the host path leaves its
-            # preallocated array, so predict / transform see one shape whichever path fitted
-            centers = np.concatenate([centers, np.zeros((self._n_clusters - k, dev.cols), centers.dtype)])
-        self.cluster_centers_ = centers
-        return self.cluster_centers_, self.labels_
+        return self._fit_on_handle(lambda sets: self._device_handle(dev, k, sets), dev.rows, dev.cols,
+                                   dev.dtype, k, start)
 
     def sklearn_fit(self, X, y=None):
         assert self.cluster_centers_ is not None, "Centroids are None. Run fit() first."
@@ -339,6 +369,19 @@ class KMeansH2O:
         # n_init restarts (seed, seed+1, ...) keep the lowest inertia; the reference runs one
         # (kmeans.py:722-725). Restarts are pointless when the start is given.
         restarts = 1 if c_init == 2 else max(1, int(self.n_init or 1))
+        if restarts > 1:
+            # the rows go to the device once and stay there for all restarts
+            from ..libs import kmeans_hip
+            k = min(self._n_clusters, rows)
+            dtype = np.float64 if self.double_precision else np.float32
+            host = np.ascontiguousarray(np.reshape(c_data, (rows, cols)), dtype=dtype)
+
+            def make_handle(sets):
+                h = kmeans_hip.Handle(rows, cols, k, dtype, gpu_id=self._gpu_id, verbose=self.verbose,
+                                      sets=sets)
+                h.set_data(host)
+                return h
+            return self._fit_on_handle(make_handle, rows, cols, dtype, k, None)
         best = None
         owned = getattr(lib, "kmeans_fit_owned", None)
         for r in range(restarts):

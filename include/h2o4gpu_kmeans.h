@@ -145,6 +145,25 @@ int h2o4gpu_kmeans_create(h2o4gpu_kmeans_handle **out, int elem_size,
                           int verbose);
 int h2o4gpu_kmeans_destroy(h2o4gpu_kmeans_handle *h);
 
+/* Stacked restarts (the reference documents n_init > 1 as unsupported,
+ * src/interface_py/h2o4gpu/solvers/kmeans.py:722-725): a handle holding `sets` independent
+ * centroid sets of k centroids each over the same rows. One kernel labels every row against
+ * all sets (the sets lie end to end as one model, the argmin taken per set) and sums the
+ * rows per set, so the rows are read once per iteration for all restarts.
+ * stack_width: the largest number of sets (<= max_sets) such a handle can hold for this
+ * shape, 1 when the shape does not stack (restarts then run one after another on an
+ * ordinary handle). create_stacked with sets < 2 is create.
+ * On a stacked handle select_set picks the set addressed by set_centroids_host, init_*,
+ * get_centroids / labels / counts / min_distances / seed_rows and inertia; fit, iterate and
+ * assign work on all sets. With a threshold every set stops at its own iteration (its
+ * centroids then stay as they are); set_iterations returns the [sets] update counts of the
+ * last fit. update, set_labels_host, predict_host and transform_* are not offered. */
+int h2o4gpu_kmeans_stack_width(int elem_size, size_t rows, size_t cols, int k, int max_sets);
+int h2o4gpu_kmeans_create_stacked(h2o4gpu_kmeans_handle **out, int elem_size, size_t rows,
+                                  size_t cols, int k, int sets, int gpu_id, int verbose);
+int h2o4gpu_kmeans_select_set(h2o4gpu_kmeans_handle *h, int set);
+int h2o4gpu_kmeans_set_iterations(h2o4gpu_kmeans_handle *h, int *iterations);
+
 /* Upload rows from host memory (copies) / adopt a device pointer (no copy,
  * caller keeps it alive). Row norms are computed on the device either way. */
 int h2o4gpu_kmeans_set_data_host(h2o4gpu_kmeans_handle *h, const void *X);

@@ -1,0 +1,129 @@
+"""Stacked restarts: several centroid sets of one fit as one model through the fused
+row-stationary kernel, per-set argmin and per-set sums, against the same restarts run one
+after another on ordinary handles (through the C ABI)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def blobs(n, d, k, dtype, seed):
+    rng = np.random.default_rng(seed)
+    centres = rng.uniform(-8, 8, size=(k, d))
+    return np.ascontiguousarray((centres[rng.integers(0, k, size=n)] +
+                                 1.5 * rng.standard_normal((n, d))).astype(dtype))
+
+
+def serial_fit(hip, X, k, C0, iters, tol):
+    n, d = X.shape
+    with hip.Handle(n, d, k, X.dtype) as h:
+        h.set_data(X)
+        h.set_option("assign", "mfma_rowstat")  # the kernel family a stacked handle runs
+        h.set_centroids(C0)
+        it = h.fit(iters, tol)
+        return h.centroids(), h.labels(), h.counts(), h.inertia(), it
+
+
+SHAPES = [(50000, 32, 20, 3), (40000, 64, 64, 2), (60000, 16, 8, 4), (30000, 24, 33, 2), (20000, 8, 5, 6)]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n,d,k,sets", SHAPES)
+def test_stacked_sets_equal_serial_restarts(hip, n, d, k, sets, dtype):
+    X = blobs(n, d, k, dtype, seed=n + d)
+    if hip.stack_width(n, d, k, dtype, sets) < sets:
+        pytest.skip("shape does not hold %d sets" % sets)
+    rng = np.random.default_rng(7)
+    starts = [np.ascontiguousarray(X[rng.choice(n, size=k, replace=False)]) for _ in range(sets)]
+    iters = 7
+    with hip.Handle(n, d, k, dtype, sets=sets) as h:
+        h.set_data(X)
+        for s in range(sets):
+            h.select_set(s)
+            h.set_centroids(starts[s])
+        assert h.fit(iters, 0.0) == iters
+        got = []
+        for s in range(sets):
+            h.select_set(s)
+            got.append((h.centroids(), h.labels(), h.counts(), h.inertia()))
+        assert h.set_iterations().tolist() == [iters] * sets
+    for s in range(sets):
+        C, L, cnt, inertia, _ = serial_fit(hip, X, k, starts[s], iters, 0.0)
+        gC, gL, gcnt, ginertia = got[s]
+        assert np.array_equal(gL, L), "set %d: %d labels differ" % (s, int((gL != L).sum()))
+        assert np.array_equal(gcnt, cnt)
+        if dtype == np.float32:
+            # float32 rows add up exactly in the double-precision sums: bit for bit
+            assert np.array_equal(gC, C)
+            assert ginertia == inertia
+        else:
+            assert np.allclose(gC, C, rtol=1e-12, atol=1e-12)
+            assert abs(ginertia - inertia) <= 1e-12 * inertia
+
+
+def test_every_set_stops_at_its_own_iteration(hip):
+    """With a threshold a set stops after the update whose squared shift is below it and keeps
+    its centroids while the others go on (kmeans_impl.h:189-232, per set)."""
+    n, d, k, sets = 40000, 32, 12, 3
+    X = blobs(n, d, k, np.float32, seed=3)
+    rng = np.random.default_rng(11)
+    # one start at the true optimum's doorstep (converges at once), two poor ones
+    good = serial_fit(hip, X, k, np.ascontiguousarray(X[rng.choice(n, size=k, replace=False)]), 40, 0.0)[0]
+    starts = [good, np.ascontiguousarray(X[:k]), np.ascontiguousarray(X[rng.choice(n, size=k, replace=False)])]
+    tol = 1e-3
+    want = [serial_fit(hip, X, k, c0, 60, tol) for c0 in starts]
+    with hip.Handle(n, d, k, np.float32, sets=sets) as h:
+        h.set_data(X)
+        for s in range(sets):
+            h.select_set(s)
+            h.set_centroids(starts[s])
+        h.fit(60, tol)
+        its = h.set_iterations().tolist()
+        assert its == [w[4] for w in want], (its, [w[4] for w in want])
+        assert len(set(its)) > 1, "the starts were meant to converge at different iterations"
+        for s in range(sets):
+            h.select_set(s)
+            assert np.array_equal(h.centroids(), want[s][0])
+            assert np.array_equal(h.labels(), want[s][1])
+            assert h.inertia() == want[s][3]
+
+
+def test_per_set_seeding_and_limits(hip):
+    n, d, k = 20000, 16, 10
+    X = blobs(n, d, k, np.float32, seed=5)
+    width = hip.stack_width(n, d, k, np.float32, 4096)  # as many as one CU's LDS holds
+    assert 2 <= width < 4096
+    assert hip.stack_width(500000, 784, 4096, np.float32, 4) == 1   # far beyond one CU's LDS
+    with pytest.raises(hip.KMeansHipError):
+        hip.Handle(n, d, k, np.float32, sets=width + 1)
+    with hip.Handle(n, d, k, np.float32) as single, hip.Handle(n, d, k, np.float32, sets=2) as h:
+        single.set_data(X)
+        h.set_data(X)
+        for s, (init, seed) in enumerate([("init_random_rows", 4), ("init_parallel", 9)]):
+            getattr(single, init)(seed)
+            h.select_set(s)
+            getattr(h, init)(seed)
+            assert np.array_equal(h.seed_rows(), single.seed_rows())
+            assert np.array_equal(h.centroids(), single.centroids())
+        h.select_set(0)
+        h.init_plusplus(3)
+        single.init_plusplus(3)
+        assert np.array_equal(h.centroids(), single.centroids())
+        with pytest.raises(hip.KMeansHipError):
+            h.predict(X[:10])
+        with pytest.raises(hip.KMeansHipError):
+            h.select_set(2)
+
+
+def test_estimator_restarts_keep_the_best(hip):
+    import h2o4gpu_amd
+    n, d, k = 30000, 32, 16
+    X = blobs(n, d, k, np.float32, seed=8)
+    data = X
+    best = h2o4gpu_amd.KMeans(n_clusters=k, init="random", n_init=5, max_iter=15, tol=0, random_state=20).fit(data)
+    singles = [h2o4gpu_amd.KMeans(n_clusters=k, init="random", n_init=1, max_iter=15, tol=0,
+                                  random_state=20 + r).fit(data) for r in range(5)]
+    inertias = [m.inertia_ for m in singles]
+    assert abs(best.inertia_ - min(inertias)) <= 1e-6 * min(inertias)
+    assert best.cluster_centers_.shape == (k, d) and best.labels_.shape == (n,)
+    assert best.n_iter_ == 15

@@ -24,7 +24,7 @@ def test_device_tensors_give_the_results_of_host_arrays(hip):
     r = json.loads(proc.stdout.strip().splitlines()[-1])
     for tag in ("float32", "float64"):
         for key in ("labels_equal", "predict_equal", "transform_is_tensor", "random_close",
-                    "k-means++_close"):
+                    "k-means++_close", "restarts_close"):
             assert r["%s_%s" % (tag, key)] is True, (tag, key, r)
         # float32 sums are exact in double and repeat bit for bit; float64 sums depend on
         # the arrival order of the LDS adds and repeat to rounding only

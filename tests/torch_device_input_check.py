@@ -44,6 +44,12 @@ def main():
             b = KMeans(n_clusters=k, init=init, max_iter=3, tol=0.0, random_state=11).fit(Xd)
             out["%s_%s_close" % (tag, init)] = bool(np.allclose(a.cluster_centers_, b.cluster_centers_,
                                                                 rtol=1e-12, atol=1e-12))
+        # restarts (stacked where the shape allows) on device rows and on host rows agree
+        a = KMeans(n_clusters=k, init="random", n_init=3, max_iter=3, tol=0.0, random_state=5).fit(X)
+        b = KMeans(n_clusters=k, init="random", n_init=3, max_iter=3, tol=0.0, random_state=5).fit(Xd)
+        out[tag + "_restarts_close"] = bool(np.allclose(a.cluster_centers_, b.cluster_centers_, rtol=1e-12,
+                                                       atol=1e-12) and
+                                           abs(a.inertia_ - b.inertia_) <= 1e-12 * a.inertia_)
     # device rows that start 4 or 8 bytes into an allocation (not 16-byte aligned): every
     # kernel family must take its unaligned path and give the aligned result
     unaligned = {}
