@@ -225,7 +225,9 @@ def test_estimator_restarts_and_score(oracle):
         singles.append(m.inertia_)
     multi = KMeans(n_clusters=8, init="random", n_init=4, max_iter=30, tol=1e-6, random_state=40)
     multi.fit(Xb)
-    assert multi.inertia_ == min(singles)
+    # (the restarts run stacked through the matrix-core kernel, the single fits of this small
+    # shape through the scalar-order one: same optimum, minimum distances equal to rounding)
+    assert abs(multi.inertia_ - min(singles)) <= 1e-5 * min(singles)
     want = ((Xb.astype(np.float64) - multi.cluster_centers_.astype(np.float64)[multi.labels_]) ** 2).sum()
     assert abs(multi.inertia_ - want) <= 1e-5 * want
     Xn, _ = blobs(1500, 6, 8, np.float32, 22)
