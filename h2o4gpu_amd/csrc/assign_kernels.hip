@@ -158,10 +158,13 @@ template <typename T, int DREG, bool SUMS>
 __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
     const T *__restrict__ X, const T *__restrict__ xnorm, const T *__restrict__ C,
     const T *__restrict__ cnorm, int *__restrict__ labels, T *__restrict__ mindist,
-    double *__restrict__ psums, int *__restrict__ pcounts, int64_t n, int k) {
+    double *__restrict__ psums, int *__restrict__ pcounts, int64_t n, int k,
+    T *__restrict__ D, int64_t ldn) {
 #pragma clang fp contract(off)
   extern __shared__ __align__(16) unsigned char smem_raw[];
   constexpr int d = DREG;
+  // D (assignment-only form): write every distance to D[c * ldn + row] instead of labels
+  const bool full = !SUMS && D != nullptr;
   constexpr int VEC = Mfma<T>::VW;
   const int sx = staged_row_stride(d);                           // row stride of the staged block
   // SUMS false: assignment only (predict, final relabel, inertia): no sums, no counts
@@ -236,13 +239,16 @@ __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
         for (int j = 0; j < DREG; j++) dot = dot + xr[j] * cp[j];
         const T t = xx + ccs[c];
         const T dist = fabs(t - (T)2 * dot);
+        if (full) D[(size_t)c * ldn + row] = dist;
         if (dist < best) {
           best = dist;
           bidx = c;
         }
       }
-      labels[row] = bidx;
-      if (mindist) mindist[row] = best;
+      if (!full) {
+        labels[row] = bidx;
+        if (mindist) mindist[row] = best;
+      }
       if (SUMS && bidx >= 0) {
         // Lane l starts at feature l mod d: with only a handful of centroids the
         // lanes of a wavefront would otherwise all add to the same few addresses
@@ -288,9 +294,11 @@ template <typename T, int DMAX, int VEC, int KREG, bool SUMS>
 __global__ __launch_bounds__(WG) void lloyd_valu_anyd_kernel(
     const T *__restrict__ X, const T *__restrict__ xnorm, const T *__restrict__ C,
     const T *__restrict__ cnorm, int *__restrict__ labels, T *__restrict__ mindist,
-    double *__restrict__ psums, int *__restrict__ pcounts, int64_t n, int d, int k) {
+    double *__restrict__ psums, int *__restrict__ pcounts, int64_t n, int d, int k,
+    T *__restrict__ D, int64_t ldn) {
 #pragma clang fp contract(off)
   extern __shared__ __align__(16) unsigned char smem_raw[];
+  const bool full = !SUMS && D != nullptr;  // as in lloyd_valu_fused_kernel
   const int sx = staged_row_stride(d);
   const int pad = sx - d;                                        // 0 or 1
   double *sums = reinterpret_cast<double *>(smem_raw);           // [k][sx]; SUMS false: none
@@ -424,14 +432,17 @@ __global__ __launch_bounds__(WG) void lloyd_valu_anyd_kernel(
         if (c < k) {
           const T t = xx + ccs[c];
           const T dist = fabs(t - (T)2 * dot[c]);
+          if (full) D[(size_t)c * ldn + row] = dist;
           if (dist < best) {
             best = dist;
             bidx = c;
           }
         }
       }
-      labels[row] = bidx;
-      if (mindist) mindist[row] = best;
+      if (!full) {
+        labels[row] = bidx;
+        if (mindist) mindist[row] = best;
+      }
       if (SUMS && bidx >= 0) {
         double *srow = sums + (size_t)bidx * sx;
         int jj = jrot;  // rotated start, as in lloyd_valu_fused_kernel
@@ -1386,7 +1397,8 @@ int fused_slots(int requested_variant, int64_t n, int d, int k, int num_cu) {
 template <typename T, bool SUMS>
 static int launch_valu_fused(hipStream_t s, const T *X, const T *xnorm, const T *C,
                              const T *cnorm, int *labels, T *mindist, int64_t n, int d, int k,
-                             int num_cu, double *psums, int *pcounts, int *slots) {
+                             int num_cu, double *psums, int *pcounts, int *slots, T *D = nullptr,
+                             int64_t ldn = 0) {
   const size_t lds = valu_fused_lds<T>(d, k, SUMS);
   const int grid = valu_fused_grid(n, lds, num_cu);
   if (slots) *slots = grid;
@@ -1399,7 +1411,7 @@ static int launch_valu_fused(hipStream_t s, const T *X, const T *xnorm, const T 
     auto kern = lloyd_valu_fused_kernel<T, DREG, SUMS>;                                    \
     KM_VF_SETUP(kern);                                                                     \
     hipLaunchKernelGGL(kern, dim3(grid), dim3(WG), lds, s, X, xnorm, C, cnorm, labels,     \
-                       mindist, psums, pcounts, n, k);                                     \
+                       mindist, psums, pcounts, n, k, D, ldn);                             \
   } while (0)
   // any other d: dot products in registers, KREG >= k of them
 #define KM_VA_LAUNCH(DMAX, VEC, KREG)                                                      \
@@ -1407,7 +1419,7 @@ static int launch_valu_fused(hipStream_t s, const T *X, const T *xnorm, const T 
     auto kern = lloyd_valu_anyd_kernel<T, DMAX, VEC, KREG, SUMS>;                          \
     KM_VF_SETUP(kern);                                                                     \
     hipLaunchKernelGGL(kern, dim3(grid), dim3(WG), lds, s, X, xnorm, C, cnorm, labels,     \
-                       mindist, psums, pcounts, n, d, k);                                  \
+                       mindist, psums, pcounts, n, d, k, D, ldn);                          \
   } while (0)
 #define KM_VA_K(DMAX, VEC)                       \
   do {                                           \
@@ -1554,11 +1566,17 @@ template <typename T>
 int launch_transform(hipStream_t s, const T *X, const T *xnorm, const T *C,
                      const T *cnorm, T *D, int64_t n, int64_t ldn, int d, int k,
                      int num_cu) {
-  (void)num_cu;
   if (n <= 0) return 0;
   if (d < 1 || k < 1) return H2O4GPU_KMEANS_EARG;
-  if (k <= 16 && d <= 64)
+  if (k <= 16 && d <= 64) {
+    // the staged kernels of the small-shape Lloyd step (coalesced 16-byte loads of the rows,
+    // scalar-order arithmetic) with every distance stored; rows of a few values keep the
+    // one-thread-per-row kernel, as in launch_assign
+    if (valu_fused_applies(d, k) && (d >= 8 || d * sizeof(T) == 32))
+      return launch_valu_fused<T, false>(s, X, xnorm, C, cnorm, nullptr, nullptr, n, d, k, num_cu,
+                                         nullptr, nullptr, nullptr, D, ldn);
     return launch_valu<T, 1>(s, X, xnorm, C, cnorm, nullptr, nullptr, D, n, ldn, d, k);
+  }
   return launch_tiled<T, 1>(s, X, xnorm, C, cnorm, nullptr, nullptr, D, n, ldn, d, k);
 }
 

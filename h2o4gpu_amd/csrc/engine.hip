@@ -180,6 +180,7 @@ struct h2o4gpu_kmeans_handle {
   int opt_fuse = 1;  // 1: use the fused assign+accumulate kernel where the shape allows
   int opt_buckets = 1;  // 1: bucketed centroid sums where the sums do not fit LDS
   int opt_exact = 0;    // 1: float32 MFMA argmin on the float distances, not on 16-ulp keys
+  int opt_transform_batch_mb = 4096;  // device buffer of transform_host's output, per batch of rows
   int last_variant = ASSIGN_AUTO;
 
   // profiling
@@ -1257,7 +1258,7 @@ struct Engine : h2o4gpu_kmeans_handle {
     KM_HIP_TRY(hipSetDevice(dev));
     if (!have_centroids || sets > 1) return H2O4GPU_KMEANS_ESTATE;
     if (rows == 0) return 0;
-    size_t batch = ((size_t)4 << 30) / ((size_t)k * sizeof(T));
+    size_t batch = ((size_t)opt_transform_batch_mb << 20) / ((size_t)k * sizeof(T));
     batch = batch / 128 * 128;
     if (batch < 128) batch = 128;
     if (batch > rows) batch = rows;
@@ -1833,6 +1834,11 @@ KM_API int h2o4gpu_kmeans_set_option(h2o4gpu_kmeans_handle *h, const char *name,
   if (strcmp(name, "exact_argmin") == 0) {
     if (value != 0 && value != 1) return H2O4GPU_KMEANS_EARG;
     h->opt_exact = value;
+    return 0;
+  }
+  if (strcmp(name, "transform_batch_mb") == 0) {
+    if (value < 1 || value > 65536) return H2O4GPU_KMEANS_EARG;
+    h->opt_transform_batch_mb = value;
     return 0;
   }
   if (strcmp(name, "fuse") == 0) {

@@ -232,6 +232,8 @@ int h2o4gpu_kmeans_transform_resident(h2o4gpu_kmeans_handle *h, void *d_dist);
  * fit LDS by bucketing rows by label, 0 uses the chunked LDS kernel for them too;
  * "exact_argmin" = 1 makes the float32 matrix-core kernels compare the float distances
  * themselves instead of 16-ulp integer keys (slower, never fused; 0 is the default).
+ * "transform_batch_mb" (default 4096) bounds the device buffer transform_host fills per
+ * batch of rows; smaller values force more, shorter batches.
  * Unknown names return EARG. */
 int h2o4gpu_kmeans_set_option(h2o4gpu_kmeans_handle *h, const char *name,
                               int value);

@@ -131,6 +131,30 @@ def test_predict_and_transform_entry_points(shim, oracle, dtype):
     assert rc == 0 and (res2 == res).mean() > 0.999
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_transform_in_several_batches(hip, dtype):
+    """transform_host fills its [k][rows] host result batch by batch (strided copies, a
+    ragged last batch that is not a multiple of the row tile) when the output exceeds its
+    device buffer: the result must be the single-batch one and the float64 brute force."""
+    n, d, k = 33333, 40, 300
+    rng = np.random.default_rng(12)
+    X = rng.standard_normal((n, d)).astype(dtype)
+    C = rng.standard_normal((k, d)).astype(dtype)
+    with hip.Handle(k, d, k, dtype) as h:
+        h.set_centroids(C)
+        whole = h.transform(X)
+        # 1 MB per batch: 33333 rows x 300 distances go out in 38 (float32) / 77 batches
+        h.set_option("transform_batch_mb", 1)
+        parts = h.transform(X)
+        assert parts.shape == (k, n) and np.array_equal(parts, whole)
+        h.set_option("transform_batch_mb", 16)  # three batches, the last one ragged
+        assert np.array_equal(h.transform(X), whole)
+    rows = rng.choice(n, size=200, replace=False)
+    want = ((X[rows][:, None, :].astype(np.float64) - C[None].astype(np.float64)) ** 2).sum(-1).T
+    scale = 2 * (X.astype(np.float64) ** 2).sum(1).max()
+    assert np.max(np.abs(whole[:, rows].astype(np.float64) - want)) <= 64 * np.finfo(dtype).eps * scale
+
+
 def test_bad_arguments_return_codes(shim):
     X = np.zeros((10, 2), np.float32)
     pc, pl = np.zeros(4, np.float32), np.zeros(10, np.int32)
