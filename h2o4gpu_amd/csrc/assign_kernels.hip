@@ -908,7 +908,15 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
   const int wr = wave / BCW;  // which half of the row block
   const int r = lane % MT;
   const int g = lane / MT;
-  const int64_t row0 = (int64_t)blockIdx.x * BR;
+  // MODE 0: one workgroup per row block. MODE 1: one per (row block, centroid block) pair
+  // on a linear grid with the centroid block running fastest: workgroups that are resident
+  // together then share a handful of row blocks (which stay in L2) instead of all reading
+  // different ones (500k x 784, k = 4096, 100,000 rows: 5.94 -> 5.64 ms against the row
+  // block running fastest; L2-sized patches of both measured the same as this order).
+  const int ncb = MODE == 1 ? (k + BC - 1) / BC : 1;
+  const int64_t rt_id = MODE == 1 ? (int64_t)blockIdx.x / ncb : (int64_t)blockIdx.x;
+  const int cb_id = MODE == 1 ? (int)((int64_t)blockIdx.x - rt_id * ncb) : 0;
+  const int64_t row0 = rt_id * BR;
   const int nstage = (d + BK - 1) / BK;
   // steps of the last stage that hold features: its ceil(rest / VW) vectors, KL per step
   const int nq_tail = ((d - (nstage - 1) * BK + VW - 1) / VW + KL - 1) / KL;
@@ -1004,10 +1012,10 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
       *reinterpret_cast<vec_t *>(Bs + buf * B_ELEMS + lds_off[q]) = breg[q];
   };
 
-  // MODE 1 has no dependency between centroid blocks: each workgroup takes the single
-  // block blockIdx.y, which keeps a short batch of rows (a transform of 100,000 rows is
+  // MODE 1 has no dependency between centroid blocks: each workgroup takes a single
+  // block, which keeps a short batch of rows (a transform of 100,000 rows is
   // 782 row tiles on 512 workgroup slots) from ending in a half-empty last round.
-  const int c_begin = MODE == 1 ? (int)blockIdx.y * BC : 0;
+  const int c_begin = MODE == 1 ? cb_id * BC : 0;
   const int c_end = MODE == 1 ? min(k, c_begin + BC) : k;
   for (int c0 = c_begin; c0 < c_end; c0 += BC) {
     acc_t acc[CT][RT];
@@ -1474,8 +1482,10 @@ static int launch_tiled_bcw(hipStream_t s, const T *X, const T *xnorm, const T *
                             int64_t ldn, int d, int k, bool exact) {
   typedef TiledCfg<T, BCW> Cfg;
   const size_t lds = (size_t)2 * (Cfg::BC + Cfg::BR) * Cfg::BK * sizeof(T);
-  const dim3 grid((unsigned)((n + Cfg::BR - 1) / Cfg::BR),
-                  MODE == 1 ? (unsigned)((k + Cfg::BC - 1) / Cfg::BC) : 1u);
+  const int64_t row_tiles = (n + Cfg::BR - 1) / Cfg::BR;
+  const int64_t tiles = MODE == 1 ? row_tiles * ((k + Cfg::BC - 1) / Cfg::BC) : row_tiles;
+  if (tiles > 2147483647ll) return H2O4GPU_KMEANS_EARG;
+  const dim3 grid((unsigned)tiles, 1u);
   const bool vec = d >= Mfma<T>::VW;  // 16-byte loads need element alignment only
   const bool tail = (d % Cfg::BK) != 0;
 #define KM_TILED_X(VEC, TAIL, EXACT)                                                         \
