@@ -857,10 +857,13 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
 // workgroup and come from HBM/MALL every time they are re-read, centroid blocks
 // are shared by all workgroups and hit L2, so for large k the wider centroid
 // block (BCW = 4) halves the expensive traffic.
-template <typename T, int BCW>
+template <typename T, int BCW, bool WIDE = false>
 struct TiledCfg {
   static constexpr int TPB = 2 * BCW * 64;
-  static constexpr int BC = 64 * BCW;
+  // WIDE: every wavefront holds twice as many centroid tiles (a 256-centroid block for four
+  // wavefronts) at half the stage depth: the same matrix work per stage and barrier, half as
+  // many passes over the workgroup's row slice.
+  static constexpr int BC = 64 * BCW * (WIDE ? 2 : 1);
   // 128 rows for both precisions: with 64 rows the double kernel issued only 32 MFMAs per
   // staged tile pair and its staging instructions weighed twice as much (2M x 256, k = 1024
   // double: 0.75 -> 0.81 of peak with 128 rows, a few spilled registers included)
@@ -868,17 +871,17 @@ struct TiledCfg {
   // features per stage. The 64-centroid form serves bandwidth-bound shapes (k <= 64): half
   // the stage depth halves its LDS image, so twice as many workgroups keep loads in flight
   // (500k x 784, k = 10: 0.62 -> 0.49 ms; a quarter of the depth was slower again).
-  static constexpr int BK = (sizeof(T) == 4 ? 32 : 16) / (BCW == 1 ? 2 : 1);
+  static constexpr int BK = (sizeof(T) == 4 ? 32 : 16) / (BCW == 1 || WIDE ? 2 : 1);
 };
 
-template <typename T, int MODE, bool VECLOAD, bool DTAIL, int BCW, bool EXACT = false>
+template <typename T, int MODE, bool VECLOAD, bool DTAIL, int BCW, bool EXACT = false, bool WIDE = false>
 __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_kernel(
     const T *__restrict__ X, const T *__restrict__ xnorm,
     const T *__restrict__ C, const T *__restrict__ cnorm,
     int *__restrict__ labels, T *__restrict__ mindist, T *__restrict__ D,
     int64_t n, int64_t ldn, int d, int k) {
   typedef Mfma<T> M;
-  typedef TiledCfg<T, BCW> Cfg;
+  typedef TiledCfg<T, BCW, WIDE> Cfg;
   constexpr int MT = M::MT, KL = M::KL, NACC = M::NACC, VW = M::VW;
   constexpr int BC = Cfg::BC, BR = Cfg::BR, BK = Cfg::BK, WG = Cfg::TPB;
   constexpr int DCH = BK / KL;       // features per lane group per stage
@@ -1476,11 +1479,11 @@ int launch_assign_accumulate(hipStream_t s, int variant, const T *X, const T *xn
                                        num_cu, psums, pcounts, slots, 0, 0, false, st);
 }
 
-template <typename T, int MODE, int BCW>
+template <typename T, int MODE, int BCW, bool WIDE = false>
 static int launch_tiled_bcw(hipStream_t s, const T *X, const T *xnorm, const T *C,
                             const T *cnorm, int *labels, T *mindist, T *D, int64_t n,
                             int64_t ldn, int d, int k, bool exact) {
-  typedef TiledCfg<T, BCW> Cfg;
+  typedef TiledCfg<T, BCW, WIDE> Cfg;
   const size_t lds = (size_t)2 * (Cfg::BC + Cfg::BR) * Cfg::BK * sizeof(T);
   const int64_t row_tiles = (n + Cfg::BR - 1) / Cfg::BR;
   const int64_t tiles = MODE == 1 ? row_tiles * ((k + Cfg::BC - 1) / Cfg::BC) : row_tiles;
@@ -1490,7 +1493,7 @@ static int launch_tiled_bcw(hipStream_t s, const T *X, const T *xnorm, const T *
   const bool tail = (d % Cfg::BK) != 0;
 #define KM_TILED_X(VEC, TAIL, EXACT)                                                         \
   do {                                                                                       \
-    auto kern = assign_tiled_kernel<T, MODE, VEC, TAIL, BCW, EXACT>;                         \
+    auto kern = assign_tiled_kernel<T, MODE, VEC, TAIL, BCW, EXACT, WIDE>;                   \
     KM_TRY(ensure_dynamic_lds(reinterpret_cast<const void *>(kern), lds));                   \
     hipLaunchKernelGGL(kern, grid, dim3(Cfg::TPB), lds, s, X, xnorm, C, cnorm, labels,       \
                        mindist, D, n, ldn, d, k);                                            \
@@ -1528,6 +1531,14 @@ static int launch_tiled(hipStream_t s, const T *X, const T *xnorm, const T *C,
   // (two wavefronts) halves the matrix work spent on padding; such shapes are bandwidth-bound.
   if (k <= 64)
     return launch_tiled_bcw<T, MODE, 1>(s, X, xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k, exact);
+  // A float32 model beyond one XCD's 4 MB of L2 (500k x 784, k = 4096: 12.8 MB): the centroid
+  // stream misses L2 as well as the row slices, and the 256-centroid block, which passes over
+  // a workgroup's row slice half as often, is ahead (26.9 -> 26.3 ms, 53 -> 30 GB through the
+  // L2 miss path); while the model fits L2 it is behind (2M x 256, k = 1024: 8.37 -> 8.53 ms).
+  if constexpr (MODE == 0 && sizeof(T) == 4) {
+    if ((size_t)k * d * sizeof(T) > ((size_t)4 << 20))
+      return launch_tiled_bcw<T, MODE, 2, true>(s, X, xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k, exact);
+  }
   return launch_tiled_bcw<T, MODE, 2>(s, X, xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k, exact);
 }
 

@@ -24,6 +24,9 @@ ASSIGN_CASES = [
     (64, 8, 64), (1, 4, 1), (130, 2, 2), (3000, 40, 600), (2100, 66, 1030),
     # rows that are not a whole number of 16-byte vectors
     (1800, 255, 140), (1300, 101, 300), (900, 30, 70), (1100, 127, 1030), (700, 9, 40), (513, 63, 20),
+    # float32 models beyond 4 MB: the tiled kernel's 256-centroid block (integer keys below 128
+    # features, float compare from there on; 520 features leave a quarter-filled last stage)
+    (1500, 120, 9000), (1200, 520, 2304),
 ]
 
 
@@ -32,7 +35,10 @@ ASSIGN_CASES = [
 @pytest.mark.parametrize("n,d,k", ASSIGN_CASES)
 def test_assign_matches_oracle(hip, oracle, n, d, k, variant, dtype):
     X = blobs(n, d, max(k, 2), dtype, seed=n + d + k)
-    C = np.ascontiguousarray(X[RNG.choice(n, size=k, replace=False)]) if k <= n else None
+    if k <= n:
+        C = np.ascontiguousarray(X[RNG.choice(n, size=k, replace=False)])
+    else:  # more centroids than rows: rows drawn with repeats, nudged apart
+        C = np.ascontiguousarray((X[RNG.choice(n, size=k)] + 0.5 * RNG.standard_normal((k, d))).astype(dtype))
     with hip.Handle(n, d, k, dtype) as h:
         h.set_data(X)
         h.set_centroids(C)
@@ -136,6 +142,37 @@ def test_duplicate_centroids_lowest_index_wins(hip, oracle, variant, k, pairs, e
         assert np.allclose(C1, wC, rtol=tol, atol=tol * np.abs(wC).max())
         for lo, hi in pairs:
             assert np.array_equal(C1[hi], C0[hi]) and not np.array_equal(C1[lo], C0[lo])
+
+
+@pytest.mark.parametrize("d,k,pairs", [
+    # 7 / 36: two tiles of one wavefront; 3 / 160: the two wavefronts of a 256-centroid block;
+    # 3 / 300 and 100 / 8000: different blocks
+    (120, 9000, [(7, 36), (3, 160), (40, 300), (100, 8000)]),
+    (520, 2304, [(7, 36), (3, 160), (40, 300), (100, 2100)]),
+])
+def test_duplicate_centroids_in_the_wide_block(hip, oracle, d, k, pairs):
+    """The tie rule in the tiled kernel's 256-centroid form (float32 models beyond 4 MB)."""
+    n = 6000
+    rng = np.random.default_rng(k)
+    centers = rng.uniform(-10, 10, size=(k, d))
+    lab = rng.integers(0, k, size=n)
+    lab[:40] = np.repeat([lo for lo, _ in pairs], 10)  # every duplicated centroid has rows
+    X = np.ascontiguousarray((centers[lab] + 0.3 * rng.standard_normal((n, d))).astype(np.float32))
+    C0 = np.ascontiguousarray((centers + 0.05).astype(np.float32))
+    for lo, hi in pairs:
+        C0[hi] = C0[lo]
+    want = oracle.assign(X, C0, threads=4)
+    assert not np.isin(want, [hi for _, hi in pairs]).any()
+    with hip.Handle(n, d, k, np.float32) as h:
+        h.set_data(X)
+        h.set_centroids(C0)
+        h.set_option("assign", "mfma_tiled")
+        h.assign()
+        assert np.array_equal(h.labels(), want)
+        h.iterate(1)
+        C1 = h.centroids()
+    for lo, hi in pairs:
+        assert np.array_equal(C1[hi], C0[hi]) and not np.array_equal(C1[lo], C0[lo])
 
 
 @pytest.mark.parametrize("n,d,k,dtype,exact", [
