@@ -1535,7 +1535,7 @@ static int launch_tiled(hipStream_t s, const T *X, const T *xnorm, const T *C,
   // stream misses L2 as well as the row slices, and the 256-centroid block, which passes over
   // a workgroup's row slice half as often, is ahead (26.9 -> 26.3 ms, 53 -> 30 GB through the
   // L2 miss path); while the model fits L2 it is behind (2M x 256, k = 1024: 8.37 -> 8.53 ms).
-  if constexpr (MODE == 0 && sizeof(T) == 4) {
+  if constexpr (sizeof(T) == 4) {
     if ((size_t)k * d * sizeof(T) > ((size_t)4 << 20))
       return launch_tiled_bcw<T, MODE, 2, true>(s, X, xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k, exact);
   }
