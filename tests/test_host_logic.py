@@ -233,3 +233,67 @@ def test_cluster_namespace_clone_and_pipeline(monkeypatch):
     # the CPU backend clones into the CPU backend
     cpu = clone(cluster.KMeans(n_clusters=2, n_gpus=0, random_state=1, n_init=1))
     assert cpu.backend == "sklearn"
+
+
+class FakeHandle:
+    """Stands in for kmeans_hip.Handle: records which set got which seed and lets each
+    restart end with an inertia that depends on its seed only."""
+
+    def __init__(self, log, sets):
+        self.log, self.sets, self.cur = log, sets, 0
+        self.seed = [None] * sets
+        log.append(("create", sets))
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.log.append(("close",))
+
+    def select_set(self, s):
+        assert 0 <= s < self.sets
+        self.cur = s
+
+    def init_random_rows(self, seed):
+        self.seed[self.cur] = seed
+        self.log.append(("seed", self.cur, seed))
+
+    def fit(self, max_iter, tol):
+        assert all(s is not None for s in self.seed)
+        self.log.append(("fit", tuple(self.seed)))
+        return max_iter
+
+    def set_iterations(self):
+        return np.array([3 + s for s in self.seed], np.int32)
+
+    def inertia(self):
+        return float((self.seed[self.cur] * 7) % 11)
+
+    def centroids(self):
+        return np.full((3, 2), self.seed[self.cur], np.float32)
+
+    def labels(self):
+        return np.full(10, self.seed[self.cur], np.int32)
+
+
+@pytest.mark.parametrize("restarts,width,want_sets,want_groups", [(4, 3, 2, 2), (5, 8, 5, 1), (7, 3, 3, 3),
+                                                                  (3, 1, 1, 3)])
+def test_restarts_are_grouped_into_balanced_stacks(model, monkeypatch, restarts, width, want_sets, want_groups):
+    """n_init restarts use seeds random_state, random_state + 1, ...; as many as the shape
+    allows run stacked, in balanced groups on one handle (one upload); a spare set of the last
+    group repeats a seed and is ignored; the restart with the lowest inertia is kept."""
+    m, _ = model
+    m.n_init = restarts
+    log = []
+    monkeypatch.setattr("h2o4gpu_amd.libs.kmeans_hip.stack_width", lambda rows, cols, k, dtype, r: min(width, r))
+    m._fit_on_handle(lambda sets: FakeHandle(log, sets), 10, 2, np.float32, 3, None)
+    assert log[0] == ("create", want_sets) and log[-1] == ("close",)
+    assert sum(1 for e in log if e[0] == "create") == 1          # the rows are set up once
+    fits = [e for e in log if e[0] == "fit"]
+    assert len(fits) == want_groups
+    seeds = sorted({s for f in fits for s in f[1]})
+    assert seeds == list(range(42, 42 + restarts))                # every restart ran, none beyond
+    best = min(range(42, 42 + restarts), key=lambda s: ((s * 7) % 11, s))
+    assert m.inertia_ == float((best * 7) % 11)
+    assert (m.cluster_centers_ == best).all() and (m.labels_ == best).all()
+    assert m.n_iter_ == (3 + best if want_sets > 1 else 7)
