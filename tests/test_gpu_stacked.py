@@ -24,7 +24,8 @@ def serial_fit(hip, X, k, C0, iters, tol):
         return h.centroids(), h.labels(), h.counts(), h.inertia(), it
 
 
-SHAPES = [(50000, 32, 20, 3), (40000, 64, 64, 2), (60000, 16, 8, 4), (30000, 24, 33, 2), (20000, 8, 5, 6)]
+SHAPES = [(50000, 32, 20, 3), (40000, 64, 64, 2), (60000, 16, 8, 4), (30000, 24, 33, 2), (20000, 8, 5, 6),
+          (25000, 7, 9, 3), (20000, 3, 4, 2), (15000, 101, 12, 2), (1000, 30, 70, 2), (37, 5, 3, 2)]
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
