@@ -953,20 +953,25 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
   for (int q = 0; q < B_VECS; q++)
     xrow[q] = X + min(row0 + rr0 + q * ROWS_PER_PASS, n - 1) * (int64_t)d;
 
+  // The accumulators hold -1/2 of the reference's value: they start at -(xx + cc)/2 and the
+  // matrix cores add +x.c with the centroids staged as they are, which spares the staging of
+  // every tile a multiplication by -2. Halving and doubling are exact, so every accumulator
+  // is bit for bit -1/2 of (xx + cc) - 2 x.c accumulated in the same order; the comparisons
+  // are unaffected and the distance that leaves the kernel is 2 |acc|.
   T xx[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; rt++)
-    xx[rt] = xnorm[min(row0 + (wr * RT + rt) * MT + r, n - 1)];
+    xx[rt] = (T)-0.5 * xnorm[min(row0 + (wr * RT + rt) * MT + r, n - 1)];
   T best[RT];
   int bidx[RT];
   unsigned bkey[RT];
   int bblk[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; rt++) {
-    best[rt] = argmin_start<T>();
+    best[rt] = (T)0.5 * argmin_start<T>();  // the start value FLT_MAX on the accumulators' scale
     bidx[rt] = -1;
-    bkey[rt] = 0x7F7FFFF0u;  // first tile start (a multiple of MT) of the best key
-    bblk[rt] = -1;
+    bkey[rt] = 0x7EFFFFF0u;  // FLT_MAX / 2 with the index bits cleared
+    bblk[rt] = -1;  // first centroid of the tile the best key came from
   }
 
   vec_t areg[A_VECS], breg[B_VECS];
@@ -1001,7 +1006,7 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
     };
     const T *cbase = C + (size_t)(c0 + rr0) * d;
 #pragma unroll
-    for (int q = 0; q < A_VECS; q++)  // scaled by -2 when stored to LDS, after this stage's matrix work
+    for (int q = 0; q < A_VECS; q++)
       areg[q] = fetch(cbase + (size_t)q * ROWS_PER_PASS * d, true);
 #pragma unroll
     for (int q = 0; q < B_VECS; q++) breg[q] = fetch(xrow[q], false);
@@ -1009,7 +1014,7 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
   auto lstore = [&](int buf) {
 #pragma unroll
     for (int q = 0; q < A_VECS; q++)
-      *reinterpret_cast<vec_t *>(As + buf * A_ELEMS + lds_off[q]) = areg[q] * (T)-2;
+      *reinterpret_cast<vec_t *>(As + buf * A_ELEMS + lds_off[q]) = areg[q];
 #pragma unroll
     for (int q = 0; q < B_VECS; q++)
       *reinterpret_cast<vec_t *>(Bs + buf * B_ELEMS + lds_off[q]) = breg[q];
@@ -1026,7 +1031,7 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
     for (int ct = 0; ct < CT; ct++) {
 #pragma unroll
       for (int v = 0; v < NACC; v++) {
-        const T cc = cnorm[c0 + (wc * CT + ct) * MT + M::acc_row(v, g)];
+        const T cc = (T)-0.5 * cnorm[c0 + (wc * CT + ct) * MT + M::acc_row(v, g)];
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) acc[ct][rt][v] = xx[rt] + cc;
       }
@@ -1075,7 +1080,7 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
 #pragma unroll
           for (int rt = 0; rt < RT; rt++) {
             const int64_t row = row0 + (wr * RT + rt) * MT + r;
-            if (c < k && row < n) D[(size_t)c * ldn + row] = fabs(acc[ct][rt][v]);
+            if (c < k && row < n) D[(size_t)c * ldn + row] = (T)2 * fabs(acc[ct][rt][v]);
           }
         }
       }
@@ -1158,7 +1163,7 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
         const int64_t row = row0 + lr;
         if (row < n) {
           labels[row] = bidx[rt];
-          if (mindist) mindist[row] = best[rt];
+          if (mindist) mindist[row] = (T)2 * best[rt];
         }
       }
     }
