@@ -1106,19 +1106,33 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
         }
       }
     } else {
+      // The compare chain, three vector instructions per distance: the running best keeps
+      // the accumulator's sign (the comparison takes both magnitudes through operand
+      // modifiers), and the winner is remembered as its place inside the block, a small
+      // constant, with the block itself noted once per block. Accumulators are visited in
+      // ascending centroid order, so the strict '<' keeps the lowest index on ties.
+      int loc[RT];
+#pragma unroll
+      for (int rt = 0; rt < RT; rt++) loc[rt] = -1;
 #pragma unroll
       for (int ct = 0; ct < CT; ct++) {
 #pragma unroll
         for (int v = 0; v < NACC; v++) {
-          const int c = c0 + (wc * CT + ct) * MT + M::acc_row(v, g);
 #pragma unroll
           for (int rt = 0; rt < RT; rt++) {
-            const T dist = fabs(acc[ct][rt][v]);
-            if (dist < best[rt]) {
-              best[rt] = dist;
-              bidx[rt] = c;
+            const T a = acc[ct][rt][v];
+            if (fabs(a) < fabs(best[rt])) {
+              best[rt] = a;
+              loc[rt] = ct * NACC + v;
             }
           }
+        }
+      }
+#pragma unroll
+      for (int rt = 0; rt < RT; rt++) {
+        if (loc[rt] >= 0) {
+          bblk[rt] = c0;
+          bidx[rt] = loc[rt];
         }
       }
     }
@@ -1129,6 +1143,13 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
       for (int rt = 0; rt < RT; rt++) {
         best[rt] = __uint_as_float(bkey[rt] & 0xFFFFFFF0u);
         bidx[rt] = bblk[rt] < 0 ? -1 : bblk[rt] + key_row(bkey[rt] & 15u, g);
+      }
+    } else {
+#pragma unroll
+      for (int rt = 0; rt < RT; rt++) {
+        best[rt] = fabs(best[rt]);
+        if (bblk[rt] >= 0)
+          bidx[rt] = bblk[rt] + (wc * CT + bidx[rt] / NACC) * MT + M::acc_row(bidx[rt] % NACC, g);
       }
     }
     // lane groups of one wavefront, then the two wavefronts sharing the rows
