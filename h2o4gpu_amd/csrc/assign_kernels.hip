@@ -745,17 +745,28 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
           }
         }
       } else {
-        const int cbase = t * MT + M::acc_row(0, g);
+        // the compare chain: the running best keeps the accumulator's sign (magnitudes are
+        // compared through operand modifiers), the winner is remembered as its accumulator
+        // number, and the tile is noted once per tile
+        int loc[ROWT];
+#pragma unroll
+        for (int rt = 0; rt < ROWT; rt++) loc[rt] = -1;
 #pragma unroll
         for (int v = 0; v < NACC; v++) {
-          const int cidx = cbase + (M::acc_row(v, 0) - M::acc_row(0, 0));
 #pragma unroll
           for (int rt = 0; rt < ROWT; rt++) {
-            const T dist = fabs(acc[rt][v]);
-            if (dist < best[rt]) {
-              best[rt] = dist;
-              bidx[rt] = cidx;
+            const T a = acc[rt][v];
+            if (fabs(a) < fabs(best[rt])) {
+              best[rt] = a;
+              loc[rt] = v;
             }
+          }
+        }
+#pragma unroll
+        for (int rt = 0; rt < ROWT; rt++) {
+          if (loc[rt] >= 0) {
+            btile[rt] = t;
+            bidx[rt] = loc[rt];
           }
         }
       }
@@ -782,6 +793,12 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
         for (int rt = 0; rt < ROWT; rt++) {
           best[rt] = __uint_as_float(bkey[rt] & 0xFFFFFFF0u);
           bidx[rt] = btile[rt] < 0 ? -1 : btile[rt] * MT + key_row(bkey[rt] & 15u, g);
+        }
+      } else {
+#pragma unroll
+        for (int rt = 0; rt < ROWT; rt++) {
+          best[rt] = fabs(best[rt]);
+          if (btile[rt] >= 0) bidx[rt] = btile[rt] * MT + M::acc_row(bidx[rt], g);
         }
       }
 #pragma unroll
