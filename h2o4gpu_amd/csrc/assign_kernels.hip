@@ -859,7 +859,8 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
 // current stage's matrix work). The four wavefronts split the block 2 x 2, each
 // holding (BC/2/MT) x (BR/2/MT) result tiles in accumulators.
 // MODE 0: running argmin kept in registers across centroid blocks, halves
-// merged through LDS at the end.  MODE 1: |acc| stored to D[c*ldn + i].
+// merged through LDS at the end.  MODE 1: one centroid block per workgroup, the
+// distances stored to D[c*ldn + i].
 //
 // Preconditions (the engine's buffers satisfy them): C holds round_up(k, BC)
 // rows and cnorm round_up(k, BC) entries, the entries past k being +inf, so the
