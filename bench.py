@@ -102,6 +102,7 @@ def traffic_child(args):
         h.set_option("fuse", 0)
     if args.exact_argmin:
         h.set_option("exact_argmin", 1)
+    h.set_option("fp32_split", args.fp32_split)
     h.iterate(4)
     h.assign()
     h.close()
@@ -201,6 +202,9 @@ def main():
     ap.add_argument("--assign", default="auto", choices=sorted(kmeans_hip.ASSIGN_VARIANTS))
     ap.add_argument("--exact-argmin", action="store_true",
                     help="float32 matrix-core kernels: compare float distances instead of 16-ulp keys")
+    ap.add_argument("--fp32-split", type=int, default=0, choices=[0, 6, 9],
+                    help="float32 row-stationary shapes: dot products as this many bfloat16 products per "
+                         "feature pair on the bfloat16 matrix pipe (9: every product exact)")
     ap.add_argument("--no-fuse", action="store_true",
                     help="keep assignment and accumulation as separate kernels")
     ap.add_argument("--transform-rows", type=int, default=0,
@@ -229,7 +233,7 @@ def main():
     if not args.no_traffic:
         tail = ["--workload", args.workload, "--scale", str(args.scale), "--dtype", args.dtype,
                 "--assign", args.assign] + (["--no-fuse"] if args.no_fuse else []) + \
-               (["--exact-argmin"] if args.exact_argmin else [])
+               (["--exact-argmin"] if args.exact_argmin else []) + ["--fp32-split", str(args.fp32_split)]
         t0 = time.perf_counter()
         traffic, traffic_details = measure_traffic(tail)
         log("traffic passes: %s in %.1f s" % ("%.4g bytes per launch" % traffic if traffic else
@@ -266,6 +270,7 @@ def main():
         h.set_option("fuse", 0)
     if args.exact_argmin:
         h.set_option("exact_argmin", 1)
+    h.set_option("fp32_split", args.fp32_split)
     variant = h.assign_variant()
     log("upload %.3f s (%.1f GB/s incl. pageable staging; first call of the process %.3f s); "
         "assign variant %s" % (h2d_s, n * d * s / h2d_s / 1e9, h2d_first_s, variant))

@@ -478,6 +478,32 @@ __device__ __forceinline__ int key_row(unsigned v, int g) {
   return (int)((v >> 2) * 8 + (unsigned)g * 4 + (v & 3));
 }
 
+// float32 products on the bfloat16 matrix pipe. A float is the exact sum of three
+// bfloat16 values (8 significant bits each: the float with its low half-word cleared, the
+// same of the remainder, and the rest, every subtraction exact), so x * c is the exact sum
+// of the nine products of their parts, each of which a float holds exactly (16 bits).
+// v_mfma_f32_32x32x16_bf16 adds such products into float accumulators: the result carries
+// float rounding of the running sum only, as the float32 instruction's does. On gfx950
+// the instruction runs at 16 times the float32 rate (nine of them per 16 features take
+// 288 cycles where eight v_mfma_f32_32x32x2_f32 take 512) and, unlike the float32 one,
+// leaves the vector ALU free for the epilogue of another wavefront.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void split_bf16x3(float x, float &h, float &m, float &l) {
+  h = __uint_as_float(__float_as_uint(x) & 0xFFFF0000u);
+  const float r = x - h;
+  m = __uint_as_float(__float_as_uint(r) & 0xFFFF0000u);
+  l = r - m;  // at most 8 significant bits are left: its upper half-word holds it exactly
+}
+// upper half-words of two floats as one register: lo in bits 0-15, hi in bits 16-31
+__device__ __forceinline__ unsigned pack_bf16x2(float lo, float hi) {
+  return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
+}
+__device__ __forceinline__ floatx16 mma_bf16(uintx4 a, uintx4 b, floatx16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                 __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
 // ---------------------------------------------------------------------------
 // MFMA row-stationary variant (d <= DP, all centroids resident in LDS).
 //
@@ -501,7 +527,12 @@ __device__ __forceinline__ int key_row(unsigned v, int g) {
 // aligned to its elements: 16-byte loads that stay inside the row (padded features are
 // zero, or finite values meeting zeros on the centroid side).
 // 0: d below the vector width: scalar loads, zero padded.
-template <typename T, int DP, int ROWT, int LOAD, bool FUSE, int NW, bool EXACT = false>
+// SPLIT (float32 only; 0, 6 or 9): the dot products run on the bfloat16 matrix pipe as that
+// many products of bfloat16 parts per feature pair (see split_bf16x3). 9: every product
+// exact. 6: the three smallest (below 2^-24 of |x||c|) left out. The centroid parts are
+// staged in LDS in operand order, [tile][16-feature step][part][lane] 16 bytes each; the
+// data rows are split in registers once per row tile.
+template <typename T, int DP, int ROWT, int LOAD, bool FUSE, int NW, bool EXACT = false, int SPLIT = 0>
 __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
     const T *__restrict__ X, const T *__restrict__ xnorm,
     const T *__restrict__ C, const T *__restrict__ cnorm,
@@ -519,10 +550,14 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
   constexpr bool VECLOAD = LOAD == 1;
   // float32 argmin on integer keys (16-ulp resolution) unless the exact compare chain is asked for
   constexpr bool KEYS = sizeof(T) == 4 && !EXACT;
+  static_assert(SPLIT == 0 || (sizeof(T) == 4 && NV % 2 == 0 && LOAD != 0 && (SPLIT == 6 || SPLIT == 9)),
+                "bfloat16 parts: float32, whole 16-feature steps, vector loads");
+  constexpr int NS = NV / 2;  // (SPLIT) 16-feature steps: two of a lane's vectors each
 
   extern __shared__ __align__(16) unsigned char smem_raw[];
   T *Cs = reinterpret_cast<T *>(smem_raw);  // [KT][NV][64][VW], see cs_slot
-  T *ccs = Cs + (size_t)kp * DP;            // [kp]
+  // (SPLIT: [KT][NS][3][64] vectors of 8 bfloat16, 6 bytes per element instead of 4)
+  T *ccs = SPLIT ? reinterpret_cast<T *>(smem_raw + (size_t)kp * DP * 6) : Cs + (size_t)kp * DP;  // [kp]
   constexpr int SD = DP + 1;
   // (FUSE) sums in double: ds_add_f64 is the fast LDS floating-point atomic on gfx950
   double *sums = reinterpret_cast<double *>(ccs + kp + (kp & 1));  // [k][SD], 8-byte aligned
@@ -549,7 +584,32 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
     for (int c = tid; c < k; c += TPB) cnt[c] = 0;
   }
 
-  if (VECLOAD) {
+  if constexpr (SPLIT != 0) {
+    // one (centroid, step, lane group) per thread and turn: its 8 features, times -2
+    // (exact), split into three parts and stored as the lane's operand of that step
+    for (int e = tid; e < kp * NS * KL; e += TPB) {
+      const int c = e / (NS * KL), rem = e - c * (NS * KL), st = rem / KL, gg = rem - st * KL;
+      float h[8], m[8], l[8];
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        const int f = ((2 * st + j / VW) * KL + gg) * VW + j % VW;
+        const float v = (c < k && f < d) ? -2.0f * (float)C[(size_t)c * d + f] : 0.0f;
+        split_bf16x3(v, h[j], m[j], l[j]);
+      }
+      uintx4 ph, pm, pl;
+#pragma unroll
+      for (int w = 0; w < 4; w++) {
+        ph[w] = pack_bf16x2(h[2 * w], h[2 * w + 1]);
+        pm[w] = pack_bf16x2(m[2 * w], m[2 * w + 1]);
+        pl[w] = pack_bf16x2(l[2 * w], l[2 * w + 1]);
+      }
+      const int t = c / MT, i = c - t * MT;
+      uintx4 *dst = reinterpret_cast<uintx4 *>(smem_raw) + (size_t)((t * NS + st) * 3) * 64 + gg * MT + i;
+      dst[0] = ph;
+      dst[64] = pm;
+      dst[128] = pl;
+    }
+  } else if (VECLOAD) {
     // d == DP: 16-byte loads, four in flight per thread, one 16-byte LDS store each
     constexpr int VPR = DP / VW;  // vectors per centroid row
     const int nvec = k * VPR;
@@ -600,7 +660,7 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
       if ((c % kps) >= kset) continue;
       T acc = 0;
       for (int j = 0; j < d; j++) {
-        const T v = (T)-0.5 * Cs[cs_slot(c, j)];
+        const T v = SPLIT ? C[(size_t)c * d + j] : (T)-0.5 * Cs[cs_slot(c, j)];
         acc = acc + v * v;
       }
       ccs[c] = acc;
@@ -692,6 +752,26 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
       pl[rt] = pln[rt];
     }
     if (wrow0 + row_stride < n) fetch_rows(wrow0 + row_stride);
+    // (SPLIT) the row tile's three bfloat16 parts, packed in operand order
+    uintx4 xh[SPLIT ? ROWT : 1][SPLIT ? NS : 1], xm[SPLIT ? ROWT : 1][SPLIT ? NS : 1],
+        xl[SPLIT ? ROWT : 1][SPLIT ? NS : 1];
+    if constexpr (SPLIT != 0) {
+#pragma unroll
+      for (int rt = 0; rt < ROWT; rt++) {
+#pragma unroll
+        for (int st = 0; st < NS; st++) {
+          float h[8], m[8], l[8];
+#pragma unroll
+          for (int j = 0; j < 8; j++) split_bf16x3((float)x[rt][2 * st * VW + j], h[j], m[j], l[j]);
+#pragma unroll
+          for (int w = 0; w < 4; w++) {
+            xh[rt][st][w] = pack_bf16x2(h[2 * w], h[2 * w + 1]);
+            xm[rt][st][w] = pack_bf16x2(m[2 * w], m[2 * w + 1]);
+            xl[rt][st][w] = pack_bf16x2(l[2 * w], l[2 * w + 1]);
+          }
+        }
+      }
+    }
     T best[ROWT];
     int bidx[ROWT];
     unsigned bkey[ROWT];  // float32 path: running minimum key and its tile
@@ -702,6 +782,31 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
         const T cc = ccs[t * MT + M::acc_row(v, g)];
 #pragma unroll
         for (int rt = 0; rt < ROWT; rt++) acc[rt][v] = xx[rt] + cc;
+      }
+      if constexpr (SPLIT != 0) {
+        const uintx4 *ap = reinterpret_cast<const uintx4 *>(smem_raw) + (size_t)t * NS * 3 * 64 + lane;
+#pragma unroll
+        for (int st = 0; st < NS; st++) {
+          if (LOAD == 1 || 2 * st < nq) {
+            const uintx4 ah = ap[(st * 3 + 0) * 64], am = ap[(st * 3 + 1) * 64], al = ap[(st * 3 + 2) * 64];
+            // smallest products first
+#pragma unroll
+            for (int rt = 0; rt < ROWT; rt++) {
+              if constexpr (SPLIT == 9) {
+                acc[rt] = mma_bf16(al, xl[rt][st], acc[rt]);
+                acc[rt] = mma_bf16(al, xm[rt][st], acc[rt]);
+                acc[rt] = mma_bf16(am, xl[rt][st], acc[rt]);
+              }
+              acc[rt] = mma_bf16(al, xh[rt][st], acc[rt]);
+              acc[rt] = mma_bf16(ah, xl[rt][st], acc[rt]);
+              acc[rt] = mma_bf16(am, xm[rt][st], acc[rt]);
+              acc[rt] = mma_bf16(am, xh[rt][st], acc[rt]);
+              acc[rt] = mma_bf16(ah, xm[rt][st], acc[rt]);
+              acc[rt] = mma_bf16(ah, xh[rt][st], acc[rt]);
+            }
+          }
+        }
+        return;
       }
       const vec_t *ap = reinterpret_cast<const vec_t *>(Cs) + (size_t)t * NV * 64 + lane;
 #pragma unroll
@@ -1230,20 +1335,21 @@ static int rowstat_dp(int d) {
     if (d <= dp) return dp;
   return 0;
 }
+// split != 0: the staged centroids are three bfloat16 parts per element (6 bytes)
 template <typename T>
-static size_t rowstat_lds(int d, int k) {
+static size_t rowstat_lds(int d, int k, int split = 0) {
   const int MT = Mfma<T>::MT;
   const int kp = (k + MT - 1) / MT * MT;
-  return ((size_t)kp * rowstat_dp<T>(d) + kp) * sizeof(T);
+  return (size_t)kp * rowstat_dp<T>(d) * (split ? 6 : sizeof(T)) + (size_t)kp * sizeof(T);
 }
 
 static const size_t ROWSTAT_LDS_MAX = 96 * 1024;
 // centroids per chunk of a chunked row-stationary sweep (a multiple of the MFMA tile)
 template <typename T>
-static int rowstat_chunk(int d, int k) {
-  if (rowstat_lds<T>(d, k) <= ROWSTAT_LDS_MAX) return k;
+static int rowstat_chunk(int d, int k, int split = 0) {
+  if (rowstat_lds<T>(d, k, split) <= ROWSTAT_LDS_MAX) return k;
   const int MT = Mfma<T>::MT;
-  const size_t per = ((size_t)rowstat_dp<T>(d) + 1) * sizeof(T);
+  const size_t per = (size_t)rowstat_dp<T>(d) * (split ? 6 : sizeof(T)) + sizeof(T);
   const int kc_max = (int)(ROWSTAT_LDS_MAX / per) / MT * MT;
   const int chunks = (k + kc_max - 1) / kc_max;
   const int kc = ((k + chunks - 1) / chunks + MT - 1) / MT * MT;  // balanced
@@ -1295,9 +1401,22 @@ static int launch_valu(hipStream_t s, const T *X, const T *xnorm, const T *C,
 }
 
 template <typename T>
-static size_t rowstat_fused_lds(int d, int k) {
+static size_t rowstat_fused_lds(int d, int k, int split = 0) {
   const int dp = rowstat_dp<T>(d);
-  return rowstat_lds<T>(d, k) + 8 + (size_t)k * (dp + 1) * sizeof(double) + (size_t)k * sizeof(int);
+  return rowstat_lds<T>(d, k, split) + 8 + (size_t)k * (dp + 1) * sizeof(double) + (size_t)k * sizeof(int);
+}
+static const size_t ROWSTAT_FUSED_LDS_MAX = 150 * 1024;
+// The number of bfloat16 products (0, 6 or 9) a row-stationary launch of this shape runs
+// with when `split` is asked for: float32 rows of whole 16-feature steps whose staged parts
+// (half as large again as the floats) still fit.
+template <typename T>
+static int rowstat_split(int split, int d, int k, bool fused) {
+  if (sizeof(T) != 4 || (split != 6 && split != 9)) return 0;
+  if (rowstat_dp<T>(d) < 16 || rowstat_dp<T>(d) > 64 || d < Mfma<T>::VW) return 0;
+  if (fused ? rowstat_fused_lds<T>(d, k, split) > ROWSTAT_FUSED_LDS_MAX
+            : rowstat_lds<T>(d, k, split) > ROWSTAT_LDS_MAX)
+    return 0;  // (an assignment-only sweep is cut into chunks that fit before it gets here)
+  return split;
 }
 
 // Persistent grid of the row-stationary kernels: as many workgroups as stay
@@ -1305,7 +1424,7 @@ static size_t rowstat_fused_lds(int d, int k) {
 // one 8-wave workgroup per CU), never more than there are row tiles.
 static bool rowstat_two_per_cu(size_t lds) { return lds <= (size_t)80 * 1024; }
 
-template <typename T, int DP, int ROWT, bool FUSE, int NW>
+template <typename T, int DP, int ROWT, bool FUSE, int NW, int SPLIT = 0>
 static int launch_rowstat_nw(hipStream_t s, const T *X, const T *xnorm, const T *C,
                              const T *cnorm, int *labels, T *mindist, int64_t n, int d,
                              int k, int num_cu, double *psums, int *pcounts, int *slots,
@@ -1329,7 +1448,7 @@ static int launch_rowstat_nw(hipStream_t s, const T *X, const T *xnorm, const T 
   const bool padvec = !vec && d >= Mfma<T>::VW;
 #define KM_RS_LAUNCH_X(LOAD, EXACT)                                                           \
   do {                                                                                        \
-    auto kern = assign_rowstat_kernel<T, DP, ROWT, LOAD, FUSE, NW, EXACT>;                    \
+    auto kern = assign_rowstat_kernel<T, DP, ROWT, LOAD, FUSE, NW, EXACT, SPLIT>;             \
     KM_TRY(ensure_dynamic_lds(reinterpret_cast<const void *>(kern), lds));                    \
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), lds, s, X, xnorm, C, cnorm, \
                        labels, mindist, n, d, k, kp, psums, pcounts, c_off, merge, sets, kps, \
@@ -1338,7 +1457,10 @@ static int launch_rowstat_nw(hipStream_t s, const T *X, const T *xnorm, const T 
   // the exact-compare form exists for the float32 assignment-only kernels
 #define KM_RS_LAUNCH(LOAD)                                       \
   do {                                                           \
-    if constexpr (!FUSE && sizeof(T) == 4) {                     \
+    if constexpr (SPLIT != 0) {                                  \
+      if constexpr (LOAD != 0) KM_RS_LAUNCH_X(LOAD, false);      \
+      else return H2O4GPU_KMEANS_EARG;                           \
+    } else if constexpr (!FUSE && sizeof(T) == 4) {              \
       if (exact) KM_RS_LAUNCH_X(LOAD, true);                     \
       else KM_RS_LAUNCH_X(LOAD, false);                          \
     } else {                                                     \
@@ -1378,6 +1500,28 @@ static int launch_rowstat_dp(hipStream_t s, const T *X, const T *xnorm,
                                                    k, num_cu, psums, pcounts, slots, lds, c_off, merge, exact, st);
 }
 
+// The float32 shapes on the bfloat16 matrix pipe: the three parts of a row tile take half
+// as many registers again as the floats, so one row tile per wavefront.
+template <bool FUSE, int SPLIT>
+static int launch_rowstat_split(hipStream_t s, const float *X, const float *xnorm, const float *C,
+                                const float *cnorm, int *labels, float *mindist, int64_t n, int d,
+                                int k, int num_cu, double *psums, int *pcounts, int *slots,
+                                int c_off, int merge, const StackShape &st) {
+  const size_t lds = FUSE ? rowstat_fused_lds<float>(d, k, SPLIT) : rowstat_lds<float>(d, k, SPLIT);
+#define KM_SPLIT_CASE(DP, ROWT, NW)                                                              \
+  case DP:                                                                                       \
+    return launch_rowstat_nw<float, DP, ROWT, FUSE, NW, SPLIT>(s, X, xnorm, C, cnorm, labels,    \
+                                                               mindist, n, d, k, num_cu, psums,  \
+                                                               pcounts, slots, lds, c_off, merge, false, st)
+  switch (rowstat_dp<float>(d)) {
+    KM_SPLIT_CASE(16, 1, 16);
+    KM_SPLIT_CASE(32, 1, 16);
+    KM_SPLIT_CASE(64, 1, 8);
+  }
+#undef KM_SPLIT_CASE
+  return H2O4GPU_KMEANS_EARG;
+}
+
 template <typename T, bool FUSE>
 struct RowstatDispatch;
 #define KM_ROWSTAT_CASE(T, DP, ROWT)                                                  \
@@ -1389,7 +1533,17 @@ struct RowstatDispatch<float, FUSE> {
   static int run(hipStream_t s, const float *X, const float *xnorm, const float *C,
                  const float *cnorm, int *labels, float *mindist, int64_t n, int d,
                  int k, int num_cu, double *psums, int *pcounts, int *slots, int c_off = 0,
-                 int merge = 0, bool exact = false, const StackShape &st = StackShape()) {
+                 int merge = 0, bool exact = false, const StackShape &st = StackShape(),
+                 int split = 0) {
+    if (!exact) {
+      split = rowstat_split<float>(split, d, k, FUSE);
+      if (split == 9)
+        return launch_rowstat_split<FUSE, 9>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu,
+                                             psums, pcounts, slots, c_off, merge, st);
+      if (split == 6)
+        return launch_rowstat_split<FUSE, 6>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu,
+                                             psums, pcounts, slots, c_off, merge, st);
+    }
     switch (rowstat_dp<float>(d)) {
       KM_ROWSTAT_CASE(float, 8, 2);
       KM_ROWSTAT_CASE(float, 16, 2);
@@ -1405,7 +1559,9 @@ struct RowstatDispatch<double, FUSE> {
   static int run(hipStream_t s, const double *X, const double *xnorm, const double *C,
                  const double *cnorm, int *labels, double *mindist, int64_t n, int d,
                  int k, int num_cu, double *psums, int *pcounts, int *slots, int c_off = 0,
-                 int merge = 0, bool exact = false, const StackShape &st = StackShape()) {
+                 int merge = 0, bool exact = false, const StackShape &st = StackShape(),
+                 int split = 0) {
+    (void)split;  // float32 only
     switch (rowstat_dp<double>(d)) {
       // two row tiles keep these within 128 registers, i.e. 16 wavefronts per CU
       KM_ROWSTAT_CASE(double, 8, 2);
@@ -1444,7 +1600,7 @@ int fused_slots(int requested_variant, int64_t n, int d, int k, int num_cu) {
   if (v == ASSIGN_VALU && valu_fused_applies(d, k)) return 8 * num_cu;
   if (v != ASSIGN_ROWSTAT) return 0;
   const size_t lds = rowstat_fused_lds<T>(d, k);
-  if (lds > 150 * 1024) return 0;
+  if (lds > ROWSTAT_FUSED_LDS_MAX) return 0;
   return 2 * num_cu;  // upper bound of the grid = number of partial slots
 }
 
@@ -1509,7 +1665,7 @@ template <typename T>
 int launch_assign_accumulate(hipStream_t s, int variant, const T *X, const T *xnorm, const T *C,
                              const T *cnorm, int *labels, T *mindist, int64_t n, int d,
                              int k, int num_cu, double *psums, int *pcounts, int *slots,
-                             int *used, StackShape st) {
+                             int *used, StackShape st, int split) {
   // cnorm == nullptr: the kernel computes the centroid norms from C itself
   if (n <= 0 || d < 1 || k < 1) return H2O4GPU_KMEANS_EARG;
   const int v = pick_assign_variant<T>(variant, n, d, k);
@@ -1520,7 +1676,7 @@ int launch_assign_accumulate(hipStream_t s, int variant, const T *X, const T *xn
                                       psums, pcounts, slots);
   if (v != ASSIGN_ROWSTAT) return H2O4GPU_KMEANS_EARG;
   return RowstatDispatch<T, true>::run(s, X, xnorm, C, cnorm, labels, mindist, n, d, k,
-                                       num_cu, psums, pcounts, slots, 0, 0, false, st);
+                                       num_cu, psums, pcounts, slots, 0, 0, false, st, split);
 }
 
 template <typename T, int MODE, int BCW, bool WIDE = false>
@@ -1589,7 +1745,7 @@ static int launch_tiled(hipStream_t s, const T *X, const T *xnorm, const T *C,
 template <typename T>
 int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
                   const T *C, const T *cnorm, int *labels, T *mindist, int64_t n,
-                  int d, int k, int num_cu, int *used, bool exact, StackShape st) {
+                  int d, int k, int num_cu, int *used, bool exact, StackShape st, int split) {
   if (n <= 0) return 0;
   if (d < 1 || k < 1) return H2O4GPU_KMEANS_EARG;
   const int v = pick_assign_variant<T>(variant, n, d, k);
@@ -1598,7 +1754,7 @@ int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
   if (st.sets > 1) {  // stacked sets: the row-stationary kernel with the whole model in LDS
     if (v != ASSIGN_ROWSTAT || rowstat_chunk<T>(d, k) < k || !mindist) return H2O4GPU_KMEANS_EARG;
     return RowstatDispatch<T, false>::run(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu,
-                                          nullptr, nullptr, nullptr, 0, 0, exact, st);
+                                          nullptr, nullptr, nullptr, 0, 0, exact, st, split);
   }
   switch (v) {
     case ASSIGN_VALU:
@@ -1610,7 +1766,11 @@ int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
                                            nullptr, nullptr, nullptr);
       return launch_valu<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k);
     case ASSIGN_ROWSTAT: {
-      const int kc = rowstat_chunk<T>(d, k);
+      // (the staged bfloat16 parts are half as large again as the floats: smaller chunks)
+      const int split_dp = rowstat_dp<T>(d);
+      const bool split_ok = sizeof(T) == 4 && (split == 6 || split == 9) && !exact && split_dp >= 16 &&
+                            split_dp <= 64 && d >= Mfma<T>::VW;
+      const int kc = rowstat_chunk<T>(d, k, split_ok ? split : 0);
       if (kc < k && !mindist) {  // merging chunks needs the running minimum in memory
         if (used) *used = ASSIGN_TILED;
         return launch_tiled<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k, exact);
@@ -1618,7 +1778,8 @@ int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
       for (int c0 = 0; c0 < k; c0 += kc)
         KM_TRY((RowstatDispatch<T, false>::run(s, X, xnorm, C + (size_t)c0 * d, cnorm + c0, labels,
                                                mindist, n, d, min(kc, k - c0), num_cu, nullptr,
-                                               nullptr, nullptr, c0, c0 > 0, exact)));
+                                               nullptr, nullptr, c0, c0 > 0, exact, StackShape(),
+                                               split)));
       return 0;
     }
     case ASSIGN_TILED:
@@ -1645,24 +1806,36 @@ int launch_transform(hipStream_t s, const T *X, const T *xnorm, const T *C,
   return launch_tiled<T, 1>(s, X, xnorm, C, cnorm, nullptr, nullptr, D, n, ldn, d, k);
 }
 
+template <typename T>
+int assign_split_products(int variant, int split, int64_t n, int d, int k, bool fused) {
+  if (pick_assign_variant<T>(variant, n, d, k) != ASSIGN_ROWSTAT) return 0;
+  if (fused) return rowstat_split<T>(split, d, k, true);
+  const int dp = rowstat_dp<T>(d);
+  if (sizeof(T) != 4 || (split != 6 && split != 9) || dp < 16 || dp > 64 || d < Mfma<T>::VW) return 0;
+  const int kc = rowstat_chunk<T>(d, k, split);  // (a chunked sweep runs every chunk the same way)
+  return rowstat_split<T>(split, d, kc < k ? kc : k, false);
+}
+template int assign_split_products<float>(int, int, int64_t, int, int, bool);
+template int assign_split_products<double>(int, int, int64_t, int, int, bool);
+
 template int fused_slots<float>(int, int64_t, int, int, int);
 template int fused_slots<double>(int, int64_t, int, int, int);
 template int launch_assign_accumulate<float>(hipStream_t, int, const float *, const float *,
                                              const float *, const float *, int *, float *,
                                              int64_t, int, int, int, double *, int *, int *,
-                                             int *, StackShape);
+                                             int *, StackShape, int);
 template int launch_assign_accumulate<double>(hipStream_t, int, const double *, const double *,
                                               const double *, const double *, int *, double *,
                                               int64_t, int, int, int, double *, int *, int *,
-                                              int *, StackShape);
+                                              int *, StackShape, int);
 template int pick_assign_variant<float>(int, int64_t, int, int);
 template int pick_assign_variant<double>(int, int64_t, int, int);
 template int launch_assign<float>(hipStream_t, int, const float *, const float *,
                                   const float *, const float *, int *, float *,
-                                  int64_t, int, int, int, int *, bool, StackShape);
+                                  int64_t, int, int, int, int *, bool, StackShape, int);
 template int launch_assign<double>(hipStream_t, int, const double *, const double *,
                                    const double *, const double *, int *, double *,
-                                   int64_t, int, int, int, int *, bool, StackShape);
+                                   int64_t, int, int, int, int *, bool, StackShape, int);
 template int launch_transform<float>(hipStream_t, const float *, const float *,
                                      const float *, const float *, float *, int64_t,
                                      int64_t, int, int, int);

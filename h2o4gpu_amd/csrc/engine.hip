@@ -180,6 +180,7 @@ struct h2o4gpu_kmeans_handle {
   int opt_fuse = 1;  // 1: use the fused assign+accumulate kernel where the shape allows
   int opt_buckets = 1;  // 1: bucketed centroid sums where the sums do not fit LDS
   int opt_exact = 0;    // 1: float32 MFMA argmin on the float distances, not on 16-ulp keys
+  int opt_split = 0;    // 6 or 9: float32 row-stationary shapes as that many bfloat16 products per feature pair
   int opt_transform_batch_mb = 4096;  // device buffer of transform_host's output, per batch of rows
   int last_variant = ASSIGN_AUTO;
 
@@ -973,7 +974,7 @@ struct Engine : h2o4gpu_kmeans_handle {
     KM_TRY(ensure_cnorm());
     PROFILED("assign", launch_assign<T>(stream, opt_assign, X, xnorm, C[cur], cnorm,
                                         labels, mindist, n, d, k, num_cu, &last_variant,
-                                        opt_exact != 0, shape()));
+                                        opt_exact != 0, shape(), opt_split));
     have_mindist = true;
     return 0;
   }
@@ -1001,7 +1002,7 @@ struct Engine : h2o4gpu_kmeans_handle {
       PROFILED("assign_accumulate",
                launch_assign_accumulate<T>(stream, opt_assign, X, xnorm, C[cur], (const T *)nullptr,
                                            labels, mindist, n, d, k, num_cu, psums, pcounts, &slots,
-                                           &last_variant, shape()));
+                                           &last_variant, shape(), opt_split));
       have_mindist = true;
       return finish_update(slots, want_shift);
     }
@@ -1841,6 +1842,11 @@ KM_API int h2o4gpu_kmeans_set_option(h2o4gpu_kmeans_handle *h, const char *name,
     h->opt_transform_batch_mb = value;
     return 0;
   }
+  if (strcmp(name, "fp32_split") == 0) {
+    if (value != 0 && value != 6 && value != 9) return H2O4GPU_KMEANS_EARG;
+    h->opt_split = value;
+    return 0;
+  }
   if (strcmp(name, "fuse") == 0) {
     if (value != 0 && value != 1) return H2O4GPU_KMEANS_EARG;
     h->opt_fuse = value;
@@ -1888,7 +1894,13 @@ KM_API const char *h2o4gpu_kmeans_assign_variant(h2o4gpu_kmeans_handle *h) {
   if (!h) return "";
   int v = h->elem_size == 4 ? pick_assign_variant<float>(h->opt_assign, h->n, h->d, h->k)
                             : pick_assign_variant<double>(h->opt_assign, h->n, h->d, h->k);
-  return v < 0 ? "unsupported" : assign_variant_name(v);
+  if (v < 0) return "unsupported";
+  if (v == ASSIGN_ROWSTAT && h->elem_size == 4) {
+    const int sp = assign_split_products<float>(h->opt_assign, h->opt_split, h->n, h->d, h->k, false);
+    if (sp == 9) return "mfma_rowstat_bf16x9";
+    if (sp == 6) return "mfma_rowstat_bf16x6";
+  }
+  return assign_variant_name(v);
 }
 
 KM_API int h2o4gpu_kmeans_copy_probe(int gpu_id, size_t bytes, int reps, float *ms) {

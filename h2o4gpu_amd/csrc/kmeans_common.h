@@ -83,10 +83,18 @@ template <typename T>
 int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
                   const T *C, const T *cnorm, int *labels, T *mindist,
                   int64_t n, int d, int k, int num_cu, int *used, bool exact = false,
-                  StackShape st = StackShape());
+                  StackShape st = StackShape(), int split = 0);
 template <typename T>
 int pick_assign_variant(int requested, int64_t n, int d, int k);
 const char *assign_variant_name(int variant);
+// split (float32 row-stationary kernels only; 0, 6 or 9): run the dot products on the
+// bfloat16 matrix pipe as that many products of bfloat16 parts per feature pair (9: every
+// product exact, 6: the three below 2^-24 of |x||c| left out). assign_split_products()
+// returns the number a launch of this shape uses: 0 where the option does not apply (other
+// kernels, float64, rows padded to fewer than 16 or more than 64 features, staged parts
+// beyond the LDS budget), and such launches run the float32 matrix instructions.
+template <typename T>
+int assign_split_products(int variant, int split, int64_t n, int d, int k, bool fused);
 
 // Fused assign + accumulate (row-stationary MFMA shapes and the small VALU shapes): labels/mindist as
 // launch_assign, plus per-workgroup partial sums psums[slot][k][d] and counts
@@ -101,7 +109,7 @@ template <typename T>
 int launch_assign_accumulate(hipStream_t s, int variant, const T *X, const T *xnorm, const T *C,
                              const T *cnorm, int *labels, T *mindist, int64_t n, int d,
                              int k, int num_cu, double *psums, int *pcounts, int *slots,
-                             int *used, StackShape st = StackShape());
+                             int *used, StackShape st = StackShape(), int split = 0);
 
 // Full squared-distance matrix, centroid-major: D[c * ldn + i], i < n.
 template <typename T>

@@ -1,0 +1,161 @@
+"""The float32 row-stationary kernels with their dot products on the bfloat16 matrix pipe
+(option "fp32_split": 9 products of bfloat16 parts per feature pair, every one exact, or 6,
+the three smallest left out) against the CPU oracle and against float64 brute force, through
+the C ABI. The bar is the float32 matrix-core path's own: labels equal the oracle's except
+rows whose two nearest centroids lie within rounding of each other, minimum distances within
+the rounding of (xx + cc)."""
+import numpy as np
+import pytest
+
+from parity import assert_centroids_close, label_report
+
+pytestmark = pytest.mark.gpu
+
+
+def blobs(n, d, k, spread=5.0, sigma=1.0, seed=0, scale=1.0):
+    rng = np.random.default_rng(seed)
+    centers = rng.uniform(-spread, spread, size=(k, d))
+    X = centers[rng.integers(0, k, size=n)] + sigma * rng.standard_normal((n, d))
+    return np.ascontiguousarray((scale * X).astype(np.float32))
+
+
+# rows of exactly 16 / 32 / 64 features (16-byte loads of the slice as it lies in memory),
+# rows padded up to those widths (9..63 features, whole vectors or not), models of one tile,
+# of several, with a partly filled last tile, and one swept in LDS-sized chunks
+SHAPES = [(4096, 32, 256), (5000, 32, 100), (3001, 64, 64), (2000, 24, 33), (1000, 16, 8),
+          (900, 30, 70), (700, 9, 40), (513, 63, 20), (2500, 50, 130), (1, 16, 1), (130, 20, 2),
+          (3000, 40, 600), (2000, 16, 3000)]
+
+
+@pytest.mark.parametrize("split", [9, 6])
+@pytest.mark.parametrize("n,d,k", SHAPES)
+def test_assign_matches_oracle(hip, oracle, n, d, k, split):
+    X = blobs(n, d, max(k, 2), seed=n + d + k)
+    rng = np.random.default_rng(k)
+    if k <= n:
+        C = np.ascontiguousarray(X[rng.choice(n, size=k, replace=False)])
+    else:
+        C = np.ascontiguousarray((X[rng.choice(n, size=k)] + 0.5 * rng.standard_normal((k, d))).astype(np.float32))
+    with hip.Handle(n, d, k, np.float32) as h:
+        h.set_data(X)
+        h.set_centroids(C)
+        h.set_option("assign", "mfma_rowstat")
+        h.set_option("fp32_split", split)
+        name = h.assign_variant()
+        h.assign()
+        got, mind = h.labels(), h.min_distances()
+        h.set_option("fp32_split", 0)
+        assert h.assign_variant() == "mfma_rowstat"
+        h.assign()
+        plain, pmind = h.labels(), h.min_distances()
+    want, wmind = oracle.assign(X, C, return_mindist=True)
+    rep = label_report(oracle, X, C, got, want)
+    scale = (X.astype(np.float64) ** 2).sum(1).max() + (C.astype(np.float64) ** 2).sum(1).max()
+    eps = np.finfo(np.float32).eps
+    assert np.max(np.abs(mind.astype(np.float64) - wmind)) <= (4 * np.sqrt(d) + 40) * eps * scale
+    assert name == "mfma_rowstat_bf16x%d" % split
+    print("split %d n=%d d=%d k=%d: %s; %d labels differ from the float32 instructions'" %
+          (split, n, d, k, rep, int((got != plain).sum())))
+
+
+@pytest.mark.parametrize("split", [9, 6])
+def test_distances_are_as_close_to_float64_as_the_float32_instructions(hip, split):
+    """Minimum distances of both paths against float64 brute force, in units of the rounding
+    of (xx + cc). The keys the argmin compares drop four mantissa bits on both paths, so the
+    exact-compare option is used for the float32 side and the split side is given twice its
+    worst error plus those four bits."""
+    n, d, k = 20000, 32, 96
+    X = blobs(n, d, k, spread=40.0, sigma=3.0, seed=5)
+    C = np.ascontiguousarray(X[np.random.default_rng(1).choice(n, size=k, replace=False)])
+    X64, C64 = X.astype(np.float64), C.astype(np.float64)
+    D = (X64 * X64).sum(1)[:, None] + (C64 * C64).sum(1)[None, :] - 2.0 * X64 @ C64.T
+    truth, tl = D.min(1), D.argmin(1)
+    unit = np.finfo(np.float32).eps * ((X64 * X64).sum(1) + (C64[tl] ** 2).sum(1))
+    out = {}
+    for name, opts in (("f32", {"exact_argmin": 1}), ("split", {"fp32_split": split})):
+        with hip.Handle(n, d, k, np.float32) as h:
+            h.set_data(X)
+            h.set_centroids(C)
+            h.set_option("assign", "mfma_rowstat")
+            for o, v in opts.items():
+                h.set_option(o, v)
+            h.assign()
+            out[name] = (h.labels(), np.abs(h.min_distances().astype(np.float64) - truth) / unit)
+    f32_err, split_err = out["f32"][1], out["split"][1]
+    print("max error in units of eps*(xx+cc): float32 instructions %.2f, %d bfloat16 products %.2f" %
+          (f32_err.max(), split, split_err.max()))
+    assert split_err.max() <= 2 * f32_err.max() + 16
+    assert int((out["split"][0] != tl).sum()) <= int((out["f32"][0] != tl).sum()) + 2
+
+
+@pytest.mark.parametrize("split", [9, 6])
+@pytest.mark.parametrize("n,d,k", [(60000, 32, 256), (30000, 64, 64), (20000, 20, 40), (15000, 48, 100)])
+def test_fit_matches_oracle(hip, oracle, n, d, k, split):
+    """The fused step (labels and sums in one kernel) from given centroids."""
+    X = blobs(n, d, k, spread=20.0, sigma=1.0, seed=n)
+    rng = np.random.default_rng(3)
+    centres = np.stack([X[rng.choice(n, 40)].mean(0) for _ in range(k)])  # rough, distinct starts
+    C0 = np.ascontiguousarray(centres.astype(np.float32))
+    iters = 6
+    with hip.Handle(n, d, k, np.float32) as h:
+        h.set_data(X)
+        h.set_option("fp32_split", split)
+        h.set_centroids(C0)
+        assert h.assign_variant() == "mfma_rowstat_bf16x%d" % split
+        assert h.fit(iters, 0.0) == iters
+        C, L, counts, inertia = h.centroids(), h.labels(), h.counts(), h.inertia()
+        h.set_centroids(C0)
+        h.fit(iters, 0.0)
+        assert np.array_equal(h.centroids(), C), "two fits from the same start differ"
+    wC, wL, _, _ = oracle.lloyd(X, C0, iters, 0.0, threads=4)
+    rep = label_report(oracle, X, C, L, oracle.assign(X, C, threads=4))
+    print("fit split %d n=%d d=%d k=%d: %s" % (split, n, d, k, rep))
+    assert counts.sum() == n  # (the counts of the last update; the labels are one assignment later)
+    if np.array_equal(L, wL):
+        assert_centroids_close(C, wC, np.float32)
+    X64 = X.astype(np.float64)
+    want_inertia = ((X64 - wC.astype(np.float64)[wL]) ** 2).sum()
+    assert abs(inertia - want_inertia) <= 1e-4 * want_inertia
+
+
+def test_stacked_sets_take_the_option(hip):
+    n, d, k, sets = 30000, 32, 20, 3
+    X = blobs(n, d, k, seed=9)
+    rng = np.random.default_rng(7)
+    starts = [np.ascontiguousarray(X[rng.choice(n, size=k, replace=False)]) for _ in range(sets)]
+    with hip.Handle(n, d, k, np.float32, sets=sets) as h:
+        h.set_data(X)
+        h.set_option("fp32_split", 9)
+        for s in range(sets):
+            h.select_set(s)
+            h.set_centroids(starts[s])
+        h.fit(5, 0.0)
+        got = []
+        for s in range(sets):
+            h.select_set(s)
+            got.append((h.centroids(), h.labels(), h.inertia()))
+    for s in range(sets):
+        with hip.Handle(n, d, k, np.float32) as h:
+            h.set_data(X)
+            h.set_option("assign", "mfma_rowstat")
+            h.set_option("fp32_split", 9)
+            h.set_centroids(starts[s])
+            h.fit(5, 0.0)
+            assert np.array_equal(h.labels(), got[s][1])
+            assert np.array_equal(h.centroids(), got[s][0])
+            assert h.inertia() == got[s][2]
+
+
+def test_option_values(hip):
+    with hip.Handle(100, 32, 4, np.float32) as h:
+        for bad in (1, 3, 12, -9):
+            with pytest.raises(hip.KMeansHipError):
+                h.set_option("fp32_split", bad)
+    X = blobs(2000, 32, 40, seed=2).astype(np.float64)
+    with hip.Handle(2000, 32, 40, np.float64) as h:  # float64: accepted, without effect
+        h.set_data(X)
+        h.set_centroids(X[:40])
+        h.set_option("assign", "mfma_rowstat")
+        h.set_option("fp32_split", 9)
+        assert h.assign_variant() == "mfma_rowstat"
+        h.assign()
