@@ -330,6 +330,27 @@ def main():
         transform = {"rows": int(H.shape[0]), "kernel_ms": ms, "launches": cnt, "tflops": tf,
                      "mfma_frac": tf / peak, "end_to_end_seconds": wall,
                      "output_bytes": float(H.shape[0]) * k * s}
+    # the same steps with the float32 dot products on the bfloat16 matrix pipe (an option of
+    # the row-stationary kernels, off by default; never part of `value`)
+    split_leg = None
+    if args.fp32_split == 0 and args.dtype == "f32" and variant == "mfma_rowstat":
+        h.set_option("fp32_split", 6)
+        if h.assign_variant() == "mfma_rowstat_bf16x6":
+            h.set_centroids(C0)
+            h.iterate(args.warmup)
+            h.timer_start()
+            h.iterate(args.steps)
+            ms6 = h.timer_stop() / args.steps
+            h.profile(True)
+            h.iterate(args.steps)
+            cnt6, kms6 = h.kernel_time(dom)
+            h.profile(False)
+            h.assign()
+            split_leg = {"option": "fp32_split=6", "assign_variant": "mfma_rowstat_bf16x6",
+                         "ms_per_step": ms6, "iterations_per_s": 1000.0 / ms6,
+                         "kernel_avg_ms": kms6 / max(cnt6, 1), "inertia": h.inertia(),
+                         "note": "products of bfloat16 parts, float32 accumulation; same parity bars"}
+        h.set_option("fp32_split", 0)
     h.close()
 
     out = {
@@ -354,6 +375,8 @@ def main():
     }
     if transform:
         out["transform"] = transform
+    if split_leg:
+        out["fp32_split"] = split_leg
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(X, C0, args.cpu_iters)
         out["cpu_reference_path"] = sklearn_baseline(X, C0, args.sklearn_rows)

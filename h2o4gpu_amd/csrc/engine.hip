@@ -1326,6 +1326,12 @@ static int create_engine(h2o4gpu_kmeans_handle **out, size_t rows, size_t cols, 
     e->k = sets * e->kps;
   }
   e->verbose = verbose;
+  // The reference's entry points have no argument for it: H2O4GPU_KMEANS_FP32_SPLIT=6 (or 9)
+  // in the environment turns the "fp32_split" option on for every handle created afterwards.
+  if (const char *env = getenv("H2O4GPU_KMEANS_FP32_SPLIT")) {
+    const int v = atoi(env);
+    if (v == 6 || v == 9) e->opt_split = v;
+  }
   if (gpu_id < 0) gpu_id = 0;
   e->dev = gpu_id % nvis;  // kmeans_init: gpu_id = gpu_idtry % n_gpuvis
   int rc = e->create();

@@ -159,3 +159,32 @@ def test_option_values(hip):
         h.set_option("fp32_split", 9)
         assert h.assign_variant() == "mfma_rowstat"
         h.assign()
+
+
+@pytest.mark.timeout(900)
+@pytest.mark.parametrize("split", [9, 6])
+@pytest.mark.parametrize("name,e2e_iters", [("C3", 6), ("C2", 20)])
+def test_full_benchmark_shape(hip, oracle, name, e2e_iters, split):
+    """10M x 32, k = 256 and 1M x 64, k = 64 at full size with the option on: one Lloyd step
+    on all rows beside the oracle at the start and at the fitted centroids, and a fixed number
+    of iterations end to end, to the same bars as the float32 instructions' full-size test."""
+    from h2o4gpu_amd import datasets
+    from test_gpu_configs import _end_to_end_all_rows, _lockstep_all_rows
+    X, k, _ = datasets.make(name, 1.0, np.float32)
+    n, d = X.shape
+    C0 = datasets.seeded_row_init(X, k, datasets.SHAPES[name][3])
+    tag = "%s float32 bf16x%d" % (name, split)
+    with hip.Handle(n, d, k, np.float32) as h:
+        h.set_data(X)
+        h.set_option("fp32_split", split)
+        assert h.assign_variant() == "mfma_rowstat_bf16x%d" % split
+        start = _lockstep_all_rows(hip, oracle, h, X, C0, np.float32, tag + " start")
+        h.set_centroids(C0)
+        h.fit(20, 0.0)
+        C, L = h.centroids(), h.labels()
+        h.set_centroids(C0)
+        h.fit(20, 0.0)
+        assert np.array_equal(h.centroids(), C) and np.array_equal(h.labels(), L), "fit does not repeat"
+        fitted = _lockstep_all_rows(hip, oracle, h, X, C, np.float32, tag + " fitted")
+        e2e = _end_to_end_all_rows(hip, oracle, h, X, C0, np.float32, e2e_iters, tag)
+    print("full shape %s: start %s\nfitted %s\nend to end %s" % (tag, start, fitted, e2e))
