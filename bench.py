@@ -203,7 +203,7 @@ def main():
     ap.add_argument("--exact-argmin", action="store_true",
                     help="float32 matrix-core kernels: compare float distances instead of 16-ulp keys")
     ap.add_argument("--fp32-split", type=int, default=0, choices=[0, 6, 9],
-                    help="float32 row-stationary shapes: dot products as this many bfloat16 products per "
+                    help="float32 matrix-core kernels: dot products as this many bfloat16 products per "
                          "feature pair on the bfloat16 matrix pipe (9: every product exact)")
     ap.add_argument("--no-fuse", action="store_true",
                     help="keep assignment and accumulation as separate kernels")
@@ -331,11 +331,11 @@ def main():
                      "mfma_frac": tf / peak, "end_to_end_seconds": wall,
                      "output_bytes": float(H.shape[0]) * k * s}
     # the same steps with the float32 dot products on the bfloat16 matrix pipe (an option of
-    # the row-stationary kernels, off by default; never part of `value`)
+    # the matrix-core kernels, off by default; never part of `value`)
     split_leg = None
-    if args.fp32_split == 0 and args.dtype == "f32" and variant == "mfma_rowstat":
+    if args.fp32_split == 0 and args.dtype == "f32" and variant in ("mfma_rowstat", "mfma_tiled"):
         h.set_option("fp32_split", 6)
-        if h.assign_variant() == "mfma_rowstat_bf16x6":
+        if h.assign_variant() == variant + "_bf16x6":
             h.set_centroids(C0)
             h.iterate(args.warmup)
             h.timer_start()
@@ -346,7 +346,7 @@ def main():
             cnt6, kms6 = h.kernel_time(dom)
             h.profile(False)
             h.assign()
-            split_leg = {"option": "fp32_split=6", "assign_variant": "mfma_rowstat_bf16x6",
+            split_leg = {"option": "fp32_split=6", "assign_variant": variant + "_bf16x6",
                          "ms_per_step": ms6, "iterations_per_s": 1000.0 / ms6,
                          "kernel_avg_ms": kms6 / max(cnt6, 1), "inertia": h.inertia(),
                          "note": "products of bfloat16 parts, float32 accumulation; same parity bars"}

@@ -980,7 +980,7 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
 // workgroup and come from HBM/MALL every time they are re-read, centroid blocks
 // are shared by all workgroups and hit L2, so for large k the wider centroid
 // block (BCW = 4) halves the expensive traffic.
-template <typename T, int BCW, bool WIDE = false>
+template <typename T, int BCW, bool WIDE = false, int SPLIT = 0>
 struct TiledCfg {
   static constexpr int TPB = 2 * BCW * 64;
   // WIDE: every wavefront holds twice as many centroid tiles (a 256-centroid block for four
@@ -994,17 +994,24 @@ struct TiledCfg {
   // features per stage. The 64-centroid form serves bandwidth-bound shapes (k <= 64): half
   // the stage depth halves its LDS image, so twice as many workgroups keep loads in flight
   // (500k x 784, k = 10: 0.62 -> 0.49 ms; a quarter of the depth was slower again).
-  static constexpr int BK = (sizeof(T) == 4 ? 32 : 16) / (BCW == 1 || WIDE ? 2 : 1);
+  // SPLIT (float32 dot products as products of bfloat16 parts, see split_bf16x3): a stage is
+  // one 16-feature step of the bfloat16 instruction; its three parts per element take 6 bytes
+  // of LDS where the float takes 4.
+  static constexpr int BK = SPLIT ? 16 : (sizeof(T) == 4 ? 32 : 16) / (BCW == 1 || WIDE ? 2 : 1);
+  static constexpr size_t LDS_BYTES = (size_t)2 * (BC + BR) * BK * (SPLIT ? 6 : sizeof(T));
 };
 
-template <typename T, int MODE, bool VECLOAD, bool DTAIL, int BCW, bool EXACT = false, bool WIDE = false>
+template <typename T, int MODE, bool VECLOAD, bool DTAIL, int BCW, bool EXACT = false, bool WIDE = false,
+          int SPLIT = 0>
 __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_kernel(
     const T *__restrict__ X, const T *__restrict__ xnorm,
     const T *__restrict__ C, const T *__restrict__ cnorm,
     int *__restrict__ labels, T *__restrict__ mindist, T *__restrict__ D,
     int64_t n, int64_t ldn, int d, int k) {
   typedef Mfma<T> M;
-  typedef TiledCfg<T, BCW, WIDE> Cfg;
+  typedef TiledCfg<T, BCW, WIDE, SPLIT> Cfg;
+  static_assert(SPLIT == 0 || (sizeof(T) == 4 && VECLOAD && (SPLIT == 6 || SPLIT == 9)),
+                "bfloat16 parts: float32 rows fetched as vectors");
   constexpr int MT = M::MT, KL = M::KL, NACC = M::NACC, VW = M::VW;
   constexpr int BC = Cfg::BC, BR = Cfg::BR, BK = Cfg::BK, WG = Cfg::TPB;
   constexpr int DCH = BK / KL;       // features per lane group per stage
@@ -1026,6 +1033,10 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
   T *As = reinterpret_cast<T *>(smem_raw);  // [2][A_ELEMS]
   T *Bs = As + 2 * A_ELEMS;                 // [2][B_ELEMS]
   // after the main loop the same memory is reused for the cross-wave merge
+  // SPLIT: [2][tile][16-feature step][part][64 lanes] vectors of 8 bfloat16 for either operand
+  constexpr int NSB = SPLIT ? NV / 2 : 1;  // 16-feature steps per stage
+  constexpr int A_BYTES = BC * BK * 6, B_BYTES = BR * BK * 6;
+  unsigned char *Ab = smem_raw, *Bb = smem_raw + 2 * A_BYTES;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -1067,6 +1078,14 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
     // of the vector its access stays a conflict-free permutation.
     const int slot = (gg * MT + i) ^ (((s / VW) * KL + gg) & 7);
     lds_off[q] = ((t * NV + s / VW) * 64 + slot) * VW;
+    if constexpr (SPLIT != 0) {
+      // byte offset of the high part: lane group step sf = s / VW is half sf % 2 of the
+      // 16-feature step sf / 2; the middle and low parts follow 1 KB and 2 KB behind. (The 64
+      // threads of a wavefront write 16 consecutive lane slots of 2 lane groups and both
+      // halves: every bank equally often, no swizzle needed.)
+      const int sf = s / VW;
+      lds_off[q] = ((((t * NSB + sf / 2) * 3) * 64 + gg * MT + i) * 16) + (sf % 2) * 8;
+    }
   }
   int rd_slot[NV];  // this lane's (swizzled) slot when it reads vector q of a tile
 #pragma unroll
@@ -1134,7 +1153,33 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
 #pragma unroll
     for (int q = 0; q < B_VECS; q++) breg[q] = fetch(xrow[q], false);
   };
+  // (SPLIT) the three bfloat16 parts of a staged vector, 8 bytes each
+  auto store_parts = [&](unsigned char *dst, const vec_t &v) {
+    if constexpr (SPLIT != 0) {
+      float h[4], m[4], l[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) split_bf16x3((float)v[e], h[e], m[e], l[e]);
+      typedef unsigned uintx2 __attribute__((ext_vector_type(2)));
+      uintx2 ph, pm, pl;
+      ph[0] = pack_bf16x2(h[0], h[1]);
+      ph[1] = pack_bf16x2(h[2], h[3]);
+      pm[0] = pack_bf16x2(m[0], m[1]);
+      pm[1] = pack_bf16x2(m[2], m[3]);
+      pl[0] = pack_bf16x2(l[0], l[1]);
+      pl[1] = pack_bf16x2(l[2], l[3]);
+      *reinterpret_cast<uintx2 *>(dst) = ph;
+      *reinterpret_cast<uintx2 *>(dst + 1024) = pm;
+      *reinterpret_cast<uintx2 *>(dst + 2048) = pl;
+    }
+  };
   auto lstore = [&](int buf) {
+    if constexpr (SPLIT != 0) {
+#pragma unroll
+      for (int q = 0; q < A_VECS; q++) store_parts(Ab + buf * A_BYTES + lds_off[q], areg[q]);
+#pragma unroll
+      for (int q = 0; q < B_VECS; q++) store_parts(Bb + buf * B_BYTES + lds_off[q], breg[q]);
+      return;
+    }
 #pragma unroll
     for (int q = 0; q < A_VECS; q++)
       *reinterpret_cast<vec_t *>(As + buf * A_ELEMS + lds_off[q]) = areg[q];
@@ -1168,10 +1213,45 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
       const int buf = st & 1;
       if (st + 2 < nstage || (!DTAIL && st + 1 < nstage)) gload(c0, st + 1, std::false_type{});
       else if (st + 1 < nstage) gload(c0, st + 1, std::true_type{});
+      if constexpr (SPLIT != 0) {
+        const uintx4 *ap = reinterpret_cast<const uintx4 *>(Ab + buf * A_BYTES) + lane;
+        const uintx4 *bp = reinterpret_cast<const uintx4 *>(Bb + buf * B_BYTES) + lane;
+#pragma unroll
+        for (int sb = 0; sb < NSB; sb++) {
+          uintx4 bh[RT], bm[RT], bl[RT];
+#pragma unroll
+          for (int rt = 0; rt < RT; rt++) {
+            const int o = (((wr * RT + rt) * NSB + sb) * 3) * 64;
+            bh[rt] = bp[o];
+            bm[rt] = bp[o + 64];
+            bl[rt] = bp[o + 128];
+          }
+#pragma unroll
+          for (int ct = 0; ct < CT; ct++) {
+            const int o = (((wc * CT + ct) * NSB + sb) * 3) * 64;
+            const uintx4 ah = ap[o], am = ap[o + 64], al = ap[o + 128];
+            // smallest products first
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++) {
+              if constexpr (SPLIT == 9) {
+                acc[ct][rt] = mma_bf16(al, bl[rt], acc[ct][rt]);
+                acc[ct][rt] = mma_bf16(al, bm[rt], acc[ct][rt]);
+                acc[ct][rt] = mma_bf16(am, bl[rt], acc[ct][rt]);
+              }
+              acc[ct][rt] = mma_bf16(al, bh[rt], acc[ct][rt]);
+              acc[ct][rt] = mma_bf16(ah, bl[rt], acc[ct][rt]);
+              acc[ct][rt] = mma_bf16(am, bm[rt], acc[ct][rt]);
+              acc[ct][rt] = mma_bf16(am, bh[rt], acc[ct][rt]);
+              acc[ct][rt] = mma_bf16(ah, bm[rt], acc[ct][rt]);
+              acc[ct][rt] = mma_bf16(ah, bh[rt], acc[ct][rt]);
+            }
+          }
+        }
+      }
       const vec_t *ap = reinterpret_cast<const vec_t *>(As + buf * A_ELEMS);
       const vec_t *bp = reinterpret_cast<const vec_t *>(Bs + buf * B_ELEMS);
 #pragma unroll
-      for (int q = 0; q < NV; q++) {
+      for (int q = 0; q < (SPLIT ? 0 : NV); q++) {
         if (DTAIL && st + 1 == nstage && q >= nq_tail) continue;  // nothing but zeros there
         vec_t a[CT], b[RT];
 #pragma unroll
@@ -1679,12 +1759,12 @@ int launch_assign_accumulate(hipStream_t s, int variant, const T *X, const T *xn
                                        num_cu, psums, pcounts, slots, 0, 0, false, st, split);
 }
 
-template <typename T, int MODE, int BCW, bool WIDE = false>
+template <typename T, int MODE, int BCW, bool WIDE = false, int SPLIT = 0>
 static int launch_tiled_bcw(hipStream_t s, const T *X, const T *xnorm, const T *C,
                             const T *cnorm, int *labels, T *mindist, T *D, int64_t n,
                             int64_t ldn, int d, int k, bool exact) {
-  typedef TiledCfg<T, BCW, WIDE> Cfg;
-  const size_t lds = (size_t)2 * (Cfg::BC + Cfg::BR) * Cfg::BK * sizeof(T);
+  typedef TiledCfg<T, BCW, WIDE, SPLIT> Cfg;
+  const size_t lds = Cfg::LDS_BYTES;
   const int64_t row_tiles = (n + Cfg::BR - 1) / Cfg::BR;
   const int64_t tiles = MODE == 1 ? row_tiles * ((k + Cfg::BC - 1) / Cfg::BC) : row_tiles;
   if (tiles > 2147483647ll) return H2O4GPU_KMEANS_EARG;
@@ -1693,7 +1773,7 @@ static int launch_tiled_bcw(hipStream_t s, const T *X, const T *xnorm, const T *
   const bool tail = (d % Cfg::BK) != 0;
 #define KM_TILED_X(VEC, TAIL, EXACT)                                                         \
   do {                                                                                       \
-    auto kern = assign_tiled_kernel<T, MODE, VEC, TAIL, BCW, EXACT, WIDE>;                   \
+    auto kern = assign_tiled_kernel<T, MODE, VEC, TAIL, BCW, EXACT, WIDE, SPLIT>;            \
     KM_TRY(ensure_dynamic_lds(reinterpret_cast<const void *>(kern), lds));                   \
     hipLaunchKernelGGL(kern, grid, dim3(Cfg::TPB), lds, s, X, xnorm, C, cnorm, labels,       \
                        mindist, D, n, ldn, d, k);                                            \
@@ -1714,17 +1794,45 @@ static int launch_tiled_bcw(hipStream_t s, const T *X, const T *xnorm, const T *
   } while (0)
   if (vec && !tail) KM_TILED(true, false);
   else if (vec) KM_TILED(true, true);
-  else KM_TILED(false, true);
+  else if constexpr (SPLIT == 0) KM_TILED(false, true);
+  else return H2O4GPU_KMEANS_EARG;
 #undef KM_TILED
 #undef KM_TILED_X
   KM_HIP_TRY(hipGetLastError());
   return 0;
 }
 
+// The shapes of the tiled kernel that take the bfloat16-parts option: float32 rows fetched
+// as 16-byte vectors, more than 64 centroids (below that the kernel waits for memory, not
+// for the matrix pipe).
+template <typename T>
+static int tiled_split(int split, int d, int k) {
+  if (sizeof(T) != 4 || (split != 6 && split != 9)) return 0;
+  if (d < Mfma<T>::VW || k <= 64) return 0;
+  return split;
+}
+
 template <typename T, int MODE>
 static int launch_tiled(hipStream_t s, const T *X, const T *xnorm, const T *C,
                         const T *cnorm, int *labels, T *mindist, T *D, int64_t n,
-                        int64_t ldn, int d, int k, bool exact = false) {
+                        int64_t ldn, int d, int k, bool exact = false, int split = 0) {
+  if constexpr (sizeof(T) == 4) {
+    // (with the parts the 256-centroid block is ahead whenever it has the centroids to fill
+    // it: 2M x 256, k = 1024 5.87 -> 5.37 ms, 500k x 784, k = 4096 14.96 -> 13.52 ms)
+    const bool wide = k > 128;
+    switch (tiled_split<T>(split, d, k)) {
+#define KM_TILED_SPLIT(SP)                                                                         \
+  case SP:                                                                                         \
+    if (wide)                                                                                      \
+      return launch_tiled_bcw<T, MODE, 2, true, SP>(s, X, xnorm, C, cnorm, labels, mindist, D, n,  \
+                                                    ldn, d, k, exact);                             \
+    return launch_tiled_bcw<T, MODE, 2, false, SP>(s, X, xnorm, C, cnorm, labels, mindist, D, n,   \
+                                                   ldn, d, k, exact)
+      KM_TILED_SPLIT(6);
+      KM_TILED_SPLIT(9);
+#undef KM_TILED_SPLIT
+    }
+  }
   // Measured at 2M x 256, k = 1024 and 500k x 784, k = 4096: two 4-wave workgroups per CU
   // (BCW = 2) beat one 8-wave workgroup with the wider centroid block (BCW = 4) by 5-10 %,
   // so the 128-centroid form is used for large models. Up to 64 centroids a 64-wide block
@@ -1773,7 +1881,7 @@ int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
       const int kc = rowstat_chunk<T>(d, k, split_ok ? split : 0);
       if (kc < k && !mindist) {  // merging chunks needs the running minimum in memory
         if (used) *used = ASSIGN_TILED;
-        return launch_tiled<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k, exact);
+        return launch_tiled<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k, exact, split);
       }
       for (int c0 = 0; c0 < k; c0 += kc)
         KM_TRY((RowstatDispatch<T, false>::run(s, X, xnorm, C + (size_t)c0 * d, cnorm + c0, labels,
@@ -1783,7 +1891,7 @@ int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
       return 0;
     }
     case ASSIGN_TILED:
-      return launch_tiled<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k, exact);
+      return launch_tiled<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k, exact, split);
   }
   return H2O4GPU_KMEANS_EARG;
 }
@@ -1791,7 +1899,7 @@ int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
 template <typename T>
 int launch_transform(hipStream_t s, const T *X, const T *xnorm, const T *C,
                      const T *cnorm, T *D, int64_t n, int64_t ldn, int d, int k,
-                     int num_cu) {
+                     int num_cu, int split) {
   if (n <= 0) return 0;
   if (d < 1 || k < 1) return H2O4GPU_KMEANS_EARG;
   if (k <= 16 && d <= 64) {
@@ -1803,12 +1911,14 @@ int launch_transform(hipStream_t s, const T *X, const T *xnorm, const T *C,
                                          nullptr, nullptr, nullptr, D, ldn);
     return launch_valu<T, 1>(s, X, xnorm, C, cnorm, nullptr, nullptr, D, n, ldn, d, k);
   }
-  return launch_tiled<T, 1>(s, X, xnorm, C, cnorm, nullptr, nullptr, D, n, ldn, d, k);
+  return launch_tiled<T, 1>(s, X, xnorm, C, cnorm, nullptr, nullptr, D, n, ldn, d, k, false, split);
 }
 
 template <typename T>
 int assign_split_products(int variant, int split, int64_t n, int d, int k, bool fused) {
-  if (pick_assign_variant<T>(variant, n, d, k) != ASSIGN_ROWSTAT) return 0;
+  const int v = pick_assign_variant<T>(variant, n, d, k);
+  if (v == ASSIGN_TILED) return fused ? 0 : tiled_split<T>(split, d, k);
+  if (v != ASSIGN_ROWSTAT) return 0;
   if (fused) return rowstat_split<T>(split, d, k, true);
   const int dp = rowstat_dp<T>(d);
   if (sizeof(T) != 4 || (split != 6 && split != 9) || dp < 16 || dp > 64 || d < Mfma<T>::VW) return 0;
@@ -1838,9 +1948,9 @@ template int launch_assign<double>(hipStream_t, int, const double *, const doubl
                                    int64_t, int, int, int, int *, bool, StackShape, int);
 template int launch_transform<float>(hipStream_t, const float *, const float *,
                                      const float *, const float *, float *, int64_t,
-                                     int64_t, int, int, int);
+                                     int64_t, int, int, int, int);
 template int launch_transform<double>(hipStream_t, const double *, const double *,
                                       const double *, const double *, double *,
-                                      int64_t, int64_t, int, int, int);
+                                      int64_t, int64_t, int, int, int, int);
 
 }  // namespace kmhip

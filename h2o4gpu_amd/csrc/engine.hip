@@ -180,7 +180,7 @@ struct h2o4gpu_kmeans_handle {
   int opt_fuse = 1;  // 1: use the fused assign+accumulate kernel where the shape allows
   int opt_buckets = 1;  // 1: bucketed centroid sums where the sums do not fit LDS
   int opt_exact = 0;    // 1: float32 MFMA argmin on the float distances, not on 16-ulp keys
-  int opt_split = 0;    // 6 or 9: float32 row-stationary shapes as that many bfloat16 products per feature pair
+  int opt_split = 0;    // 6 or 9: float32 matrix-core kernels as that many bfloat16 products per feature pair
   int opt_transform_batch_mb = 4096;  // device buffer of transform_host's output, per batch of rows
   int last_variant = ASSIGN_AUTO;
 
@@ -1284,7 +1284,8 @@ struct Engine : h2o4gpu_kmeans_handle {
     KM_TRY(upload_rows(dev, stream, dX, src, cur_rows * d * sizeof(T)));
     PROFILED("row_norms", launch_row_norms<T>(stream, dX, dxn, (int64_t)cur_rows, d));
     PROFILED("transform", launch_transform<T>(stream, dX, dxn, C[cur], cnorm, dD,
-                                              (int64_t)cur_rows, (int64_t)cur_rows, d, k, num_cu));
+                                              (int64_t)cur_rows, (int64_t)cur_rows, d, k, num_cu,
+                                              opt_split));
     T *dst = static_cast<T *>(hD) + lo;
     if (cur_rows == rows)  // a single batch is one contiguous [k][rows] block
       KM_TRY(download_rows(dev, stream, dst, dD, (size_t)k * rows * sizeof(T)));
@@ -1299,7 +1300,7 @@ struct Engine : h2o4gpu_kmeans_handle {
     if (!have_data || !have_centroids || !d_dist || sets > 1) return H2O4GPU_KMEANS_ESTATE;
     KM_TRY(ensure_cnorm());
     PROFILED("transform", launch_transform<T>(stream, X, xnorm, C[cur], cnorm,
-                                              static_cast<T *>(d_dist), n, n, d, k, num_cu));
+                                              static_cast<T *>(d_dist), n, n, d, k, num_cu, opt_split));
     KM_HIP_TRY(hipStreamSynchronize(stream));
     return 0;
   }
@@ -1901,10 +1902,12 @@ KM_API const char *h2o4gpu_kmeans_assign_variant(h2o4gpu_kmeans_handle *h) {
   int v = h->elem_size == 4 ? pick_assign_variant<float>(h->opt_assign, h->n, h->d, h->k)
                             : pick_assign_variant<double>(h->opt_assign, h->n, h->d, h->k);
   if (v < 0) return "unsupported";
-  if (v == ASSIGN_ROWSTAT && h->elem_size == 4) {
+  if (h->elem_size == 4) {
     const int sp = assign_split_products<float>(h->opt_assign, h->opt_split, h->n, h->d, h->k, false);
-    if (sp == 9) return "mfma_rowstat_bf16x9";
-    if (sp == 6) return "mfma_rowstat_bf16x6";
+    if (v == ASSIGN_ROWSTAT && sp == 9) return "mfma_rowstat_bf16x9";
+    if (v == ASSIGN_ROWSTAT && sp == 6) return "mfma_rowstat_bf16x6";
+    if (v == ASSIGN_TILED && sp == 9) return "mfma_tiled_bf16x9";
+    if (v == ASSIGN_TILED && sp == 6) return "mfma_tiled_bf16x6";
   }
   return assign_variant_name(v);
 }

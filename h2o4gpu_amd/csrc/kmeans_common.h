@@ -87,12 +87,14 @@ int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
 template <typename T>
 int pick_assign_variant(int requested, int64_t n, int d, int k);
 const char *assign_variant_name(int variant);
-// split (float32 row-stationary kernels only; 0, 6 or 9): run the dot products on the
-// bfloat16 matrix pipe as that many products of bfloat16 parts per feature pair (9: every
-// product exact, 6: the three below 2^-24 of |x||c| left out). assign_split_products()
-// returns the number a launch of this shape uses: 0 where the option does not apply (other
-// kernels, float64, rows padded to fewer than 16 or more than 64 features, staged parts
-// beyond the LDS budget), and such launches run the float32 matrix instructions.
+// split (float32 matrix-core kernels; 0, 6 or 9): run the dot products on the bfloat16
+// matrix pipe as that many products of bfloat16 parts per feature pair (9: every product
+// exact, 6: the three below 2^-24 of |x||c| left out). assign_split_products() returns the
+// number a launch of this shape uses: 0 where the option does not apply (float64, the
+// vector-ALU kernels, rows of fewer than 4 features; row-stationary kernel: rows padded to
+// fewer than 16 or more than 64 features, fused step whose staged parts exceed the LDS
+// budget; tiled kernel: 64 centroids or fewer), and such launches run the float32 matrix
+// instructions.
 template <typename T>
 int assign_split_products(int variant, int split, int64_t n, int d, int k, bool fused);
 
@@ -115,7 +117,7 @@ int launch_assign_accumulate(hipStream_t s, int variant, const T *X, const T *xn
 template <typename T>
 int launch_transform(hipStream_t s, const T *X, const T *xnorm, const T *C,
                      const T *cnorm, T *D, int64_t n, int64_t ldn, int d, int k,
-                     int num_cu);
+                     int num_cu, int split = 0);
 
 // out[i] = sum_j X[i][j]^2, j ascending, no contraction.
 template <typename T>

@@ -1,4 +1,4 @@
-"""The float32 row-stationary kernels with their dot products on the bfloat16 matrix pipe
+"""The float32 matrix-core kernels with their dot products on the bfloat16 matrix pipe
 (option "fp32_split": 9 products of bfloat16 parts per feature pair, every one exact, or 6,
 the three smallest left out) against the CPU oracle and against float64 brute force, through
 the C ABI. The bar is the float32 matrix-core path's own: labels equal the oracle's except
@@ -25,11 +25,18 @@ def blobs(n, d, k, spread=5.0, sigma=1.0, seed=0, scale=1.0):
 SHAPES = [(4096, 32, 256), (5000, 32, 100), (3001, 64, 64), (2000, 24, 33), (1000, 16, 8),
           (900, 30, 70), (700, 9, 40), (513, 63, 20), (2500, 50, 130), (1, 16, 1), (130, 20, 2),
           (3000, 40, 600), (2000, 16, 3000)]
+# the tiled kernel (more than 64 centroids): whole 16-feature stages, a last stage with 1 to
+# 15 features, rows that are not whole vectors, 128- and 256-centroid blocks with partly
+# filled last blocks, integer keys (below 128 features) and the float compare chain
+TILED_SHAPES = [(4096, 32, 256), (1500, 128, 200), (2500, 100, 70), (1200, 256, 130), (900, 300, 257),
+                (1800, 255, 140), (1300, 101, 300), (1100, 127, 1030), (1500, 120, 9000),
+                (1200, 520, 2304), (700, 9, 100), (513, 63, 200), (600, 6, 80), (3, 17, 65)]
 
 
 @pytest.mark.parametrize("split", [9, 6])
-@pytest.mark.parametrize("n,d,k", SHAPES)
-def test_assign_matches_oracle(hip, oracle, n, d, k, split):
+@pytest.mark.parametrize("variant,n,d,k", [("mfma_rowstat",) + c for c in SHAPES] +
+                         [("mfma_tiled",) + c for c in TILED_SHAPES])
+def test_assign_matches_oracle(hip, oracle, variant, n, d, k, split):
     X = blobs(n, d, max(k, 2), seed=n + d + k)
     rng = np.random.default_rng(k)
     if k <= n:
@@ -39,13 +46,13 @@ def test_assign_matches_oracle(hip, oracle, n, d, k, split):
     with hip.Handle(n, d, k, np.float32) as h:
         h.set_data(X)
         h.set_centroids(C)
-        h.set_option("assign", "mfma_rowstat")
+        h.set_option("assign", variant)
         h.set_option("fp32_split", split)
         name = h.assign_variant()
         h.assign()
         got, mind = h.labels(), h.min_distances()
         h.set_option("fp32_split", 0)
-        assert h.assign_variant() == "mfma_rowstat"
+        assert h.assign_variant() == variant
         h.assign()
         plain, pmind = h.labels(), h.min_distances()
     want, wmind = oracle.assign(X, C, return_mindist=True)
@@ -53,13 +60,57 @@ def test_assign_matches_oracle(hip, oracle, n, d, k, split):
     scale = (X.astype(np.float64) ** 2).sum(1).max() + (C.astype(np.float64) ** 2).sum(1).max()
     eps = np.finfo(np.float32).eps
     assert np.max(np.abs(mind.astype(np.float64) - wmind)) <= (4 * np.sqrt(d) + 40) * eps * scale
-    assert name == "mfma_rowstat_bf16x%d" % split
-    print("split %d n=%d d=%d k=%d: %s; %d labels differ from the float32 instructions'" %
-          (split, n, d, k, rep, int((got != plain).sum())))
+    assert name == "%s_bf16x%d" % (variant, split)
+    print("%s split %d n=%d d=%d k=%d: %s; %d labels differ from the float32 instructions'" %
+          (variant, split, n, d, k, rep, int((got != plain).sum())))
+
+
+def test_shapes_the_option_leaves_alone(hip):
+    """Rows of fewer than 4 features, 64 centroids or fewer in the tiled kernel, rows padded to
+    128 features in the row-stationary kernel, the small-model kernels: the float32
+    instructions (or the vector ALU) run, and the results are the option-free ones bit for bit."""
+    for n, d, k, variant, name in [(3000, 3, 100, "mfma_tiled", "mfma_tiled"), (3000, 40, 50, "mfma_tiled", "mfma_tiled"),
+                                   (3000, 100, 90, "mfma_rowstat", "mfma_rowstat"), (3000, 20, 10, "auto", "valu")]:
+        X = blobs(n, d, k, seed=n + d)
+        C = np.ascontiguousarray(X[:k])
+        out = []
+        for split in (0, 6):
+            with hip.Handle(n, d, k, np.float32) as h:
+                h.set_data(X)
+                h.set_centroids(C)
+                h.set_option("assign", variant)
+                h.set_option("fp32_split", split)
+                assert h.assign_variant() == name
+                h.assign()
+                out.append((h.labels(), h.min_distances()))
+        assert np.array_equal(out[0][0], out[1][0]) and np.array_equal(out[0][1], out[1][1])
 
 
 @pytest.mark.parametrize("split", [9, 6])
-def test_distances_are_as_close_to_float64_as_the_float32_instructions(hip, split):
+@pytest.mark.parametrize("n,d,k", [(3000, 100, 300), (1000, 784, 4096), (2500, 37, 130), (129, 16, 65)])
+def test_transform_matches_oracle(hip, oracle, n, d, k, split):
+    X = blobs(n, d, 20, seed=k)
+    rng = np.random.default_rng(d)
+    C = np.ascontiguousarray((X[rng.choice(n, size=k)] + 0.5 * rng.standard_normal((k, d))).astype(np.float32))
+    with hip.Handle(n, d, k, np.float32) as h:
+        h.set_data(X)
+        h.set_centroids(C)
+        h.set_option("fp32_split", split)
+        D = h.transform(X)
+        h.set_option("fp32_split", 0)
+        D0 = h.transform(X)
+    want = oracle.distances(X, C)
+    scale = (X.astype(np.float64) ** 2).sum(1).max() + (C.astype(np.float64) ** 2).sum(1).max()
+    eps = np.finfo(np.float32).eps
+    bound = (4 * np.sqrt(d) + 40) * eps * scale
+    assert np.max(np.abs(D.astype(np.float64) - want)) <= bound
+    assert np.max(np.abs(D0.astype(np.float64) - want)) <= bound
+    assert not np.array_equal(D, D0)  # (the parts did run: same values to rounding, not bit for bit)
+
+
+@pytest.mark.parametrize("variant", ["mfma_rowstat", "mfma_tiled"])
+@pytest.mark.parametrize("split", [9, 6])
+def test_distances_are_as_close_to_float64_as_the_float32_instructions(hip, split, variant):
     """Minimum distances of both paths against float64 brute force, in units of the rounding
     of (xx + cc). The keys the argmin compares drop four mantissa bits on both paths, so the
     exact-compare option is used for the float32 side and the split side is given twice its
@@ -76,7 +127,7 @@ def test_distances_are_as_close_to_float64_as_the_float32_instructions(hip, spli
         with hip.Handle(n, d, k, np.float32) as h:
             h.set_data(X)
             h.set_centroids(C)
-            h.set_option("assign", "mfma_rowstat")
+            h.set_option("assign", variant)
             for o, v in opts.items():
                 h.set_option(o, v)
             h.assign()
@@ -162,29 +213,33 @@ def test_option_values(hip):
 
 
 @pytest.mark.timeout(900)
-@pytest.mark.parametrize("split", [9, 6])
-@pytest.mark.parametrize("name,e2e_iters", [("C3", 6), ("C2", 20)])
-def test_full_benchmark_shape(hip, oracle, name, e2e_iters, split):
-    """10M x 32, k = 256 and 1M x 64, k = 64 at full size with the option on: one Lloyd step
-    on all rows beside the oracle at the start and at the fitted centroids, and a fixed number
-    of iterations end to end, to the same bars as the float32 instructions' full-size test."""
+@pytest.mark.parametrize("name,e2e_iters,fit_iters,split", [("C3", 6, 20, 9), ("C3", 6, 20, 6), ("C2", 20, 20, 9),
+                                                            ("C2", 20, 20, 6), ("C4", 2, 4, 6), ("C5", 1, 2, 6)])
+def test_full_benchmark_shape(hip, oracle, name, e2e_iters, fit_iters, split):
+    """The float32 benchmark shapes that run on the matrix cores, at full size with the option
+    on: one Lloyd step on all rows beside the oracle at the start and at the fitted centroids,
+    and a fixed number of iterations end to end, to the same bars as the float32 instructions'
+    full-size test. 500k x 784, k = 4096 also transforms its 100,000 held-out rows."""
     from h2o4gpu_amd import datasets
-    from test_gpu_configs import _end_to_end_all_rows, _lockstep_all_rows
+    from test_gpu_configs import _end_to_end_all_rows, _lockstep_all_rows, _start, _transform_check
     X, k, _ = datasets.make(name, 1.0, np.float32)
     n, d = X.shape
-    C0 = datasets.seeded_row_init(X, k, datasets.SHAPES[name][3])
     tag = "%s float32 bf16x%d" % (name, split)
     with hip.Handle(n, d, k, np.float32) as h:
         h.set_data(X)
+        C0 = _start(name, X, k, h)
         h.set_option("fp32_split", split)
-        assert h.assign_variant() == "mfma_rowstat_bf16x%d" % split
+        assert h.assign_variant() == ("mfma_rowstat_bf16x%d" if name in ("C2", "C3") else "mfma_tiled_bf16x%d") % split
         start = _lockstep_all_rows(hip, oracle, h, X, C0, np.float32, tag + " start")
         h.set_centroids(C0)
-        h.fit(20, 0.0)
+        h.fit(fit_iters, 0.0)
         C, L = h.centroids(), h.labels()
         h.set_centroids(C0)
-        h.fit(20, 0.0)
+        h.fit(fit_iters, 0.0)
         assert np.array_equal(h.centroids(), C) and np.array_equal(h.labels(), L), "fit does not repeat"
         fitted = _lockstep_all_rows(hip, oracle, h, X, C, np.float32, tag + " fitted")
         e2e = _end_to_end_all_rows(hip, oracle, h, X, C0, np.float32, e2e_iters, tag)
+        if name == "C5":
+            h.set_centroids(C)
+            _transform_check(h, C)
     print("full shape %s: start %s\nfitted %s\nend to end %s" % (tag, start, fitted, e2e))
