@@ -24,6 +24,7 @@ from h2o4gpu_amd.libs import kmeans_hip  # noqa: E402
 
 PEAK_HBM_GBPS = 8000.0
 PEAK_MFMA_TFLOPS = {"f32": 157.3, "f64": 78.6}
+PEAK_BF16_TFLOPS = 2500.0  # dense bfloat16 matrix peak (option fp32_split)
 
 WORKLOAD_TEXT = {
     "C1": "Gaussian blobs, seeded-random row start",
@@ -102,7 +103,8 @@ def traffic_child(args):
         h.set_option("fuse", 0)
     if args.exact_argmin:
         h.set_option("exact_argmin", 1)
-    h.set_option("fp32_split", args.fp32_split)
+    if args.fp32_split is not None:
+        h.set_option("fp32_split", args.fp32_split)
     h.iterate(4)
     h.assign()
     h.close()
@@ -202,7 +204,7 @@ def main():
     ap.add_argument("--assign", default="auto", choices=sorted(kmeans_hip.ASSIGN_VARIANTS))
     ap.add_argument("--exact-argmin", action="store_true",
                     help="float32 matrix-core kernels: compare float distances instead of 16-ulp keys")
-    ap.add_argument("--fp32-split", type=int, default=0, choices=[0, 6, 9],
+    ap.add_argument("--fp32-split", type=int, default=None, choices=[0, 6, 9],
                     help="float32 matrix-core kernels: dot products as this many bfloat16 products per "
                          "feature pair on the bfloat16 matrix pipe (9: every product exact)")
     ap.add_argument("--no-fuse", action="store_true",
@@ -233,7 +235,8 @@ def main():
     if not args.no_traffic:
         tail = ["--workload", args.workload, "--scale", str(args.scale), "--dtype", args.dtype,
                 "--assign", args.assign] + (["--no-fuse"] if args.no_fuse else []) + \
-               (["--exact-argmin"] if args.exact_argmin else []) + ["--fp32-split", str(args.fp32_split)]
+               (["--exact-argmin"] if args.exact_argmin else []) + \
+               (["--fp32-split", str(args.fp32_split)] if args.fp32_split is not None else [])
         t0 = time.perf_counter()
         traffic, traffic_details = measure_traffic(tail)
         log("traffic passes: %s in %.1f s" % ("%.4g bytes per launch" % traffic if traffic else
@@ -270,7 +273,8 @@ def main():
         h.set_option("fuse", 0)
     if args.exact_argmin:
         h.set_option("exact_argmin", 1)
-    h.set_option("fp32_split", args.fp32_split)
+    if args.fp32_split is not None:
+        h.set_option("fp32_split", args.fp32_split)
     variant = h.assign_variant()
     log("upload %.3f s (%.1f GB/s incl. pageable staging; first call of the process %.3f s); "
         "assign variant %s" % (h2d_s, n * d * s / h2d_s / 1e9, h2d_first_s, variant))
@@ -300,7 +304,15 @@ def main():
     tflops = flops_per_iter / (assign_ms * 1e-3) / 1e12
     peak = PEAK_MFMA_TFLOPS[args.dtype]
     mfma_bound = variant != "valu"
-    if mfma_bound:
+    if mfma_bound and "_bf16x" in variant:
+        # the option that forms each float32 product from bfloat16 parts: the kernel executes
+        # 6 or 9 times the algorithmic flop, on the bfloat16 matrix pipe, and is priced there
+        products = int(variant[-1])
+        roofline = {"bound": "mfma", "kernel": "%s (%s)" % (dom, variant), "achieved": products * tflops,
+                    "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": products * tflops / PEAK_BF16_TFLOPS,
+                    "traffic": traffic, "algorithmic_tflops": tflops,
+                    "note": "%d bfloat16 products per float32 product, bfloat16 matrix peak" % products}
+    elif mfma_bound:
         roofline = {"bound": "mfma", "kernel": "%s (%s)" % (dom, variant), "achieved": tflops,
                     "peak": peak, "unit": "TFLOP/s", "frac": tflops / peak, "traffic": traffic}
     else:
@@ -333,7 +345,7 @@ def main():
     # the same steps with the float32 dot products on the bfloat16 matrix pipe (an option of
     # the matrix-core kernels, off by default; never part of `value`)
     split_leg = None
-    if args.fp32_split == 0 and args.dtype == "f32" and variant in ("mfma_rowstat", "mfma_tiled"):
+    if args.dtype == "f32" and variant in ("mfma_rowstat", "mfma_tiled"):  # (i.e. the main run was without it)
         h.set_option("fp32_split", 6)
         if h.assign_variant() == variant + "_bf16x6":
             h.set_centroids(C0)

@@ -234,6 +234,15 @@ int h2o4gpu_kmeans_transform_resident(h2o4gpu_kmeans_handle *h, void *d_dist);
  * themselves instead of 16-ulp integer keys (slower, never fused; 0 is the default).
  * "transform_batch_mb" (default 4096) bounds the device buffer transform_host fills per
  * batch of rows; smaller values force more, shorter batches.
+ * "fp32_split" = 9 or 6 (default 0) makes the float32 matrix-core kernels form their dot
+ * products on the bfloat16 matrix pipe: every float is the exact sum of three bfloat16
+ * parts, 9 runs all nine products of the parts (each exact, accumulated in float32), 6
+ * leaves out the three smallest (below one ulp of xx + cc per distance). 1.4 to 1.9 times
+ * faster on matrix-bound shapes, same parity bars; shapes it does not apply to (float64,
+ * k <= 16 && d <= 64, rows of fewer than 4 features, ...) run as without it, and
+ * h2o4gpu_kmeans_assign_variant() names what runs ("mfma_tiled_bf16x6", ...). The
+ * environment variable H2O4GPU_KMEANS_FP32_SPLIT=6|9 sets it for every handle created
+ * afterwards, the reference's four entry points included.
  * Unknown names return EARG. */
 int h2o4gpu_kmeans_set_option(h2o4gpu_kmeans_handle *h, const char *name,
                               int value);
