@@ -980,6 +980,47 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
 // workgroup and come from HBM/MALL every time they are re-read, centroid blocks
 // are shared by all workgroups and hit L2, so for large k the wider centroid
 // block (BCW = 4) halves the expensive traffic.
+// The centroids' bfloat16 parts for the tiled kernel, written as the LDS images it stages:
+// for centroid block cb (bc centroids) and stage st (16 features) a block of bc*16*6 bytes,
+// [32-centroid tile][part][lane group * 32 + centroid] vectors of 8 bfloat16, the lane
+// group's features in the order the row side deals them out (16-byte vectors of the stage in
+// turn: vector 0 and 2 to lane group 0, 1 and 3 to lane group 1). Rows past k and features
+// past d are zero, so the tiled kernel needs no bounds on this operand.
+__global__ void split_centroids_kernel(const float *__restrict__ C, uintx4 *__restrict__ out, int k,
+                                       int d, int bc, int nstage, int nblocks) {
+  const int tiles = bc / 32;
+  const int64_t total = (int64_t)nblocks * nstage * tiles * 64;
+  for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total;
+       e += (int64_t)gridDim.x * blockDim.x) {
+    const int slot = (int)(e & 63);
+    int64_t rest = e >> 6;
+    const int t = (int)(rest % tiles);
+    rest /= tiles;
+    const int st = (int)(rest % nstage);
+    const int cb = (int)(rest / nstage);
+    const int gg = slot >> 5, i = slot & 31;
+    const int c = cb * bc + t * 32 + i;
+    float h[8], m[8], l[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const int f = st * 16 + ((j >> 2) * 2 + gg) * 4 + (j & 3);
+      const float v = (c < k && f < d) ? C[(size_t)c * d + f] : 0.0f;
+      split_bf16x3(v, h[j], m[j], l[j]);
+    }
+    uintx4 ph, pm, pl;
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+      ph[w] = pack_bf16x2(h[2 * w], h[2 * w + 1]);
+      pm[w] = pack_bf16x2(m[2 * w], m[2 * w + 1]);
+      pl[w] = pack_bf16x2(l[2 * w], l[2 * w + 1]);
+    }
+    uintx4 *dst = out + (((size_t)cb * nstage + st) * tiles + t) * 3 * 64 + slot;
+    dst[0] = ph;
+    dst[64] = pm;
+    dst[128] = pl;
+  }
+}
+
 template <typename T, int BCW, bool WIDE = false, int SPLIT = 0>
 struct TiledCfg {
   static constexpr int TPB = 2 * BCW * 64;
@@ -1007,7 +1048,7 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
     const T *__restrict__ X, const T *__restrict__ xnorm,
     const T *__restrict__ C, const T *__restrict__ cnorm,
     int *__restrict__ labels, T *__restrict__ mindist, T *__restrict__ D,
-    int64_t n, int64_t ldn, int d, int k) {
+    int64_t n, int64_t ldn, int d, int k, const uintx4 *__restrict__ Cparts) {
   typedef Mfma<T> M;
   typedef TiledCfg<T, BCW, WIDE, SPLIT> Cfg;
   static_assert(SPLIT == 0 || (sizeof(T) == 4 && VECLOAD && (SPLIT == 6 || SPLIT == 9)),
@@ -1117,6 +1158,11 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
   }
 
   vec_t areg[A_VECS], breg[B_VECS];
+  // SPLIT: the centroid parts come ready-made from Cparts (split_centroids_kernel), one LDS
+  // image of A_BYTES per (centroid block, stage), copied as it lies
+  constexpr int A_PVECS = SPLIT ? A_BYTES / 16 / WG : 1;
+  static_assert(!SPLIT || A_BYTES % (16 * WG) == 0, "whole 16-byte vectors per thread");
+  uintx4 apreg[A_PVECS];
   // Only the last d-step can reach past the feature count: the guards live in a second
   // instance of the loader (tail_tag true) used for that step alone.
   auto gload = [&](int c0, int st, auto tail_tag) {
@@ -1146,10 +1192,16 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
       }
       return v;
     };
-    const T *cbase = C + (size_t)(c0 + rr0) * d;
+    if constexpr (SPLIT != 0) {
+      const uintx4 *cp = Cparts + ((size_t)(c0 / BC) * nstage + st) * (A_BYTES / 16) + tid;
 #pragma unroll
-    for (int q = 0; q < A_VECS; q++)
-      areg[q] = fetch(cbase + (size_t)q * ROWS_PER_PASS * d, true);
+      for (int q = 0; q < A_PVECS; q++) apreg[q] = cp[q * WG];
+    } else {
+      const T *cbase = C + (size_t)(c0 + rr0) * d;
+#pragma unroll
+      for (int q = 0; q < A_VECS; q++)
+        areg[q] = fetch(cbase + (size_t)q * ROWS_PER_PASS * d, true);
+    }
 #pragma unroll
     for (int q = 0; q < B_VECS; q++) breg[q] = fetch(xrow[q], false);
   };
@@ -1175,7 +1227,8 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
   auto lstore = [&](int buf) {
     if constexpr (SPLIT != 0) {
 #pragma unroll
-      for (int q = 0; q < A_VECS; q++) store_parts(Ab + buf * A_BYTES + lds_off[q], areg[q]);
+      for (int q = 0; q < A_PVECS; q++)
+        reinterpret_cast<uintx4 *>(Ab + buf * A_BYTES)[q * WG + tid] = apreg[q];
 #pragma unroll
       for (int q = 0; q < B_VECS; q++) store_parts(Bb + buf * B_BYTES + lds_off[q], breg[q]);
       return;
@@ -1762,9 +1815,18 @@ int launch_assign_accumulate(hipStream_t s, int variant, const T *X, const T *xn
 template <typename T, int MODE, int BCW, bool WIDE = false, int SPLIT = 0>
 static int launch_tiled_bcw(hipStream_t s, const T *X, const T *xnorm, const T *C,
                             const T *cnorm, int *labels, T *mindist, T *D, int64_t n,
-                            int64_t ldn, int d, int k, bool exact) {
+                            int64_t ldn, int d, int k, bool exact, void *cparts = nullptr) {
   typedef TiledCfg<T, BCW, WIDE, SPLIT> Cfg;
   const size_t lds = Cfg::LDS_BYTES;
+  if constexpr (SPLIT != 0) {
+    // the centroids' parts, once per launch, as the LDS images the kernel stages
+    if (!cparts) return H2O4GPU_KMEANS_EARG;
+    const int nstage = (d + Cfg::BK - 1) / Cfg::BK, nblocks = (k + Cfg::BC - 1) / Cfg::BC;
+    const int64_t items = (int64_t)nblocks * nstage * (Cfg::BC / 32) * 64;
+    hipLaunchKernelGGL(split_centroids_kernel, dim3((unsigned)std::min<int64_t>((items + 255) / 256, 4096)),
+                       dim3(256), 0, s, reinterpret_cast<const float *>(C), static_cast<uintx4 *>(cparts), k,
+                       d, Cfg::BC, nstage, nblocks);
+  }
   const int64_t row_tiles = (n + Cfg::BR - 1) / Cfg::BR;
   const int64_t tiles = MODE == 1 ? row_tiles * ((k + Cfg::BC - 1) / Cfg::BC) : row_tiles;
   if (tiles > 2147483647ll) return H2O4GPU_KMEANS_EARG;
@@ -1776,7 +1838,7 @@ static int launch_tiled_bcw(hipStream_t s, const T *X, const T *xnorm, const T *
     auto kern = assign_tiled_kernel<T, MODE, VEC, TAIL, BCW, EXACT, WIDE, SPLIT>;            \
     KM_TRY(ensure_dynamic_lds(reinterpret_cast<const void *>(kern), lds));                   \
     hipLaunchKernelGGL(kern, grid, dim3(Cfg::TPB), lds, s, X, xnorm, C, cnorm, labels,       \
-                       mindist, D, n, ldn, d, k);                                            \
+                       mindist, D, n, ldn, d, k, static_cast<const uintx4 *>(cparts));       \
   } while (0)
   // From 128 features on the float32 argmin compares the distances themselves: the
   // epilogue is then about one per cent of the matrix work (2M x 256, k = 1024: 8.30 ->
@@ -1812,22 +1874,34 @@ static int tiled_split(int split, int d, int k) {
   return split;
 }
 
+// Bytes of device scratch the tiled kernel needs for the centroids' parts (0: the option
+// does not apply to the shape).
+template <typename T>
+size_t tiled_split_scratch_bytes(int split, int d, int k) {
+  if (tiled_split<T>(split, d, k) == 0) return 0;
+  const int bc = k > 128 ? 256 : 128;
+  return (size_t)((k + bc - 1) / bc) * bc * ((d + 15) / 16) * 16 * 6;
+}
+template size_t tiled_split_scratch_bytes<float>(int, int, int);
+template size_t tiled_split_scratch_bytes<double>(int, int, int);
+
 template <typename T, int MODE>
 static int launch_tiled(hipStream_t s, const T *X, const T *xnorm, const T *C,
                         const T *cnorm, int *labels, T *mindist, T *D, int64_t n,
-                        int64_t ldn, int d, int k, bool exact = false, int split = 0) {
+                        int64_t ldn, int d, int k, bool exact = false, int split = 0,
+                        void *split_scratch = nullptr) {
   if constexpr (sizeof(T) == 4) {
     // (with the parts the 256-centroid block is ahead whenever it has the centroids to fill
     // it: 2M x 256, k = 1024 5.87 -> 5.37 ms, 500k x 784, k = 4096 14.96 -> 13.52 ms)
     const bool wide = k > 128;
-    switch (tiled_split<T>(split, d, k)) {
+    switch (split_scratch ? tiled_split<T>(split, d, k) : 0) {
 #define KM_TILED_SPLIT(SP)                                                                         \
   case SP:                                                                                         \
     if (wide)                                                                                      \
       return launch_tiled_bcw<T, MODE, 2, true, SP>(s, X, xnorm, C, cnorm, labels, mindist, D, n,  \
-                                                    ldn, d, k, exact);                             \
+                                                    ldn, d, k, exact, split_scratch);              \
     return launch_tiled_bcw<T, MODE, 2, false, SP>(s, X, xnorm, C, cnorm, labels, mindist, D, n,   \
-                                                   ldn, d, k, exact)
+                                                   ldn, d, k, exact, split_scratch)
       KM_TILED_SPLIT(6);
       KM_TILED_SPLIT(9);
 #undef KM_TILED_SPLIT
@@ -1853,7 +1927,8 @@ static int launch_tiled(hipStream_t s, const T *X, const T *xnorm, const T *C,
 template <typename T>
 int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
                   const T *C, const T *cnorm, int *labels, T *mindist, int64_t n,
-                  int d, int k, int num_cu, int *used, bool exact, StackShape st, int split) {
+                  int d, int k, int num_cu, int *used, bool exact, StackShape st, int split,
+                  void *split_scratch) {
   if (n <= 0) return 0;
   if (d < 1 || k < 1) return H2O4GPU_KMEANS_EARG;
   const int v = pick_assign_variant<T>(variant, n, d, k);
@@ -1881,7 +1956,8 @@ int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
       const int kc = rowstat_chunk<T>(d, k, split_ok ? split : 0);
       if (kc < k && !mindist) {  // merging chunks needs the running minimum in memory
         if (used) *used = ASSIGN_TILED;
-        return launch_tiled<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k, exact, split);
+        return launch_tiled<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k, exact, split,
+                                  split_scratch);
       }
       for (int c0 = 0; c0 < k; c0 += kc)
         KM_TRY((RowstatDispatch<T, false>::run(s, X, xnorm, C + (size_t)c0 * d, cnorm + c0, labels,
@@ -1891,7 +1967,8 @@ int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
       return 0;
     }
     case ASSIGN_TILED:
-      return launch_tiled<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k, exact, split);
+      return launch_tiled<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k, exact, split,
+                                split_scratch);
   }
   return H2O4GPU_KMEANS_EARG;
 }
@@ -1899,7 +1976,7 @@ int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
 template <typename T>
 int launch_transform(hipStream_t s, const T *X, const T *xnorm, const T *C,
                      const T *cnorm, T *D, int64_t n, int64_t ldn, int d, int k,
-                     int num_cu, int split) {
+                     int num_cu, int split, void *split_scratch) {
   if (n <= 0) return 0;
   if (d < 1 || k < 1) return H2O4GPU_KMEANS_EARG;
   if (k <= 16 && d <= 64) {
@@ -1911,7 +1988,8 @@ int launch_transform(hipStream_t s, const T *X, const T *xnorm, const T *C,
                                          nullptr, nullptr, nullptr, D, ldn);
     return launch_valu<T, 1>(s, X, xnorm, C, cnorm, nullptr, nullptr, D, n, ldn, d, k);
   }
-  return launch_tiled<T, 1>(s, X, xnorm, C, cnorm, nullptr, nullptr, D, n, ldn, d, k, false, split);
+  return launch_tiled<T, 1>(s, X, xnorm, C, cnorm, nullptr, nullptr, D, n, ldn, d, k, false, split,
+                            split_scratch);
 }
 
 template <typename T>
@@ -1942,15 +2020,15 @@ template int pick_assign_variant<float>(int, int64_t, int, int);
 template int pick_assign_variant<double>(int, int64_t, int, int);
 template int launch_assign<float>(hipStream_t, int, const float *, const float *,
                                   const float *, const float *, int *, float *,
-                                  int64_t, int, int, int, int *, bool, StackShape, int);
+                                  int64_t, int, int, int, int *, bool, StackShape, int, void *);
 template int launch_assign<double>(hipStream_t, int, const double *, const double *,
                                    const double *, const double *, int *, double *,
-                                   int64_t, int, int, int, int *, bool, StackShape, int);
+                                   int64_t, int, int, int, int *, bool, StackShape, int, void *);
 template int launch_transform<float>(hipStream_t, const float *, const float *,
                                      const float *, const float *, float *, int64_t,
-                                     int64_t, int, int, int, int);
+                                     int64_t, int, int, int, int, void *);
 template int launch_transform<double>(hipStream_t, const double *, const double *,
                                       const double *, const double *, double *,
-                                      int64_t, int64_t, int, int, int, int);
+                                      int64_t, int64_t, int, int, int, int, void *);
 
 }  // namespace kmhip

@@ -522,6 +522,26 @@ struct Engine : h2o4gpu_kmeans_handle {
   T *kpp_dcc = nullptr;     // [k] distances newest centre -> earlier centres
   bool have_data = false, have_centroids = false, have_mindist = false;
   int *d_frozen = nullptr;  // [sets] flags of a stacked handle's sets that have converged
+  // (option fp32_split, tiled kernel) the centroids' bfloat16 parts, rewritten by every launch
+  unsigned char *d_split = nullptr;
+  size_t split_bytes = 0;
+  // The scratch a launch with the option needs, allocated on first use (an in-flight launch
+  // may still read the old one: the stream is drained before it is replaced); null when the
+  // option is off or does not apply, and when the allocation fails (the launch then runs the
+  // float32 instructions).
+  void *split_scratch() {
+    const size_t need = opt_split ? tiled_split_scratch_bytes<T>(opt_split, d, k) : 0;
+    if (need == 0) return nullptr;
+    if (need > split_bytes) {
+      (void)hipStreamSynchronize(stream);
+      if (d_split) (void)hipFree(d_split);
+      d_split = nullptr;
+      split_bytes = 0;
+      if (dalloc(&d_split, need) != 0) return nullptr;
+      split_bytes = need;
+    }
+    return d_split;
+  }
   StackShape shape() const {
     StackShape st;
     st.sets = sets;
@@ -628,7 +648,7 @@ struct Engine : h2o4gpu_kmeans_handle {
     void *ptrs[] = {xnorm,  C[0],    C[1],           cnorm,  labels,       mindist,
                     counts, psums,   pcounts,        shift_partials, shift2,
                     sum_partials, kpp_bsums, kpp_rows, kpp_dcc, order, order_label, bucket_offsets,
-                    bucket_hist, bucket_seg, bucket_total, bucket_partials, d_frozen};
+                    bucket_hist, bucket_seg, bucket_total, bucket_partials, d_frozen, d_split};
     for (void *p : ptrs)
       if (p) (void)hipFree(p);
     if (stream) (void)hipStreamDestroy(stream);
@@ -974,7 +994,7 @@ struct Engine : h2o4gpu_kmeans_handle {
     KM_TRY(ensure_cnorm());
     PROFILED("assign", launch_assign<T>(stream, opt_assign, X, xnorm, C[cur], cnorm,
                                         labels, mindist, n, d, k, num_cu, &last_variant,
-                                        opt_exact != 0, shape(), opt_split));
+                                        opt_exact != 0, shape(), opt_split, split_scratch()));
     have_mindist = true;
     return 0;
   }
@@ -1246,7 +1266,7 @@ struct Engine : h2o4gpu_kmeans_handle {
     PROFILED("row_norms", launch_row_norms<T>(stream, dX, dxn, (int64_t)rows, d));
     PROFILED("assign", launch_assign<T>(stream, opt_assign, dX, dxn, C[cur], cnorm, dl, dmin,
                                         (int64_t)rows, d, k, num_cu, &last_variant,
-                                        opt_exact != 0));
+                                        opt_exact != 0, StackShape(), opt_split, split_scratch()));
     KM_TRY(download_rows(dev, stream, out, dl, rows * sizeof(int)));
     KM_HIP_TRY(hipStreamSynchronize(stream));
     return 0;
@@ -1285,7 +1305,7 @@ struct Engine : h2o4gpu_kmeans_handle {
     PROFILED("row_norms", launch_row_norms<T>(stream, dX, dxn, (int64_t)cur_rows, d));
     PROFILED("transform", launch_transform<T>(stream, dX, dxn, C[cur], cnorm, dD,
                                               (int64_t)cur_rows, (int64_t)cur_rows, d, k, num_cu,
-                                              opt_split));
+                                              opt_split, split_scratch()));
     T *dst = static_cast<T *>(hD) + lo;
     if (cur_rows == rows)  // a single batch is one contiguous [k][rows] block
       KM_TRY(download_rows(dev, stream, dst, dD, (size_t)k * rows * sizeof(T)));
@@ -1300,7 +1320,8 @@ struct Engine : h2o4gpu_kmeans_handle {
     if (!have_data || !have_centroids || !d_dist || sets > 1) return H2O4GPU_KMEANS_ESTATE;
     KM_TRY(ensure_cnorm());
     PROFILED("transform", launch_transform<T>(stream, X, xnorm, C[cur], cnorm,
-                                              static_cast<T *>(d_dist), n, n, d, k, num_cu, opt_split));
+                                              static_cast<T *>(d_dist), n, n, d, k, num_cu, opt_split,
+                                              split_scratch()));
     KM_HIP_TRY(hipStreamSynchronize(stream));
     return 0;
   }

@@ -83,7 +83,7 @@ template <typename T>
 int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
                   const T *C, const T *cnorm, int *labels, T *mindist,
                   int64_t n, int d, int k, int num_cu, int *used, bool exact = false,
-                  StackShape st = StackShape(), int split = 0);
+                  StackShape st = StackShape(), int split = 0, void *split_scratch = nullptr);
 template <typename T>
 int pick_assign_variant(int requested, int64_t n, int d, int k);
 const char *assign_variant_name(int variant);
@@ -97,6 +97,11 @@ const char *assign_variant_name(int variant);
 // instructions.
 template <typename T>
 int assign_split_products(int variant, int split, int64_t n, int d, int k, bool fused);
+// The tiled kernel takes the centroids' parts from device scratch of this many bytes
+// (split_scratch of launch_assign / launch_transform), written anew by every launch; without
+// the scratch (or with 0 bytes needed) it runs the float32 instructions.
+template <typename T>
+size_t tiled_split_scratch_bytes(int split, int d, int k);
 
 // Fused assign + accumulate (row-stationary MFMA shapes and the small VALU shapes): labels/mindist as
 // launch_assign, plus per-workgroup partial sums psums[slot][k][d] and counts
@@ -117,7 +122,7 @@ int launch_assign_accumulate(hipStream_t s, int variant, const T *X, const T *xn
 template <typename T>
 int launch_transform(hipStream_t s, const T *X, const T *xnorm, const T *C,
                      const T *cnorm, T *D, int64_t n, int64_t ldn, int d, int k,
-                     int num_cu, int split = 0);
+                     int num_cu, int split = 0, void *split_scratch = nullptr);
 
 // out[i] = sum_j X[i][j]^2, j ascending, no contraction.
 template <typename T>
