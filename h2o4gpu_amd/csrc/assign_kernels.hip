@@ -1876,10 +1876,13 @@ static int tiled_split(int split, int d, int k) {
 
 // Bytes of device scratch the tiled kernel needs for the centroids' parts (0: the option
 // does not apply to the shape).
+// (with the parts the 256-centroid block is ahead whenever it has the centroids to fill it:
+// 2M x 256, k = 1024 5.87 -> 5.37 ms, 500k x 784, k = 4096 14.96 -> 13.52 ms)
+static bool tiled_split_wide(int k) { return k > 128; }
 template <typename T>
 size_t tiled_split_scratch_bytes(int split, int d, int k) {
   if (tiled_split<T>(split, d, k) == 0) return 0;
-  const int bc = k > 128 ? 256 : 128;
+  const int bc = tiled_split_wide(k) ? 256 : 128;
   return (size_t)((k + bc - 1) / bc) * bc * ((d + 15) / 16) * 16 * 6;
 }
 template size_t tiled_split_scratch_bytes<float>(int, int, int);
@@ -1889,12 +1892,12 @@ template <typename T, int MODE>
 static int launch_tiled(hipStream_t s, const T *X, const T *xnorm, const T *C,
                         const T *cnorm, int *labels, T *mindist, T *D, int64_t n,
                         int64_t ldn, int d, int k, bool exact = false, int split = 0,
-                        void *split_scratch = nullptr) {
+                        SplitScratch scratch = SplitScratch()) {
   if constexpr (sizeof(T) == 4) {
-    // (with the parts the 256-centroid block is ahead whenever it has the centroids to fill
-    // it: 2M x 256, k = 1024 5.87 -> 5.37 ms, 500k x 784, k = 4096 14.96 -> 13.52 ms)
-    const bool wide = k > 128;
-    switch (split_scratch ? tiled_split<T>(split, d, k) : 0) {
+    const bool wide = tiled_split_wide(k);
+    const size_t need = tiled_split_scratch_bytes<T>(split, d, k);
+    void *split_scratch = scratch.ptr;
+    switch (need > 0 && scratch.ptr && scratch.bytes >= need ? split : 0) {
 #define KM_TILED_SPLIT(SP)                                                                         \
   case SP:                                                                                         \
     if (wide)                                                                                      \
@@ -1928,7 +1931,7 @@ template <typename T>
 int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
                   const T *C, const T *cnorm, int *labels, T *mindist, int64_t n,
                   int d, int k, int num_cu, int *used, bool exact, StackShape st, int split,
-                  void *split_scratch) {
+                  SplitScratch split_scratch) {
   if (n <= 0) return 0;
   if (d < 1 || k < 1) return H2O4GPU_KMEANS_EARG;
   const int v = pick_assign_variant<T>(variant, n, d, k);
@@ -1976,7 +1979,7 @@ int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
 template <typename T>
 int launch_transform(hipStream_t s, const T *X, const T *xnorm, const T *C,
                      const T *cnorm, T *D, int64_t n, int64_t ldn, int d, int k,
-                     int num_cu, int split, void *split_scratch) {
+                     int num_cu, int split, SplitScratch split_scratch) {
   if (n <= 0) return 0;
   if (d < 1 || k < 1) return H2O4GPU_KMEANS_EARG;
   if (k <= 16 && d <= 64) {
@@ -2020,15 +2023,15 @@ template int pick_assign_variant<float>(int, int64_t, int, int);
 template int pick_assign_variant<double>(int, int64_t, int, int);
 template int launch_assign<float>(hipStream_t, int, const float *, const float *,
                                   const float *, const float *, int *, float *,
-                                  int64_t, int, int, int, int *, bool, StackShape, int, void *);
+                                  int64_t, int, int, int, int *, bool, StackShape, int, SplitScratch);
 template int launch_assign<double>(hipStream_t, int, const double *, const double *,
                                    const double *, const double *, int *, double *,
-                                   int64_t, int, int, int, int *, bool, StackShape, int, void *);
+                                   int64_t, int, int, int, int *, bool, StackShape, int, SplitScratch);
 template int launch_transform<float>(hipStream_t, const float *, const float *,
                                      const float *, const float *, float *, int64_t,
-                                     int64_t, int, int, int, int, void *);
+                                     int64_t, int, int, int, int, SplitScratch);
 template int launch_transform<double>(hipStream_t, const double *, const double *,
                                       const double *, const double *, double *,
-                                      int64_t, int64_t, int, int, int, int, void *);
+                                      int64_t, int64_t, int, int, int, int, SplitScratch);
 
 }  // namespace kmhip

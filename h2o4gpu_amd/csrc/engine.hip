@@ -529,18 +529,21 @@ struct Engine : h2o4gpu_kmeans_handle {
   // may still read the old one: the stream is drained before it is replaced); null when the
   // option is off or does not apply, and when the allocation fails (the launch then runs the
   // float32 instructions).
-  void *split_scratch() {
+  SplitScratch split_scratch() {
+    SplitScratch sc;
     const size_t need = opt_split ? tiled_split_scratch_bytes<T>(opt_split, d, k) : 0;
-    if (need == 0) return nullptr;
+    if (need == 0) return sc;
     if (need > split_bytes) {
       (void)hipStreamSynchronize(stream);
       if (d_split) (void)hipFree(d_split);
       d_split = nullptr;
       split_bytes = 0;
-      if (dalloc(&d_split, need) != 0) return nullptr;
+      if (dalloc(&d_split, need) != 0) return sc;
       split_bytes = need;
     }
-    return d_split;
+    sc.ptr = d_split;
+    sc.bytes = split_bytes;
+    return sc;
   }
   StackShape shape() const {
     StackShape st;

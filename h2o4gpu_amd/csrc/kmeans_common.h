@@ -73,6 +73,14 @@ struct StackShape {
   int kset = 0;
 };
 
+// Device memory a launch with the bfloat16-parts option may write the centroids' parts to
+// (tiled kernel only; tiled_split_scratch_bytes() says how much a shape needs). A launch that
+// is given less runs the float32 instructions.
+struct SplitScratch {
+  void *ptr = nullptr;
+  size_t bytes = 0;
+};
+
 // Fused distance + argmin. labels[i] = argmin_c |(xx_i + cc_c) - 2 x_i.c_c|,
 // strict '<', lowest index wins, -1 when no distance is below FLT_MAX.
 // mindist (nullable) receives the minimum. Returns the variant actually used
@@ -83,7 +91,7 @@ template <typename T>
 int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
                   const T *C, const T *cnorm, int *labels, T *mindist,
                   int64_t n, int d, int k, int num_cu, int *used, bool exact = false,
-                  StackShape st = StackShape(), int split = 0, void *split_scratch = nullptr);
+                  StackShape st = StackShape(), int split = 0, SplitScratch split_scratch = SplitScratch());
 template <typename T>
 int pick_assign_variant(int requested, int64_t n, int d, int k);
 const char *assign_variant_name(int variant);
@@ -122,7 +130,7 @@ int launch_assign_accumulate(hipStream_t s, int variant, const T *X, const T *xn
 template <typename T>
 int launch_transform(hipStream_t s, const T *X, const T *xnorm, const T *C,
                      const T *cnorm, T *D, int64_t n, int64_t ldn, int d, int k,
-                     int num_cu, int split = 0, void *split_scratch = nullptr);
+                     int num_cu, int split = 0, SplitScratch split_scratch = SplitScratch());
 
 // out[i] = sum_j X[i][j]^2, j ascending, no contraction.
 template <typename T>
