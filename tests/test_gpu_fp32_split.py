@@ -243,3 +243,41 @@ def test_full_benchmark_shape(hip, oracle, name, e2e_iters, fit_iters, split):
             h.set_centroids(C)
             _transform_check(h, C)
     print("full shape %s: start %s\nfitted %s\nend to end %s" % (tag, start, fitted, e2e))
+
+
+def test_environment_variable_reaches_the_reference_entry_points(hip, oracle, monkeypatch):
+    """make_ptr_float_kmeans has no argument for the option: H2O4GPU_KMEANS_FP32_SPLIT sets it
+    for every handle created afterwards."""
+    from h2o4gpu_amd.libs import ch2o4gpu_gpu
+    n, d, k = 40000, 32, 64
+    X = blobs(n, d, k, spread=20.0, seed=4)
+    C0 = np.ascontiguousarray(X[np.random.default_rng(2).choice(n, size=k, replace=False)])
+
+    def fit():
+        centres = np.zeros(k * d, np.float32)
+        labels = np.zeros(n, np.int32)
+        rc = ch2o4gpu_gpu.make_ptr_float_kmeans(0, 0, 1, 0, 1, n, d, k, 5, 2, 0.0, X.flatten(), C0.flatten(),
+                                                centres, labels)
+        assert rc == 0
+        return centres.reshape(k, d), labels
+
+    plain = fit()
+    monkeypatch.setenv("H2O4GPU_KMEANS_FP32_SPLIT", "6")
+    with hip.Handle(n, d, k, np.float32) as h:
+        assert h.assign_variant() == "mfma_rowstat_bf16x6"
+    split = fit()
+    monkeypatch.setenv("H2O4GPU_KMEANS_FP32_SPLIT", "7")  # not a value of the option: ignored
+    with hip.Handle(n, d, k, np.float32) as h:
+        assert h.assign_variant() == "mfma_rowstat"
+    monkeypatch.delenv("H2O4GPU_KMEANS_FP32_SPLIT")
+    assert not np.array_equal(plain[0], split[0])  # another summation order: not bit for bit
+    wC, wL, _, _ = oracle.lloyd(X, C0, 5, 0.0, threads=4)
+    X64 = X.astype(np.float64)
+    want = ((X64 - wC.astype(np.float64)[wL]) ** 2).sum()
+    for C, L in (plain, split):
+        if np.array_equal(L, wL):
+            assert_centroids_close(C, wC, np.float32)
+        # (a start on random rows splits blobs: near-tie rows that flip move the trajectory,
+        # the objective stays)
+        got = ((X64 - C.astype(np.float64)[L]) ** 2).sum()
+        assert abs(got - want) <= 1e-4 * want
