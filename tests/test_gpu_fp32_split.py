@@ -281,3 +281,62 @@ def test_environment_variable_reaches_the_reference_entry_points(hip, oracle, mo
         # the objective stays)
         got = ((X64 - C.astype(np.float64)[L]) ** 2).sum()
         assert abs(got - want) <= 1e-4 * want
+
+
+@pytest.mark.parametrize("variant", ["mfma_rowstat", "mfma_tiled"])
+def test_non_finite_rows_and_centroids(hip, oracle, variant):
+    """The parts of an infinity or a NaN are not finite either: such rows get label -1, such
+    centroids are never chosen (kmeans_labels.h:360-377), their neighbours are unaffected."""
+    n, d, k = 2048, 32, 80
+    X = blobs(n, d, k, seed=99)
+    C = np.ascontiguousarray(X[np.random.default_rng(1).choice(n, size=k, replace=False)])
+    X[5, 3] = np.nan
+    X[70, :] = np.nan
+    X[130, 0] = np.inf
+    X[131, 7] = -np.inf
+    X[1999, d - 1] = np.nan
+    C[4, 2] = np.nan
+    C[17, :] = np.inf
+    bad_rows = [5, 70, 130, 131, 1999]
+    with hip.Handle(n, d, k, np.float32) as h:
+        h.set_data(X)
+        h.set_centroids(C)
+        h.set_option("assign", variant)
+        h.set_option("fp32_split", 6)
+        assert h.assign_variant() == variant + "_bf16x6"
+        h.assign()
+        got = h.labels()
+        h.update()
+        counts = h.counts()
+    want = oracle.assign(X, C)
+    assert np.all(want[bad_rows] == -1) and np.all(got[bad_rows] == -1)
+    assert not np.any(np.isin(got, [4, 17]))
+    good = np.ones(n, bool)
+    good[bad_rows] = False
+    remap = np.delete(np.arange(k), [4, 17])
+    inv = {int(c): i for i, c in enumerate(remap)}
+    g2 = np.array([inv[int(c)] for c in got[good]], np.int32)
+    w2 = np.array([inv[int(c)] for c in want[good]], np.int32)
+    label_report(oracle, np.ascontiguousarray(X[good]), np.ascontiguousarray(np.delete(C, [4, 17], axis=0)), g2, w2)
+    assert counts.sum() == n - len(bad_rows)
+
+
+@pytest.mark.parametrize("variant", ["mfma_rowstat", "mfma_tiled"])
+@pytest.mark.parametrize("scale", [1e15, 1e-15])
+def test_large_and_small_magnitudes(hip, oracle, variant, scale):
+    """bfloat16 has float32's exponent range: data scaled by 1e15 (squares near 1e32) and by
+    1e-15 (squares near 1e-28) split exactly and label as unscaled data does."""
+    n, d, k = 6000, 32, 70
+    X = blobs(n, d, k, seed=8, scale=scale)
+    C = np.ascontiguousarray(X[np.random.default_rng(5).choice(n, size=k, replace=False)])
+    with hip.Handle(n, d, k, np.float32) as h:
+        h.set_data(X)
+        h.set_centroids(C)
+        h.set_option("assign", variant)
+        h.set_option("fp32_split", 6)
+        h.assign()
+        got, mind = h.labels(), h.min_distances()
+    want, wmind = oracle.assign(X, C, return_mindist=True)
+    label_report(oracle, X, C, got, want)
+    s2 = (X.astype(np.float64) ** 2).sum(1).max() + (C.astype(np.float64) ** 2).sum(1).max()
+    assert np.max(np.abs(mind.astype(np.float64) - wmind)) <= (4 * np.sqrt(d) + 40) * np.finfo(np.float32).eps * s2
