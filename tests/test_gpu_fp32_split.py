@@ -340,3 +340,35 @@ def test_large_and_small_magnitudes(hip, oracle, variant, scale):
     label_report(oracle, X, C, got, want)
     s2 = (X.astype(np.float64) ** 2).sum(1).max() + (C.astype(np.float64) ** 2).sum(1).max()
     assert np.max(np.abs(mind.astype(np.float64) - wmind)) <= (4 * np.sqrt(d) + 40) * np.finfo(np.float32).eps * s2
+
+
+@pytest.mark.parametrize("variant,k,pairs", [("mfma_rowstat", 192, [(7, 36), (3, 160)]),
+                                             ("mfma_tiled", 192, [(7, 36), (3, 160)]),
+                                             ("mfma_tiled", 1024, [(7, 36), (3, 800), (100, 901)])])
+def test_duplicate_centroids_lowest_index_wins(hip, oracle, variant, k, pairs):
+    """Identical centroids give bit-identical distances on the bfloat16 pipe too; the strict
+    '<' of the reference (kmeans_labels.h:360-377) sends every tied row to the lower index,
+    across 32-centroid tiles and across centroid blocks."""
+    n, d = 24000, 32
+    rng = np.random.default_rng(k + 11)
+    centers = rng.uniform(-10, 10, size=(k, d))
+    X = np.ascontiguousarray((centers[rng.integers(0, k, size=n)] + 0.3 * rng.standard_normal((n, d))).astype(np.float32))
+    C0 = np.ascontiguousarray((centers + 0.05).astype(np.float32))
+    for lo, hi in pairs:
+        C0[hi] = C0[lo]
+    want = oracle.assign(X, C0, threads=4)
+    assert not np.isin(want, [hi for _, hi in pairs]).any()
+    for fuse in (1, 0):
+        with hip.Handle(n, d, k, np.float32) as h:
+            h.set_data(X)
+            h.set_centroids(C0)
+            h.set_option("assign", variant)
+            h.set_option("fp32_split", 6)
+            h.set_option("fuse", fuse)
+            h.assign()
+            assert np.array_equal(h.labels(), want), "assignment-only pass"
+            h.iterate(1)
+            assert np.array_equal(h.labels(), want), "Lloyd step, fuse=%d" % fuse
+            C1 = h.centroids()
+        for lo, hi in pairs:
+            assert np.array_equal(C1[hi], C0[hi]) and not np.array_equal(C1[lo], C0[lo])
