@@ -479,25 +479,39 @@ __device__ __forceinline__ int key_row(unsigned v, int g) {
 }
 
 // float32 products on the bfloat16 matrix pipe. A float is the exact sum of three
-// bfloat16 values (8 significant bits each: the float with its low half-word cleared, the
-// same of the remainder, and the rest, every subtraction exact), so x * c is the exact sum
-// of the nine products of their parts, each of which a float holds exactly (16 bits).
-// v_mfma_f32_32x32x16_bf16 adds such products into float accumulators: the result carries
-// float rounding of the running sum only, as the float32 instruction's does. On gfx950
-// the instruction runs at 16 times the float32 rate (nine of them per 16 features take
-// 288 cycles where eight v_mfma_f32_32x32x2_f32 take 512) and, unlike the float32 one,
-// leaves the vector ALU free for the epilogue of another wavefront.
+// bfloat16 values (8 significant bits each: the float rounded to bfloat16, the remainder
+// rounded to bfloat16, and what is left of it, which has at most 8 significant bits; every
+// subtraction is exact), so x * c is the exact sum of the nine products of their parts, each
+// of which a float holds exactly (16 bits). v_mfma_f32_32x32x16_bf16 adds such products
+// into float accumulators: the result carries float rounding of the running sum only, as
+// the float32 instruction's does. On gfx950 the instruction runs at 16 times the float32
+// rate (nine of them per 16 features take 288 cycles where eight v_mfma_f32_32x32x2_f32
+// take 512). The parts are rounded to nearest (v_cvt_pk_bf16_f32), not cut off: the
+// remainders then carry either sign, and the products the 6-product form leaves out cancel
+// on average instead of adding up to a bias of the distances (cut-off parts all have the
+// sign of the float they come from; measured on 6000 x 200 blobs far from the origin, the
+// sum of the minimum distances came out 1.6e-5 too large).
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
 typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ void split_bf16x3(float x, float &h, float &m, float &l) {
-  h = __uint_as_float(__float_as_uint(x) & 0xFFFF0000u);
-  const float r = x - h;
-  m = __uint_as_float(__float_as_uint(r) & 0xFFFF0000u);
-  l = r - m;  // at most 8 significant bits are left: its upper half-word holds it exactly
+// two floats rounded to bfloat16 in one register: a in bits 0-15, b in bits 16-31
+__device__ __forceinline__ unsigned cvt_pk_bf16(float a, float b) {
+  const floatx2 f = {a, b};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(f, bf16x2));
 }
-// upper half-words of two floats as one register: lo in bits 0-15, hi in bits 16-31
-__device__ __forceinline__ unsigned pack_bf16x2(float lo, float hi) {
-  return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
+// The three parts of two floats, each pair packed like cvt_pk_bf16 packs it: 11 vector
+// instructions (three conversions, four unpackings, four subtractions).
+struct Bf16x3Pair {
+  unsigned h, m, l;
+};
+__device__ __forceinline__ Bf16x3Pair split_pair_bf16x3(float a, float b) {
+  Bf16x3Pair p;
+  p.h = cvt_pk_bf16(a, b);
+  const float ra = a - __uint_as_float(p.h << 16), rb = b - __uint_as_float(p.h & 0xFFFF0000u);
+  p.m = cvt_pk_bf16(ra, rb);
+  p.l = cvt_pk_bf16(ra - __uint_as_float(p.m << 16), rb - __uint_as_float(p.m & 0xFFFF0000u));
+  return p;
 }
 __device__ __forceinline__ floatx16 mma_bf16(uintx4 a, uintx4 b, floatx16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
@@ -528,7 +542,7 @@ __device__ __forceinline__ floatx16 mma_bf16(uintx4 a, uintx4 b, floatx16 c) {
 // zero, or finite values meeting zeros on the centroid side).
 // 0: d below the vector width: scalar loads, zero padded.
 // SPLIT (float32 only; 0, 6 or 9): the dot products run on the bfloat16 matrix pipe as that
-// many products of bfloat16 parts per feature pair (see split_bf16x3). 9: every product
+// many products of bfloat16 parts per feature pair (see split_pair_bf16x3). 9: every product
 // exact. 6: the three smallest (below 2^-24 of |x||c|) left out. The centroid parts are
 // staged in LDS in operand order, [tile][16-feature step][part][lane] 16 bytes each; the
 // data rows are split in registers once per row tile.
@@ -589,19 +603,19 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
     // (exact), split into three parts and stored as the lane's operand of that step
     for (int e = tid; e < kp * NS * KL; e += TPB) {
       const int c = e / (NS * KL), rem = e - c * (NS * KL), st = rem / KL, gg = rem - st * KL;
-      float h[8], m[8], l[8];
+      float v[8];
 #pragma unroll
       for (int j = 0; j < 8; j++) {
         const int f = ((2 * st + j / VW) * KL + gg) * VW + j % VW;
-        const float v = (c < k && f < d) ? -2.0f * (float)C[(size_t)c * d + f] : 0.0f;
-        split_bf16x3(v, h[j], m[j], l[j]);
+        v[j] = (c < k && f < d) ? -2.0f * (float)C[(size_t)c * d + f] : 0.0f;
       }
       uintx4 ph, pm, pl;
 #pragma unroll
       for (int w = 0; w < 4; w++) {
-        ph[w] = pack_bf16x2(h[2 * w], h[2 * w + 1]);
-        pm[w] = pack_bf16x2(m[2 * w], m[2 * w + 1]);
-        pl[w] = pack_bf16x2(l[2 * w], l[2 * w + 1]);
+        const Bf16x3Pair pr = split_pair_bf16x3(v[2 * w], v[2 * w + 1]);
+        ph[w] = pr.h;
+        pm[w] = pr.m;
+        pl[w] = pr.l;
       }
       const int t = c / MT, i = c - t * MT;
       uintx4 *dst = reinterpret_cast<uintx4 *>(smem_raw) + (size_t)((t * NS + st) * 3) * 64 + gg * MT + i;
@@ -760,14 +774,13 @@ __global__ __launch_bounds__(NW * 64) void assign_rowstat_kernel(
       for (int rt = 0; rt < ROWT; rt++) {
 #pragma unroll
         for (int st = 0; st < NS; st++) {
-          float h[8], m[8], l[8];
-#pragma unroll
-          for (int j = 0; j < 8; j++) split_bf16x3((float)x[rt][2 * st * VW + j], h[j], m[j], l[j]);
 #pragma unroll
           for (int w = 0; w < 4; w++) {
-            xh[rt][st][w] = pack_bf16x2(h[2 * w], h[2 * w + 1]);
-            xm[rt][st][w] = pack_bf16x2(m[2 * w], m[2 * w + 1]);
-            xl[rt][st][w] = pack_bf16x2(l[2 * w], l[2 * w + 1]);
+            const Bf16x3Pair pr =
+                split_pair_bf16x3((float)x[rt][2 * st * VW + 2 * w], (float)x[rt][2 * st * VW + 2 * w + 1]);
+            xh[rt][st][w] = pr.h;
+            xm[rt][st][w] = pr.m;
+            xl[rt][st][w] = pr.l;
           }
         }
       }
@@ -1000,19 +1013,19 @@ __global__ void split_centroids_kernel(const float *__restrict__ C, uintx4 *__re
     const int cb = (int)(rest / nstage);
     const int gg = slot >> 5, i = slot & 31;
     const int c = cb * bc + t * 32 + i;
-    float h[8], m[8], l[8];
+    float v[8];
 #pragma unroll
     for (int j = 0; j < 8; j++) {
       const int f = st * 16 + ((j >> 2) * 2 + gg) * 4 + (j & 3);
-      const float v = (c < k && f < d) ? C[(size_t)c * d + f] : 0.0f;
-      split_bf16x3(v, h[j], m[j], l[j]);
+      v[j] = (c < k && f < d) ? C[(size_t)c * d + f] : 0.0f;
     }
     uintx4 ph, pm, pl;
 #pragma unroll
     for (int w = 0; w < 4; w++) {
-      ph[w] = pack_bf16x2(h[2 * w], h[2 * w + 1]);
-      pm[w] = pack_bf16x2(m[2 * w], m[2 * w + 1]);
-      pl[w] = pack_bf16x2(l[2 * w], l[2 * w + 1]);
+      const Bf16x3Pair pr = split_pair_bf16x3(v[2 * w], v[2 * w + 1]);
+      ph[w] = pr.h;
+      pm[w] = pr.m;
+      pl[w] = pr.l;
     }
     uintx4 *dst = out + (((size_t)cb * nstage + st) * tiles + t) * 3 * 64 + slot;
     dst[0] = ph;
@@ -1035,7 +1048,7 @@ struct TiledCfg {
   // features per stage. The 64-centroid form serves bandwidth-bound shapes (k <= 64): half
   // the stage depth halves its LDS image, so twice as many workgroups keep loads in flight
   // (500k x 784, k = 10: 0.62 -> 0.49 ms; a quarter of the depth was slower again).
-  // SPLIT (float32 dot products as products of bfloat16 parts, see split_bf16x3): a stage is
+  // SPLIT (float32 dot products as products of bfloat16 parts, see split_pair_bf16x3): a stage is
   // one 16-feature step of the bfloat16 instruction; its three parts per element take 6 bytes
   // of LDS where the float takes 4.
   static constexpr int BK = SPLIT ? 16 : (sizeof(T) == 4 ? 32 : 16) / (BCW == 1 || WIDE ? 2 : 1);
@@ -1208,17 +1221,15 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
   // (SPLIT) the three bfloat16 parts of a staged vector, 8 bytes each
   auto store_parts = [&](unsigned char *dst, const vec_t &v) {
     if constexpr (SPLIT != 0) {
-      float h[4], m[4], l[4];
-#pragma unroll
-      for (int e = 0; e < 4; e++) split_bf16x3((float)v[e], h[e], m[e], l[e]);
       typedef unsigned uintx2 __attribute__((ext_vector_type(2)));
       uintx2 ph, pm, pl;
-      ph[0] = pack_bf16x2(h[0], h[1]);
-      ph[1] = pack_bf16x2(h[2], h[3]);
-      pm[0] = pack_bf16x2(m[0], m[1]);
-      pm[1] = pack_bf16x2(m[2], m[3]);
-      pl[0] = pack_bf16x2(l[0], l[1]);
-      pl[1] = pack_bf16x2(l[2], l[3]);
+#pragma unroll
+      for (int w = 0; w < 2; w++) {
+        const Bf16x3Pair pr = split_pair_bf16x3((float)v[2 * w], (float)v[2 * w + 1]);
+        ph[w] = pr.h;
+        pm[w] = pr.m;
+        pl[w] = pr.l;
+      }
       *reinterpret_cast<uintx2 *>(dst) = ph;
       *reinterpret_cast<uintx2 *>(dst + 1024) = pm;
       *reinterpret_cast<uintx2 *>(dst + 2048) = pl;

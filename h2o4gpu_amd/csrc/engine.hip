@@ -529,9 +529,10 @@ struct Engine : h2o4gpu_kmeans_handle {
   // may still read the old one: the stream is drained before it is replaced); null when the
   // option is off or does not apply, and when the allocation fails (the launch then runs the
   // float32 instructions).
-  SplitScratch split_scratch() {
+  SplitScratch split_scratch() { return split_scratch(k); }
+  SplitScratch split_scratch(int model_rows) {  // (the seeding runs models of other sizes)
     SplitScratch sc;
-    const size_t need = opt_split ? tiled_split_scratch_bytes<T>(opt_split, d, k) : 0;
+    const size_t need = opt_split ? tiled_split_scratch_bytes<T>(opt_split, d, model_rows) : 0;
     if (need == 0) return sc;
     if (need > split_bytes) {
       (void)hipStreamSynchronize(stream);
@@ -874,7 +875,8 @@ struct Engine : h2o4gpu_kmeans_handle {
       KM_TRY(stage(recent));
       // minimum distance to this round's candidates, compared as floats (no integer keys)
       PROFILED("seed_assign", launch_assign<T>(stream, opt_assign, X, xnorm, *Cc, *ccn, labels, mindist,
-                                               n, d, (int)recent.size(), num_cu, nullptr, true));
+                                               n, d, (int)recent.size(), num_cu, nullptr, true, StackShape(),
+                                               opt_split, split_scratch((int)recent.size())));
       PROFILED("seed_fold", launch_fold_min<T>(stream, mindist, *cost, kpp_bsums, n, counter == 0));
       KM_HIP_TRY(hipMemcpyAsync(bs.data(), kpp_bsums, (size_t)nb * sizeof(double), hipMemcpyDeviceToHost,
                                 stream));
@@ -921,7 +923,8 @@ struct Engine : h2o4gpu_kmeans_handle {
     // weights: rows per nearest candidate (count_pts_per_centroid, kmeans_h2o4gpu.h:90-126)
     KM_TRY(stage(all));
     PROFILED("seed_weights", launch_assign<T>(stream, opt_assign, X, xnorm, *Cc, *ccn, labels, mindist, n, d,
-                                              M, num_cu, nullptr, true));
+                                              M, num_cu, nullptr, true, StackShape(), opt_split,
+                                              split_scratch(M)));
     int *dhist = nullptr;
     size_t cap_hist = 0;
     KM_TRY(regrow(&dhist, &cap_hist, (size_t)M));

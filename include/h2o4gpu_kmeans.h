@@ -236,7 +236,8 @@ int h2o4gpu_kmeans_transform_resident(h2o4gpu_kmeans_handle *h, void *d_dist);
  * batch of rows; smaller values force more, shorter batches.
  * "fp32_split" = 9 or 6 (default 0) makes the float32 matrix-core kernels form their dot
  * products on the bfloat16 matrix pipe: every float is the exact sum of three bfloat16
- * parts, 9 runs all nine products of the parts (each exact, accumulated in float32), 6
+ * parts (rounded to nearest), 9 runs all nine products of the parts (each exact,
+ * accumulated in float32), 6
  * leaves out the three smallest (below one ulp of xx + cc per distance). 1.4 to 1.9 times
  * faster on matrix-bound shapes, same parity bars; shapes it does not apply to (float64,
  * k <= 16 && d <= 64, rows of fewer than 4 features, ...) run as without it, and

@@ -14,12 +14,13 @@ def blobs(n, d, k, dtype, seed, spread=20.0):
                                  rng.standard_normal((n, d))).astype(dtype))
 
 
-def run_device(hip, X, k, seed, variant=None):
+def run_device(hip, X, k, seed, variant=None, split=0):
     n, d = X.shape
     with hip.Handle(n, d, k, X.dtype) as h:
         h.set_data(X)
         if variant:
             h.set_option("assign", variant)
+        h.set_option("fp32_split", split)
         h.init_parallel(seed)
         info = h.parallel_seed_info()
         info["centroids"] = h.centroids()
@@ -53,21 +54,26 @@ def test_candidates_weights_and_centres_equal_the_oracle(hip, oracle, n, d, k, s
     assert np.array_equal(got["seed_rows"], want["cand_rows"][want["chosen"]])
 
 
-@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("dtype,split", [(np.float32, 0), (np.float64, 0), (np.float32, 6)])
 @pytest.mark.parametrize("n,d,k,seed", [(20000, 32, 64, 3), (6000, 200, 300, 4), (12000, 128, 40, 8)])
-def test_matrix_core_rounds_differ_only_at_the_threshold(hip, oracle, n, d, k, seed, dtype):
-    """The matrix-core kernels sum the dot products in another order, so a cost can differ
-    from the oracle's in its last bits: a row may then fall on the other side of its
-    threshold only when 2k * cost / potential is within rounding of it."""
+def test_matrix_core_rounds_differ_only_at_the_threshold(hip, oracle, n, d, k, seed, dtype, split):
+    """The matrix-core kernels sum the dot products in another order (with the bfloat16-parts
+    option as well), so a cost can differ from the oracle's in its last bits: a row may then
+    fall on the other side of its threshold only when 2k * cost / potential is within rounding
+    of it."""
     X = blobs(n, d, k, dtype, seed=n + d)
-    got = run_device(hip, X, k, seed)
+    got = run_device(hip, X, k, seed, split=split)
     want = oracle.kmeans_parallel(X, k, seed, threads=4)
     thr = np.array([oracle.row_threshold(seed, int(r)) for r in range(n)], np.float64)
     C = got["centroids"]
     assert np.array_equal(C, X[got["cand_rows"][got["chosen"]]])
     assert len(set(got["chosen"].tolist())) == k
     if np.array_equal(got["cand_rows"], want["cand_rows"]):
-        assert np.allclose(got["phi"], want["phi"], rtol=1e-5 if dtype == np.float32 else 1e-12)
+        # (a row that is a candidate itself costs exactly 0 in the oracle, where both norms and
+        # the dot product are the same sum, and a rounding residue of a few eps * 2|x|^2 on the
+        # matrix cores: with a third of the rows among the candidates the potentials of the
+        # late rounds differ by about 1e-5)
+        assert np.allclose(got["phi"], want["phi"], rtol=3e-5 if dtype == np.float32 else 1e-12)
         # cells: a row between two candidates may be counted for either
         assert np.abs(got["weights"] - want["weights"]).sum() <= max(4, n // 1000)
         if np.array_equal(got["weights"], want["weights"].astype(np.float64)):
