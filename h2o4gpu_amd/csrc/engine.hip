@@ -834,6 +834,9 @@ struct Engine : h2o4gpu_kmeans_handle {
     for (void *p : ptrs)
       if (p) (void)hipFree(p);
     have_mindist = false;  // mindist served as scratch
+    // and so did this set's labels (they number the candidates, not the centroids)
+    if (hipMemsetAsync(labels + row_off(), 0, (size_t)n * sizeof(int), stream) != hipSuccess && rc == 0)
+      rc = H2O4GPU_KMEANS_EDEVICE;
     return rc;
   }
   // (re)allocates a device buffer of at least `count` elements
@@ -967,16 +970,32 @@ struct Engine : h2o4gpu_kmeans_handle {
       }
       return best_idx;
     };
+    // With the scalar-order kernels asked for ("assign" = valu: every distance of the seeding
+    // is then what a scalar loop gives, bit for bit) the distances between candidates are
+    // summed in feature order too, one thread per candidate on a column-major copy; otherwise
+    // by several lanes per candidate.
+    T *CcT = nullptr;
+    int prc = 0;
+    if (opt_assign == ASSIGN_VALU) {
+      KM_TRY(dalloc(&CcT, (size_t)M * d));
+      prc = launch_transpose_candidates<T>(stream, *Cc, CcT, M, d);
+    }
     int idx = pick(nullptr);
-    for (int c = 0; c < k; c++) {
+    for (int c = 0; c < k && prc == 0; c++) {
       seed_info.chosen[(size_t)c] = idx;
       w[(size_t)idx] = 0;
       if (c == k - 1) break;
-      PROFILED("seed_pick", launch_candidate_dists<T>(stream, *Cc, *ccn, idx, *best, M, d, c == 0));
-      KM_HIP_TRY(hipMemcpyAsync(hbest.data(), *best, (size_t)M * sizeof(T), hipMemcpyDeviceToHost, stream));
-      KM_HIP_TRY(hipStreamSynchronize(stream));
-      idx = pick(hbest.data());
+      prof_begin("seed_pick");
+      prc = launch_candidate_dists<T>(stream, *Cc, CcT, *ccn, idx, *best, M, d, c == 0);
+      prof_end();
+      if (prc == 0 && hipMemcpyAsync(hbest.data(), *best, (size_t)M * sizeof(T), hipMemcpyDeviceToHost, stream) != hipSuccess)
+        prc = H2O4GPU_KMEANS_EDEVICE;
+      if (prc == 0 && hipStreamSynchronize(stream) != hipSuccess) prc = H2O4GPU_KMEANS_EDEVICE;
+      if (prc == 0) idx = pick(hbest.data());
     }
+    (void)hipStreamSynchronize(stream);
+    if (CcT) (void)hipFree(CcT);
+    KM_TRY(prc);
     std::vector<int> rows((size_t)k);
     for (int c = 0; c < k; c++) rows[(size_t)c] = all[(size_t)seed_info.chosen[(size_t)c]];
     last_seed_rows = rows;
@@ -1089,7 +1108,14 @@ struct Engine : h2o4gpu_kmeans_handle {
     if (!have_data || !have_centroids) return H2O4GPU_KMEANS_ESTATE;
     maybe_install_signal_handlers();
     int updates = 0;
-    if (sets > 1) {
+    if (max_iterations <= 0) {
+      // The reference's loop then never runs, its final relabel included, and the labels it
+      // returns are the zeros its vector was created with (kmeans_impl.h:109-232,
+      // kmeans_h2o4gpu.cu:747); the centroids stay the starting ones. No minimum distances,
+      // hence no inertia, exist for such a fit.
+      KM_HIP_TRY(hipMemsetAsync(labels, 0, (size_t)n * sets * sizeof(int), stream));
+      have_mindist = false;
+    } else if (sets > 1) {
       KM_TRY(fit_stacked(max_iterations, threshold, &updates));
     } else if (threshold > 0 && max_iterations > 0) {
       KM_TRY(fit_with_threshold(max_iterations, threshold, &updates));

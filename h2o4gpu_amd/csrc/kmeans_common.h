@@ -222,9 +222,15 @@ template <typename T>
 int launch_select_rows(hipStream_t s, const T *cost, T total, uint32_t state0, int k, int *list,
                        int *count, int cap, int64_t n);
 int launch_label_histogram(hipStream_t s, const int *labels, int *counts, int64_t n);
+// CcT: column-major copy of the m candidate rows Cc (launch_transpose_candidates): the dot
+// products are then summed over the features in ascending order, as a scalar loop sums them.
+// CcT null: several lanes share a candidate (strided partial sums and a tree; much faster,
+// another summation order).
 template <typename T>
-int launch_candidate_dists(hipStream_t s, const T *Cc, const T *ccn, int centre, T *best, int m,
-                           int d, int first);
+int launch_transpose_candidates(hipStream_t s, const T *Cc, T *CcT, int m, int d);
+template <typename T>
+int launch_candidate_dists(hipStream_t s, const T *Cc, const T *CcT, const T *ccn, int centre, T *best,
+                           int m, int d, int first);
 
 // Copy rows idx[0..k-1] of X into C ([k][d]).
 template <typename T>

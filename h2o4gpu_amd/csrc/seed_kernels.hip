@@ -342,15 +342,67 @@ int launch_label_histogram(hipStream_t s, const int *labels, int *counts, int64_
   return 0;
 }
 
+// Column-major copy of the m candidate rows: out[j * m + i] = Cc[i * d + j], so that the
+// kernel below reads a feature of consecutive candidates with consecutive lanes.
+template <typename T>
+__global__ __launch_bounds__(WG) void transpose_candidates_kernel(const T *__restrict__ Cc, T *__restrict__ out,
+                                                                  int m, int d) {
+  __shared__ T tile[32][33];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8 threads
+  const int i0 = blockIdx.x * 32, j0 = blockIdx.y * 32;
+  for (int r = ty; r < 32; r += WG / 32) {
+    const int i = i0 + r, jj = j0 + tx;
+    tile[r][tx] = (i < m && jj < d) ? Cc[(size_t)i * d + jj] : (T)0;
+  }
+  __syncthreads();
+  for (int r = ty; r < 32; r += WG / 32) {
+    const int jj = j0 + r, i = i0 + tx;
+    if (i < m && jj < d) out[(size_t)jj * m + i] = tile[tx][r];
+  }
+}
+template <typename T>
+int launch_transpose_candidates(hipStream_t s, const T *Cc, T *out, int m, int d) {
+  if (m <= 0) return 0;
+  hipLaunchKernelGGL((transpose_candidates_kernel<T>), dim3((unsigned)((m + 31) / 32), (unsigned)((d + 31) / 32)),
+                     dim3(WG), 0, s, Cc, out, m, d);
+  KM_HIP_TRY(hipGetLastError());
+  return 0;
+}
+
 // One step of the host k-means++ over the candidates (kmeans_h2o4gpu.cu:226-271), the part
 // that touches every candidate: v = (xx + cc) - 2 x.c against candidate `centre` (the
 // expanded form of src/common/utils.cpp:34-57, no absolute value), best = v at the first
-// step, min(v, best) afterwards with best[centre] taken as 0. lpr lanes share a row.
+// step, min(v, best) afterwards with best[centre] taken as 0. One thread per candidate sums
+// its dot product over the features in ascending order, product and sum rounded separately,
+// as a scalar loop does; CcT is the column-major copy of the candidates, so the loads of a
+// wavefront are contiguous.
 template <typename T>
-__global__ __launch_bounds__(WG) void candidate_dists_kernel(const T *__restrict__ Cc,
+__global__ __launch_bounds__(WG) void candidate_dists_kernel(const T *__restrict__ Cc, const T *__restrict__ CcT,
                                                             const T *__restrict__ ccn, int centre,
-                                                            T *__restrict__ best, int m, int d,
-                                                            int first, int lpr) {
+                                                            T *__restrict__ best, int m, int d, int first) {
+#pragma clang fp contract(off)
+  const int i = blockIdx.x * WG + threadIdx.x;
+  if (i >= m) return;
+  const T *c = Cc + (size_t)centre * d;
+  T dot = 0;
+  for (int j = 0; j < d; j++) dot = dot + CcT[(size_t)j * m + i] * c[j];
+  const T t = ccn[i] + ccn[centre];
+  const T v = (T)-2 * dot + t;
+  if (first) {
+    best[i] = v;
+  } else {
+    const T prev = i == centre ? (T)0 : best[i];
+    best[i] = v < prev ? v : prev;
+  }
+}
+// The same step with lpr lanes sharing a candidate (strided partial sums, then a tree over
+// the lanes): another summation order, an order of magnitude faster when there are few
+// thousand candidates of several hundred features (8304 x 784: 14 against 164 us per pick).
+template <typename T>
+__global__ __launch_bounds__(WG) void candidate_dists_tree_kernel(const T *__restrict__ Cc,
+                                                                 const T *__restrict__ ccn, int centre,
+                                                                 T *__restrict__ best, int m, int d,
+                                                                 int first, int lpr) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int rps = 64 / lpr;
   const int i = (blockIdx.x * (WG / 64) + wave) * rps + lane / lpr;
@@ -371,15 +423,22 @@ __global__ __launch_bounds__(WG) void candidate_dists_kernel(const T *__restrict
     }
   }
 }
+// CcT null: the lane-parallel form on the row-major candidates.
 template <typename T>
-int launch_candidate_dists(hipStream_t s, const T *Cc, const T *ccn, int centre, T *best, int m,
-                           int d, int first) {
+int launch_candidate_dists(hipStream_t s, const T *Cc, const T *CcT, const T *ccn, int centre, T *best,
+                           int m, int d, int first) {
   if (m <= 0) return 0;
-  int lpr = 1;
-  while (lpr < d && lpr < 64) lpr <<= 1;
-  const int rows_per_block = (WG / 64) * (64 / lpr);
-  hipLaunchKernelGGL((candidate_dists_kernel<T>), dim3((unsigned)((m + rows_per_block - 1) / rows_per_block)),
-                     dim3(WG), 0, s, Cc, ccn, centre, best, m, d, first, lpr);
+  if (CcT) {
+    hipLaunchKernelGGL((candidate_dists_kernel<T>), dim3((unsigned)((m + WG - 1) / WG)), dim3(WG), 0, s, Cc,
+                       CcT, ccn, centre, best, m, d, first);
+  } else {
+    int lpr = 1;
+    while (lpr < d && lpr < 64) lpr <<= 1;
+    const int rows_per_block = (WG / 64) * (64 / lpr);
+    hipLaunchKernelGGL((candidate_dists_tree_kernel<T>),
+                       dim3((unsigned)((m + rows_per_block - 1) / rows_per_block)), dim3(WG), 0, s, Cc, ccn,
+                       centre, best, m, d, first, lpr);
+  }
   KM_HIP_TRY(hipGetLastError());
   return 0;
 }
@@ -390,8 +449,9 @@ int launch_candidate_dists(hipStream_t s, const T *Cc, const T *ccn, int centre,
   template int launch_fold_min<T>(hipStream_t, const T *, T *, double *, int64_t, int);         \
   template int launch_select_rows<T>(hipStream_t, const T *, T, uint32_t, int, int *, int *,    \
                                      int, int64_t);                                             \
-  template int launch_candidate_dists<T>(hipStream_t, const T *, const T *, int, T *, int, int, \
-                                         int);
+  template int launch_transpose_candidates<T>(hipStream_t, const T *, T *, int, int);           \
+  template int launch_candidate_dists<T>(hipStream_t, const T *, const T *, const T *, int, T *, \
+                                         int, int, int);
 KM_SEED_INSTANTIATE(float)
 KM_SEED_INSTANTIATE(double)
 

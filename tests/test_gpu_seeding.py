@@ -35,7 +35,8 @@ def run_device(hip, X, k, seed, variant=None, split=0):
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("n,d,k,seed", [(20000, 8, 12, 5), (9000, 16, 20, 9), (30000, 3, 40, 123),
-                                        (5000, 33, 7, 1), (2500, 64, 64, 77)])
+                                        (5000, 33, 7, 1), (2500, 64, 64, 77), (294, 189, 67, 3),
+                                        (3000, 300, 90, 11)])
 def test_candidates_weights_and_centres_equal_the_oracle(hip, oracle, n, d, k, seed, dtype):
     """With the scalar-order distance kernel every distance is the oracle's bit for bit, the
     sum of the costs uses the same fixed tree, and the acceptance test is integer and IEEE
@@ -108,10 +109,16 @@ def test_fit_entry_point_seeds_with_kmeans_parallel(hip, oracle):
     rc = ch2o4gpu_gpu.make_ptr_float_kmeans(0, 0, seed, 0, 1, n, d, k, 0, 1, 0.0, X.flatten(),
                                             np.empty([], np.float32), centres, labels)
     assert rc == 0
+    # no iteration, no relabel: the labels are the zeros the reference's vector starts with
+    # (kmeans_h2o4gpu.cu:747), not what the seeding left in its scratch
+    assert not labels.any()
     with hip.Handle(n, d, k, np.float32) as h:
         h.set_data(X)
         h.init_parallel(seed)
         assert np.array_equal(centres.reshape(k, d), h.centroids())
+        assert not h.labels().any()
+        with pytest.raises(hip.KMeansHipError):
+            h.inertia()
     want = oracle.kmeans_parallel(X, k, seed, threads=4)
     assert np.array_equal(centres.reshape(k, d), want["centroids"])
     # and a real fit from that start lowers the objective below the seeds' own
