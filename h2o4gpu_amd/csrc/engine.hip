@@ -301,6 +301,11 @@ struct StagingPool {
   std::mutex mu;
   void *buf[MAX_DEV][2] = {};
   hipEvent_t done[MAX_DEV][2] = {};
+  // The staged copies run on a stream of the pool's own, which lives as long as the events
+  // recorded on it. (Recorded on a handle's stream, an event outlived the stream: after some
+  // 12,000 handles created and destroyed in one process, hipEventSynchronize on such an event
+  // failed with "operation not permitted on an event last recorded in a capturing stream".)
+  hipStream_t xfer[MAX_DEV] = {};
   bool broken[MAX_DEV] = {};
 
   // Host copies run on a small set of worker threads that are created once and then wait
@@ -390,7 +395,13 @@ struct StagingPool {
   // Pinned buffers and events of a device, created on first use (caller holds mu).
   bool ensure(int dev) {
     if (broken[dev]) return false;
-    if (buf[dev][1] && done[dev][1]) return true;
+    if (buf[dev][1] && done[dev][1] && xfer[dev]) return true;
+    if (!xfer[dev] && hipStreamCreateWithFlags(&xfer[dev], hipStreamNonBlocking) != hipSuccess) {
+      (void)hipGetLastError();
+      xfer[dev] = nullptr;
+      broken[dev] = true;
+      return false;
+    }
     for (int i = 0; i < 2; i++) {
       if (hipHostMalloc(&buf[dev][i], CHUNK, hipHostMallocDefault) != hipSuccess ||
           hipEventCreateWithFlags(&done[dev][i], hipEventDisableTiming) != hipSuccess) {
@@ -413,14 +424,15 @@ struct StagingPool {
     if (threads < 1) threads = 1;
     const size_t piece = piece_size(bytes);
     size_t off = 0;
+    KM_HIP_TRY(hipStreamSynchronize(stream));  // whatever the caller's stream still does with dst
     for (int i = 0; off < bytes; i ^= 1) {
       const size_t len = std::min(piece, bytes - off);
       KM_HIP_TRY(hipEventSynchronize(done[dev][i]));  // the DMA that last read this buffer
       parallel_copy(static_cast<char *>(buf[dev][i]), static_cast<const char *>(src) + off, len,
                     threads);
       KM_HIP_TRY(hipMemcpyAsync(static_cast<char *>(dst) + off, buf[dev][i], len,
-                                hipMemcpyHostToDevice, stream));
-      KM_HIP_TRY(hipEventRecord(done[dev][i], stream));
+                                hipMemcpyHostToDevice, xfer[dev]));
+      KM_HIP_TRY(hipEventRecord(done[dev][i], xfer[dev]));
       off += len;
     }
     // both buffers must be drained before the next caller (or this one) refills them
@@ -440,13 +452,14 @@ struct StagingPool {
     if (threads < 1) threads = 1;
     const size_t piece = piece_size(bytes);
     const size_t chunks = (bytes + piece - 1) / piece;
+    KM_HIP_TRY(hipStreamSynchronize(stream));  // the kernels that produce src
     for (size_t c = 0; c <= chunks; c++) {
       const int b = (int)(c & 1);
       if (c < chunks) {
         const size_t off = c * piece, len = std::min(piece, bytes - off);
         KM_HIP_TRY(hipMemcpyAsync(buf[dev][b], static_cast<const char *>(src) + off, len,
-                                  hipMemcpyDeviceToHost, stream));
-        KM_HIP_TRY(hipEventRecord(done[dev][b], stream));
+                                  hipMemcpyDeviceToHost, xfer[dev]));
+        KM_HIP_TRY(hipEventRecord(done[dev][b], xfer[dev]));
       }
       if (c >= 1) {  // chunk c-1 sits in the other buffer
         const size_t off = (c - 1) * piece, len = std::min(piece, bytes - off);
@@ -469,6 +482,8 @@ struct StagingPool {
       done[dev][i] = nullptr;
       buf[dev][i] = nullptr;
     }
+    if (xfer[dev]) (void)hipStreamDestroy(xfer[dev]);
+    xfer[dev] = nullptr;
     broken[dev] = false;
   }
 };
@@ -1180,8 +1195,46 @@ struct Engine : h2o4gpu_kmeans_handle {
         break;
       }
     }
-    if (max_iterations > 0) KM_TRY(assign());  // final relabel of every set with its final centroids
+    if (max_iterations > 0) KM_TRY(relabel_sets());  // final relabel of every set with its final centroids
     *updates_out = updates;
+    return 0;
+  }
+
+  // The final relabel of a stacked fit, one set at a time as an ordinary model of kset
+  // centroids: the kernels (and hence the labels and minimum distances, near-ties included)
+  // are those a handle of one set runs on these centroids, so predicting the training rows
+  // with the winning centroids gives back its labels whichever way the restarts ran.
+  int relabel_sets() {
+    const size_t kpad = ((size_t)kset + CENTROID_PAD - 1) / CENTROID_PAD * CENTROID_PAD;
+    T *Cp = nullptr, *cn = nullptr;
+    KM_TRY(dalloc(&Cp, kpad * d));
+    int rc = dalloc(&cn, kpad);
+    const std::vector<T> inf(kpad, std::numeric_limits<T>::infinity());
+    for (int s = 0; s < sets && rc == 0; s++) {
+      // padded like an ordinary model: zero rows with +inf norms past the last centroid
+      if (hipMemsetAsync(Cp, 0, kpad * d * sizeof(T), stream) != hipSuccess ||
+          hipMemcpyAsync(Cp, C[cur] + (size_t)s * kps * d, (size_t)kset * d * sizeof(T),
+                         hipMemcpyDeviceToDevice, stream) != hipSuccess ||
+          hipMemcpyAsync(cn, inf.data(), kpad * sizeof(T), hipMemcpyHostToDevice, stream) != hipSuccess ||
+          hipStreamSynchronize(stream) != hipSuccess) {
+        rc = H2O4GPU_KMEANS_EDEVICE;
+        break;
+      }
+      prof_begin("row_norms");
+      rc = launch_row_norms<T>(stream, Cp, cn, kset, d);
+      prof_end();
+      if (rc != 0) break;
+      prof_begin("assign");
+      rc = launch_assign<T>(stream, opt_assign, X, xnorm, Cp, cn, labels + (size_t)s * n,
+                            mindist + (size_t)s * n, n, d, kset, num_cu, &last_variant, opt_exact != 0,
+                            StackShape(), opt_split, split_scratch(kset));
+      prof_end();
+    }
+    (void)hipStreamSynchronize(stream);
+    if (Cp) (void)hipFree(Cp);
+    if (cn) (void)hipFree(cn);
+    KM_TRY(rc);
+    have_mindist = true;
     return 0;
   }
 

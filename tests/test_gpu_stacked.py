@@ -39,6 +39,7 @@ def test_stacked_sets_equal_serial_restarts(hip, n, d, k, sets, dtype):
     iters = 7
     with hip.Handle(n, d, k, dtype, sets=sets) as h:
         h.set_data(X)
+        h.set_option("assign", "mfma_rowstat")  # (the final relabel runs ordinary kernels: these)
         for s in range(sets):
             h.select_set(s)
             h.set_centroids(starts[s])
@@ -75,6 +76,7 @@ def test_every_set_stops_at_its_own_iteration(hip):
     want = [serial_fit(hip, X, k, c0, 60, tol) for c0 in starts]
     with hip.Handle(n, d, k, np.float32, sets=sets) as h:
         h.set_data(X)
+        h.set_option("assign", "mfma_rowstat")
         for s in range(sets):
             h.select_set(s)
             h.set_centroids(starts[s])
