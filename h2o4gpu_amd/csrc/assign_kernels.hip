@@ -1470,7 +1470,6 @@ const char *assign_variant_name(int variant) {
   }
 }
 
-static const size_t LDS_LIMIT = 160 * 1024;
 
 template <typename T>
 static int rowstat_dp(int d) {
