@@ -1109,8 +1109,29 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
   const int cb_id = MODE == 1 ? (int)((int64_t)blockIdx.x - rt_id * ncb) : 0;
   const int64_t row0 = rt_id * BR;
   const int nstage = (d + BK - 1) / BK;
-  // steps of the last stage that hold features: its ceil(rest / VW) vectors, KL per step
-  const int nq_tail = ((d - (nstage - 1) * BK + VW - 1) / VW + KL - 1) / KL;
+  // A stage is NV steps of KL vectors (KL * VW features). Where d is not a whole number of
+  // stages (DTAIL) the d-steps are dealt evenly over the stages, the first `srem` stages one
+  // step longer than the rest, instead of leaving a short last stage: staging a stage costs
+  // the same whatever it holds, and a stage with a full share of matrix instructions hides
+  // more of it. Measured against whole stages and a short last one, same box, alternating
+  // runs: float32 3M x 100, k = 1000 (4, 4, 4, 1 -> 4, 3, 3, 3 steps) 5.77 -> 5.70 ms, 261k x
+  // 298, k = 1000 1.528 -> 1.507 ms, 200k x 780, k = 4096 11.47 -> 11.32 ms; with one test per
+  // step (`q >= nq_st`) for every stage instead of a second one for "last stage" the double
+  // kernels gained more than the dealing explains (1M x 100, k = 1000 4.05 -> 3.69 ms, 500k x
+  // 250, k = 1024 4.54 -> 4.24 ms, the same steps per stage before and after). The
+  // bfloat16-parts kernels keep whole stages: theirs is a single step.
+  constexpr int SF = KL * VW;
+  constexpr bool EVEN = DTAIL && SPLIT == 0;
+  const int nsteps = (d + SF - 1) / SF;
+  const int sbase = EVEN ? nsteps / nstage : NV;
+  const int srem = EVEN ? nsteps - sbase * nstage : 0;
+  auto stage_off = [&](int st) { return EVEN ? SF * (st * sbase + min(st, srem)) : st * BK; };
+  // steps of stage st that hold features
+  auto stage_nq = [&](int st) {
+    if (EVEN) return sbase + (st < srem ? 1 : 0);
+    // whole stages, the last one ceil(rest / VW) vectors, KL per step
+    return st + 1 < nstage ? NV : ((d - (nstage - 1) * BK + VW - 1) / VW + KL - 1) / KL;
+  };
 
   // staging role of this thread: operand row rr0 + q*ROWS_PER_PASS, features
   // [jj, jj+VW) of the stage. The 16-byte vector lands in LDS at tile rr/MT,
@@ -1180,7 +1201,7 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
   // instance of the loader (tail_tag true) used for that step alone.
   auto gload = [&](int c0, int st, auto tail_tag) {
     constexpr bool TAILSTEP = DTAIL && decltype(tail_tag)::value;
-    const int j = st * BK + jj;
+    const int j = stage_off(st) + jj;
     // VECLOAD: 16-byte loads at element-aligned addresses; in the tail step through
     // load_row_vector, which stays inside the row and returns zero past feature d
     auto fetch = [&](const T *src, bool zero_past_d) -> vec_t {
@@ -1195,7 +1216,9 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
         } else if (TAILSTEP) {
           v = load_row_vector<T>(src, j, d);
         } else {
-          const uvec_t u = *reinterpret_cast<const uvec_t *>(src + j);
+          // (EVEN: the vectors past a stage's own steps belong to the next stage and are not
+          // used; near the end of the row they are fetched from inside it all the same)
+          const uvec_t u = *reinterpret_cast<const uvec_t *>(src + (EVEN ? min(j, d - VW) : j));
 #pragma unroll
           for (int e = 0; e < VW; e++) v[e] = u[e];
         }
@@ -1314,9 +1337,10 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
       }
       const vec_t *ap = reinterpret_cast<const vec_t *>(As + buf * A_ELEMS);
       const vec_t *bp = reinterpret_cast<const vec_t *>(Bs + buf * B_ELEMS);
+      const int nq_st = DTAIL ? stage_nq(st) : NV;
 #pragma unroll
       for (int q = 0; q < (SPLIT ? 0 : NV); q++) {
-        if (DTAIL && st + 1 == nstage && q >= nq_tail) continue;  // nothing but zeros there
+        if (DTAIL && q >= nq_st) continue;  // nothing of this stage there
         vec_t a[CT], b[RT];
 #pragma unroll
         for (int ct = 0; ct < CT; ct++) a[ct] = ap[((wc * CT + ct) * NV + q) * 64 + rd_slot[q]];

@@ -513,6 +513,41 @@ def test_more_than_two_to_the_31_elements(hip, oracle):
         assert np.allclose(C1[c], m, rtol=1e-5, atol=1e-4)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("k", [130, 9000])
+def test_tiled_every_feature_count(hip, k, dtype):
+    """The tiled kernel deals the features of a row that is not a whole number of stages evenly
+    over its stages: every feature count from 4 to 140 (and a few long ones), with the 128-centroid
+    block (k = 130) and the 256-centroid one (float32 models beyond 4 MB: k = 9000 from 117
+    features on), against float64 brute force. A feature left out or taken twice moves a distance
+    by far more than the tolerance."""
+    n = 257
+    rng = np.random.default_rng(k)
+    eps = np.finfo(dtype).eps
+    ds = list(range(4, 141)) + [250, 271, 519, 777]
+    if k > 1000:
+        ds = [d for d in ds if d >= 117 and (d < 141 and d % 3 == 0 or d > 141)] + [118, 121, 125]
+    bad = []
+    for d in ds:
+        X = np.ascontiguousarray((3.0 * rng.standard_normal((n, d))).astype(dtype))
+        C = np.ascontiguousarray((3.0 * rng.standard_normal((k, d))).astype(dtype))
+        with hip.Handle(n, d, k, dtype) as h:
+            h.set_data(X)
+            h.set_centroids(C)
+            h.set_option("assign", "mfma_tiled")
+            assert h.assign_variant() == "mfma_tiled"
+            h.assign()
+            got, mind = h.labels(), h.min_distances()
+        X64, C64 = X.astype(np.float64), C.astype(np.float64)
+        D = (X64 ** 2).sum(1)[:, None] + (C64 ** 2).sum(1)[None, :] - 2.0 * X64 @ C64.T
+        best = D.min(1)
+        scale = (X64 ** 2).sum(1).max() + (C64 ** 2).sum(1).max()
+        tol = (4 * np.sqrt(d) + 40) * eps * scale
+        if np.abs(mind - best).max() > tol or (D[np.arange(n), got] - best).max() > tol:
+            bad.append((d, float(np.abs(mind - best).max()), float((D[np.arange(n), got] - best).max()), tol))
+    assert not bad, bad
+
+
 def _random_shapes(count, seed):
     """Seeded shapes spread over every dispatch rule: feature counts around the vector
     and MFMA-slice boundaries, models from one centroid to several LDS chunks."""
