@@ -962,7 +962,7 @@ struct Engine : h2o4gpu_kmeans_handle {
     }
     // the host k-means++ (kmeans_h2o4gpu.cu:201-279); its distances run on the device
     KM_TRY(regrow(best, &cap_best, (size_t)M));
-    std::vector<T> thr((size_t)M), hbest((size_t)M);
+    std::vector<T> thr((size_t)M), share((size_t)M);
     {
       std::mt19937 mt(seed);  // the sampler makes a fresh one on every call: same draws
       std::uniform_real_distribution<> dist(0.0, 1.0);
@@ -971,15 +971,16 @@ struct Engine : h2o4gpu_kmeans_handle {
     auto pick = [&](const T *data) -> int {  // pick_point_idx_weighted
       T weighted_sum = 0;
       for (int i = 0; i < M; i++) weighted_sum += data ? data[i] * w[(size_t)i] : w[(size_t)i];
+      // the shares first, in a loop without an exit (it vectorises; the divisions are the same
+      // IEEE divisions), then the reference's walk over them
+      for (int i = 0; i < M; i++) share[(size_t)i] = (data ? data[i] * w[(size_t)i] : w[(size_t)i]) / weighted_sum;
       T best_prob = 0;
       int best_idx = 0;
       for (int i = 0; i < M; i++) {
-        T val = w[(size_t)i];
-        if (data) val *= data[i];
-        const T share = val / weighted_sum;
-        if (share > thr[(size_t)i]) return i;
-        if (share >= best_prob) {
-          best_prob = share;
+        const T sh = share[(size_t)i];
+        if (sh > thr[(size_t)i]) return i;
+        if (sh >= best_prob) {
+          best_prob = sh;
           best_idx = i;
         }
       }
@@ -995,20 +996,27 @@ struct Engine : h2o4gpu_kmeans_handle {
       KM_TRY(dalloc(&CcT, (size_t)M * d));
       prc = launch_transpose_candidates<T>(stream, *Cc, CcT, M, d);
     }
+    // every pick ends with the M distances on the host: the kernel writes them into pinned host
+    // memory itself, beside its device copy, so a pick costs one launch and one wait and no
+    // copy command (8304 candidates, 4096 picks: 0.317 -> 0.29 s for the whole seeding)
+    T *hbest = nullptr;
+    if (prc == 0 && hipHostMalloc(reinterpret_cast<void **>(&hbest), (size_t)M * sizeof(T), hipHostMallocDefault) != hipSuccess) {
+      (void)hipGetLastError();
+      prc = H2O4GPU_KMEANS_EALLOC;
+    }
     int idx = pick(nullptr);
     for (int c = 0; c < k && prc == 0; c++) {
       seed_info.chosen[(size_t)c] = idx;
       w[(size_t)idx] = 0;
       if (c == k - 1) break;
       prof_begin("seed_pick");
-      prc = launch_candidate_dists<T>(stream, *Cc, CcT, *ccn, idx, *best, M, d, c == 0);
+      prc = launch_candidate_dists<T>(stream, *Cc, CcT, *ccn, idx, *best, hbest, M, d, c == 0);
       prof_end();
-      if (prc == 0 && hipMemcpyAsync(hbest.data(), *best, (size_t)M * sizeof(T), hipMemcpyDeviceToHost, stream) != hipSuccess)
-        prc = H2O4GPU_KMEANS_EDEVICE;
       if (prc == 0 && hipStreamSynchronize(stream) != hipSuccess) prc = H2O4GPU_KMEANS_EDEVICE;
-      if (prc == 0) idx = pick(hbest.data());
+      if (prc == 0) idx = pick(hbest);
     }
     (void)hipStreamSynchronize(stream);
+    if (hbest) (void)hipHostFree(hbest);
     if (CcT) (void)hipFree(CcT);
     KM_TRY(prc);
     std::vector<int> rows((size_t)k);

@@ -230,7 +230,7 @@ template <typename T>
 int launch_transpose_candidates(hipStream_t s, const T *Cc, T *CcT, int m, int d);
 template <typename T>
 int launch_candidate_dists(hipStream_t s, const T *Cc, const T *CcT, const T *ccn, int centre, T *best,
-                           int m, int d, int first);
+                           T *mirror, int m, int d, int first);
 
 // Copy rows idx[0..k-1] of X into C ([k][d]).
 template <typename T>

@@ -379,7 +379,8 @@ int launch_transpose_candidates(hipStream_t s, const T *Cc, T *out, int m, int d
 template <typename T>
 __global__ __launch_bounds__(WG) void candidate_dists_kernel(const T *__restrict__ Cc, const T *__restrict__ CcT,
                                                             const T *__restrict__ ccn, int centre,
-                                                            T *__restrict__ best, int m, int d, int first) {
+                                                            T *__restrict__ best, T *__restrict__ mirror, int m,
+                                                            int d, int first) {
 #pragma clang fp contract(off)
   const int i = blockIdx.x * WG + threadIdx.x;
   if (i >= m) return;
@@ -388,12 +389,13 @@ __global__ __launch_bounds__(WG) void candidate_dists_kernel(const T *__restrict
   for (int j = 0; j < d; j++) dot = dot + CcT[(size_t)j * m + i] * c[j];
   const T t = ccn[i] + ccn[centre];
   const T v = (T)-2 * dot + t;
-  if (first) {
-    best[i] = v;
-  } else {
+  T nb = v;
+  if (!first) {
     const T prev = i == centre ? (T)0 : best[i];
-    best[i] = v < prev ? v : prev;
+    nb = v < prev ? v : prev;
   }
+  best[i] = nb;
+  if (mirror) mirror[i] = nb;
 }
 // The same step with lpr lanes sharing a candidate (strided partial sums, then a tree over
 // the lanes): another summation order, an order of magnitude faster when there are few
@@ -401,8 +403,8 @@ __global__ __launch_bounds__(WG) void candidate_dists_kernel(const T *__restrict
 template <typename T>
 __global__ __launch_bounds__(WG) void candidate_dists_tree_kernel(const T *__restrict__ Cc,
                                                                  const T *__restrict__ ccn, int centre,
-                                                                 T *__restrict__ best, int m, int d,
-                                                                 int first, int lpr) {
+                                                                 T *__restrict__ best, T *__restrict__ mirror,
+                                                                 int m, int d, int first, int lpr) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int rps = 64 / lpr;
   const int i = (blockIdx.x * (WG / 64) + wave) * rps + lane / lpr;
@@ -415,29 +417,32 @@ __global__ __launch_bounds__(WG) void candidate_dists_tree_kernel(const T *__res
   if (col == 0 && i < m) {
     const T t = ccn[i] + ccn[centre];
     const T v = (T)-2 * dot + t;
-    if (first) {
-      best[i] = v;
-    } else {
+    T nb = v;
+    if (!first) {
       const T prev = i == centre ? (T)0 : best[i];
-      best[i] = v < prev ? v : prev;
+      nb = v < prev ? v : prev;
     }
+    best[i] = nb;
+    if (mirror) mirror[i] = nb;
   }
 }
-// CcT null: the lane-parallel form on the row-major candidates.
+// CcT null: the lane-parallel form on the row-major candidates. mirror (may be null): a second
+// copy of the result, meant for pinned host memory that the device writes directly, which
+// spares the caller a copy command per step.
 template <typename T>
 int launch_candidate_dists(hipStream_t s, const T *Cc, const T *CcT, const T *ccn, int centre, T *best,
-                           int m, int d, int first) {
+                           T *mirror, int m, int d, int first) {
   if (m <= 0) return 0;
   if (CcT) {
     hipLaunchKernelGGL((candidate_dists_kernel<T>), dim3((unsigned)((m + WG - 1) / WG)), dim3(WG), 0, s, Cc,
-                       CcT, ccn, centre, best, m, d, first);
+                       CcT, ccn, centre, best, mirror, m, d, first);
   } else {
     int lpr = 1;
     while (lpr < d && lpr < 64) lpr <<= 1;
     const int rows_per_block = (WG / 64) * (64 / lpr);
     hipLaunchKernelGGL((candidate_dists_tree_kernel<T>),
                        dim3((unsigned)((m + rows_per_block - 1) / rows_per_block)), dim3(WG), 0, s, Cc, ccn,
-                       centre, best, m, d, first, lpr);
+                       centre, best, mirror, m, d, first, lpr);
   }
   KM_HIP_TRY(hipGetLastError());
   return 0;
@@ -451,7 +456,7 @@ int launch_candidate_dists(hipStream_t s, const T *Cc, const T *CcT, const T *cc
                                      int, int64_t);                                             \
   template int launch_transpose_candidates<T>(hipStream_t, const T *, T *, int, int);           \
   template int launch_candidate_dists<T>(hipStream_t, const T *, const T *, const T *, int, T *, \
-                                         int, int, int);
+                                         T *, int, int, int);
 KM_SEED_INSTANTIATE(float)
 KM_SEED_INSTANTIATE(double)
 
