@@ -217,7 +217,8 @@ template <typename T>
 int launch_gather_model(hipStream_t s, const T *X, const T *xnorm, const int *idx, int m, int mpad,
                         T *Cc, T *ccn, int d);
 template <typename T>
-int launch_fold_min(hipStream_t s, const T *cur, T *cost, double *bsums, int64_t n, int init);
+int launch_fold_min(hipStream_t s, const T *cur, T *cost, double *bsums, int64_t n, int init,
+                    const int *cur_label = nullptr, int *near = nullptr, int label_off = 0);
 template <typename T>
 int launch_select_rows(hipStream_t s, const T *cost, T total, uint32_t state0, int k, int *list,
                        int *count, int cap, int64_t n);

@@ -247,10 +247,16 @@ int launch_gather_model(hipStream_t s, const T *X, const T *xnorm, const int *id
 
 // cost[i] = min(cost[i], cur[i]) (init != 0: cost[i] = min(max(T), cur[i])), then the block
 // sums of cost in double with the fixed tree of block_sum. One workgroup per KPP_BLOCK rows.
+// With near != null the pass also keeps which candidate the running minimum belongs to:
+// cur_label[i] numbers the candidates of this pass from 0, label_off is the place of the
+// first of them in the list of all candidates, and a later pass replaces an earlier
+// candidate only with a strictly smaller distance, so near[i] ends as the nearest of all
+// candidates with the lowest index on ties, which is what one pass over all of them gives.
 template <typename T>
 __global__ __launch_bounds__(WG) void fold_min_kernel(const T *__restrict__ cur, T *__restrict__ cost,
                                                      double *__restrict__ bsums, int64_t n,
-                                                     int init) {
+                                                     int init, const int *__restrict__ cur_label,
+                                                     int *__restrict__ near, int label_off) {
   __shared__ double red[WG];
   const int64_t b0 = (int64_t)blockIdx.x * KPP_BLOCK;
 #pragma unroll
@@ -260,16 +266,21 @@ __global__ __launch_bounds__(WG) void fold_min_kernel(const T *__restrict__ cur,
       const T prev = init ? std::numeric_limits<T>::max() : cost[row];
       const T c = cur[row];
       cost[row] = c < prev ? c : prev;
+      if (near && (init || c < prev)) {
+        const int l = cur_label[row];
+        near[row] = l < 0 ? -1 : label_off + l;  // (a row without a finite distance has no label)
+      }
     }
   }
   __syncthreads();  // (each thread re-reads only what it wrote; the barrier orders the LDS use)
   block_sum<T>(cost, bsums, blockIdx.x, n, red);
 }
 template <typename T>
-int launch_fold_min(hipStream_t s, const T *cur, T *cost, double *bsums, int64_t n, int init) {
+int launch_fold_min(hipStream_t s, const T *cur, T *cost, double *bsums, int64_t n, int init,
+                    const int *cur_label, int *near, int label_off) {
   if (n <= 0) return 0;
   hipLaunchKernelGGL((fold_min_kernel<T>), dim3((unsigned)((n + KPP_BLOCK - 1) / KPP_BLOCK)),
-                     dim3(WG), 0, s, cur, cost, bsums, n, init);
+                     dim3(WG), 0, s, cur, cost, bsums, n, init, cur_label, near, label_off);
   KM_HIP_TRY(hipGetLastError());
   return 0;
 }
@@ -451,7 +462,8 @@ int launch_candidate_dists(hipStream_t s, const T *Cc, const T *CcT, const T *cc
 #define KM_SEED_INSTANTIATE(T)                                                                  \
   template int launch_gather_model<T>(hipStream_t, const T *, const T *, const int *, int, int, \
                                       T *, T *, int);                                           \
-  template int launch_fold_min<T>(hipStream_t, const T *, T *, double *, int64_t, int);         \
+  template int launch_fold_min<T>(hipStream_t, const T *, T *, double *, int64_t, int,          \
+                                  const int *, int *, int);                                     \
   template int launch_select_rows<T>(hipStream_t, const T *, T, uint32_t, int, int *, int *,    \
                                      int, int64_t);                                             \
   template int launch_transpose_candidates<T>(hipStream_t, const T *, T *, int, int);           \

@@ -49,6 +49,12 @@ def test_candidates_weights_and_centres_equal_the_oracle(hip, oracle, n, d, k, s
     assert np.array_equal(got["phi"], want["phi"])
     M = len(want["cand_rows"])
     assert M > k
+    if k == 7:
+        # three rounds, and the last one still adds candidates: no round has measured the rows
+        # against those, so the engine's weights need its extra pass over them
+        assert want["round_count"][2] > 0
+    # (the engine takes the weights from the nearest candidate noted round by round, the
+    # oracle from one pass over all candidates)
     assert np.array_equal(got["weights"], want["weights"].astype(np.float64))
     assert np.array_equal(got["chosen"], want["chosen"])
     assert np.array_equal(got["centroids"], want["centroids"])
