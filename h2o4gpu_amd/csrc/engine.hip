@@ -181,6 +181,7 @@ struct h2o4gpu_kmeans_handle {
   int opt_buckets = 1;  // 1: bucketed centroid sums where the sums do not fit LDS
   int opt_exact = 0;    // 1: float32 MFMA argmin on the float distances, not on 16-ulp keys
   int opt_split = 0;    // 6 or 9: float32 matrix-core kernels as that many bfloat16 products per feature pair
+  int opt_seed_matrix = 1;  // k-means||: distances between candidates as one matrix (0: a kernel per pick)
   int opt_transform_batch_mb = 4096;  // device buffer of transform_host's output, per batch of rows
   int last_variant = ASSIGN_AUTO;
 
@@ -992,22 +993,78 @@ struct Engine : h2o4gpu_kmeans_handle {
       // the shares first, in a loop without an exit (it vectorises; the divisions are the same
       // IEEE divisions), then the reference's walk over them
       for (int i = 0; i < M; i++) share[(size_t)i] = (data ? data[i] * w[(size_t)i] : w[(size_t)i]) / weighted_sum;
+      // The walk, `if (share > threshold) return i; if (share >= best) { best = share; idx = i; }`
+      // from a best of 0, in loops without an exit where it matters: whether any entry passes
+      // its threshold at all (rarely: a share is about 1/M), then the largest share that is not
+      // below 0 and the last entry that has it (a NaN share is neither passed nor kept, as in
+      // the walk; -0 equals 0 in both).
+      int passes = 0;
+      for (int i = 0; i < M; i++) passes += share[(size_t)i] > thr[(size_t)i] ? 1 : 0;
+      if (passes)
+        for (int i = 0; i < M; i++)
+          if (share[(size_t)i] > thr[(size_t)i]) return i;
+      T lane_best[8] = {0, 0, 0, 0, 0, 0, 0, 0};  // (eight running maxima: no chain of dependent compares)
+      int i8 = 0;
+      for (; i8 + 8 <= M; i8 += 8)
+        for (int u = 0; u < 8; u++)
+          lane_best[u] = share[(size_t)(i8 + u)] > lane_best[u] ? share[(size_t)(i8 + u)] : lane_best[u];
       T best_prob = 0;
-      int best_idx = 0;
-      for (int i = 0; i < M; i++) {
-        const T sh = share[(size_t)i];
-        if (sh > thr[(size_t)i]) return i;
-        if (sh >= best_prob) {
-          best_prob = sh;
-          best_idx = i;
-        }
-      }
-      return best_idx;
+      for (; i8 < M; i8++) best_prob = share[(size_t)i8] > best_prob ? share[(size_t)i8] : best_prob;
+      for (int u = 0; u < 8; u++) best_prob = lane_best[u] > best_prob ? lane_best[u] : best_prob;
+      for (int i = M - 1; i > 0; i--)
+        if (share[(size_t)i] == best_prob) return i;
+      return 0;
     };
     // With the scalar-order kernels asked for ("assign" = valu: every distance of the seeding
     // is then what a scalar loop gives, bit for bit) the distances between candidates are
     // summed in feature order too, one thread per candidate on a column-major copy; otherwise
     // by several lanes per candidate.
+    // Otherwise, while M x M distances fit 1 GiB, all of them are computed at once by the
+    // transform kernels (the candidates against themselves, |v| where the reference has v: the
+    // two differ for v < 0 only, i.e. within rounding of a candidate's distance to a copy of
+    // itself) and brought to the host, where a pick is then a minimum over one row of that
+    // matrix and the sampler's two loops, with no launch and no wait: 8304 candidates of 784
+    // features, 4095 picks: 57 ms of kernels and as many waits become 1 ms + a 276 MB download.
+    if (opt_seed_matrix && opt_assign != ASSIGN_VALU && (size_t)M * (size_t)M * sizeof(T) <= ((size_t)1 << 30)) {
+      std::vector<T> hG, hb((size_t)M);
+      bool have_host = true;
+      try {
+        hG.resize((size_t)M * M);
+      } catch (const std::bad_alloc &) {
+        have_host = false;
+      }
+      T *G = nullptr;
+      if (have_host && dalloc(&G, (size_t)M * M) == 0) {
+        int grc = 0;
+        prof_begin("seed_gram");
+        grc = launch_transform<T>(stream, *Cc, *ccn, *Cc, *ccn, G, (int64_t)M, (int64_t)M, d, M, num_cu,
+                                  opt_split, split_scratch(M));
+        prof_end();
+        if (grc == 0) grc = download_rows(dev, stream, hG.data(), G, (size_t)M * M * sizeof(T));
+        if (grc == 0 && hipStreamSynchronize(stream) != hipSuccess) grc = H2O4GPU_KMEANS_EDEVICE;
+        (void)hipFree(G);
+        KM_TRY(grc);
+        int idx = pick(nullptr);
+        for (int c = 0; c < k; c++) {
+          seed_info.chosen[(size_t)c] = idx;
+          w[(size_t)idx] = 0;
+          if (c == k - 1) break;
+          const T *g = hG.data() + (size_t)idx * M;
+          if (c == 0) {
+            std::copy(g, g + M, hb.begin());
+          } else {
+            hb[(size_t)idx] = 0;  // (the reference takes the centre's own running value as 0)
+            for (int i = 0; i < M; i++) hb[(size_t)i] = g[i] < hb[(size_t)i] ? g[i] : hb[(size_t)i];
+          }
+          idx = pick(hb.data());
+        }
+        std::vector<int> rows((size_t)k);
+        for (int c = 0; c < k; c++) rows[(size_t)c] = all[(size_t)seed_info.chosen[(size_t)c]];
+        last_seed_rows = rows;
+        return init_from_rows(rows.data());
+      }
+      (void)hipGetLastError();  // no room for the matrix: one kernel per pick, below
+    }
     T *CcT = nullptr;
     int prc = 0;
     if (opt_assign == ASSIGN_VALU) {
@@ -1989,6 +2046,11 @@ KM_API int h2o4gpu_kmeans_set_option(h2o4gpu_kmeans_handle *h, const char *name,
   if (strcmp(name, "fuse") == 0) {
     if (value != 0 && value != 1) return H2O4GPU_KMEANS_EARG;
     h->opt_fuse = value;
+    return 0;
+  }
+  if (strcmp(name, "seed_matrix") == 0) {
+    if (value != 0 && value != 1) return H2O4GPU_KMEANS_EARG;
+    h->opt_seed_matrix = value;
     return 0;
   }
   return H2O4GPU_KMEANS_EARG;

@@ -244,6 +244,9 @@ int h2o4gpu_kmeans_transform_resident(h2o4gpu_kmeans_handle *h, void *d_dist);
  * h2o4gpu_kmeans_assign_variant() names what runs ("mfma_tiled_bf16x6", ...). The
  * environment variable H2O4GPU_KMEANS_FP32_SPLIT=6|9 sets it for every handle created
  * afterwards, the reference's four entry points included.
+ * "seed_matrix" = 1 (default) lets init_parallel compute the distances between its
+ * candidates as one matrix (while it fits 1 GiB) and pick the centres on the host from it;
+ * 0 runs one small kernel per pick, as "assign" = 1 always does.
  * Unknown names return EARG. */
 int h2o4gpu_kmeans_set_option(h2o4gpu_kmeans_handle *h, const char *name,
                               int value);

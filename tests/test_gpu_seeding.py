@@ -105,6 +105,41 @@ def test_matrix_core_rounds_differ_only_at_the_threshold(hip, oracle, n, d, k, s
         pos += len(b)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n,d,k,seed", [(20000, 32, 64, 3), (6000, 200, 300, 4), (3000, 7, 5, 2)])
+def test_picks_from_the_distance_matrix_and_from_a_kernel_per_pick_agree(hip, n, d, k, seed, dtype):
+    """The centres are picked either from one matrix of all distances between candidates
+    (the default) or with one kernel per pick (models whose matrix exceeds 1 GiB; option
+    seed_matrix = 0): the two sum the dot products in different orders, so the picks are the same
+    until two candidates' weighted distances tie within rounding (every later pick then depends
+    on which of the two was taken)."""
+    X = blobs(n, d, k, dtype, seed=n + d)
+    res = []
+    for matrix in (1, 0):
+        with hip.Handle(n, d, k, dtype) as h:
+            h.set_data(X)
+            h.set_option("seed_matrix", matrix)
+            h.init_parallel(seed)
+            info = h.parallel_seed_info()
+            res.append((info["cand_rows"], info["weights"], info["chosen"], h.centroids()))
+    assert len(res[0][0]) > k  # more candidates than centres: the picks do run
+    assert np.array_equal(res[0][0], res[1][0]) and np.array_equal(res[0][1], res[1][1])
+    ca, cb = res[0][2], res[1][2]
+    assert len(set(ca.tolist())) == k and len(set(cb.tolist())) == k
+    if np.array_equal(ca, cb):
+        assert np.array_equal(res[0][3], res[1][3])
+        return
+    p = int(np.argmax(ca != cb))  # first pick that differs: a tie within rounding
+    assert p > 0
+    cand = X[res[0][0]].astype(np.float64)
+    w = res[0][1].astype(np.float64).copy()
+    w[ca[:p]] = 0
+    best = ((cand[:, None, :] - cand[ca[:p]][None, :, :]) ** 2).sum(-1).min(1)
+    val = w * best
+    tol = 1e-4 if dtype == np.float32 else 1e-10
+    assert abs(val[ca[p]] - val[cb[p]]) <= tol * val.max(), (p, val[ca[p]], val[cb[p]], val.max())
+
+
 def test_fit_entry_point_seeds_with_kmeans_parallel(hip, oracle):
     """init_from_data == 1 through make_ptr_float_kmeans; zero iterations return the seeds."""
     from h2o4gpu_amd.libs import ch2o4gpu_gpu
