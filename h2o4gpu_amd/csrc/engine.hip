@@ -17,7 +17,9 @@
 #include <ctime>
 #include <limits>
 #include <map>
+#include <memory>
 #include <mutex>
+#include <new>
 #include <numeric>
 #include <random>
 #include <string>
@@ -1026,21 +1028,18 @@ struct Engine : h2o4gpu_kmeans_handle {
     // matrix and the sampler's two loops, with no launch and no wait: 8304 candidates of 784
     // features, 4095 picks: 57 ms of kernels and as many waits become 1 ms + a 276 MB download.
     if (opt_seed_matrix && opt_assign != ASSIGN_VALU && (size_t)M * (size_t)M * sizeof(T) <= ((size_t)1 << 30)) {
-      std::vector<T> hG, hb((size_t)M);
-      bool have_host = true;
-      try {
-        hG.resize((size_t)M * M);
-      } catch (const std::bad_alloc &) {
-        have_host = false;
-      }
+      std::vector<T> hb((size_t)M);
+      // (left uninitialised: the download fills it, and zeroing up to 1 GiB first costs as
+      // much as the download)
+      std::unique_ptr<T[]> hG(new (std::nothrow) T[(size_t)M * M]);
       T *G = nullptr;
-      if (have_host && dalloc(&G, (size_t)M * M) == 0) {
+      if (hG && dalloc(&G, (size_t)M * M) == 0) {
         int grc = 0;
         prof_begin("seed_gram");
         grc = launch_transform<T>(stream, *Cc, *ccn, *Cc, *ccn, G, (int64_t)M, (int64_t)M, d, M, num_cu,
                                   opt_split, split_scratch(M));
         prof_end();
-        if (grc == 0) grc = download_rows(dev, stream, hG.data(), G, (size_t)M * M * sizeof(T));
+        if (grc == 0) grc = download_rows(dev, stream, hG.get(), G, (size_t)M * M * sizeof(T));
         if (grc == 0 && hipStreamSynchronize(stream) != hipSuccess) grc = H2O4GPU_KMEANS_EDEVICE;
         (void)hipFree(G);
         KM_TRY(grc);
@@ -1049,7 +1048,7 @@ struct Engine : h2o4gpu_kmeans_handle {
           seed_info.chosen[(size_t)c] = idx;
           w[(size_t)idx] = 0;
           if (c == k - 1) break;
-          const T *g = hG.data() + (size_t)idx * M;
+          const T *g = hG.get() + (size_t)idx * M;
           if (c == 0) {
             std::copy(g, g + M, hb.begin());
           } else {
