@@ -155,6 +155,25 @@ def test_transform_in_several_batches(hip, dtype):
     assert np.max(np.abs(whole[:, rows].astype(np.float64) - want)) <= 64 * np.finfo(dtype).eps * scale
 
 
+@pytest.mark.parametrize("dtype,n,d,k", [(np.float32, 301234, 128, 200), (np.float64, 150001, 120, 20),
+                                         (np.float32, 2100000, 16, 8)])
+def test_predict_of_a_large_input_goes_up_in_pieces(hip, dtype, n, d, k):
+    """predict_host sends inputs of 128 MB and more to the device in pieces and assigns a piece
+    while the next one is in transfer (ragged last piece): the labels must be those of one
+    assignment pass over the same rows resident on the device."""
+    rng = np.random.default_rng(n)
+    X = rng.standard_normal((n, d)).astype(dtype)
+    assert X.nbytes >= 128 << 20
+    C = np.ascontiguousarray(X[rng.choice(n, size=k, replace=False)] + dtype(0.25))
+    with hip.Handle(n, d, k, dtype) as h:
+        h.set_data(X)
+        h.set_centroids(C)
+        h.assign()
+        want = h.labels()
+        got = h.predict(X)
+    assert np.array_equal(got, want)
+
+
 def test_bad_arguments_return_codes(shim):
     X = np.zeros((10, 2), np.float32)
     pc, pl = np.zeros(4, np.float32), np.zeros(10, np.int32)
