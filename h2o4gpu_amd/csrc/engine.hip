@@ -326,13 +326,31 @@ struct StagingPool {
     char *dst = nullptr;
     const char *src = nullptr;
     size_t bytes = 0, per = 0;
+    // width != 0: src is the stretch [base, base + bytes) of a dense [rows][width] byte matrix
+    // and dst the start of a matrix of the same rows `pitch` bytes apart
+    size_t width = 0, pitch = 0, base = 0;
     pid_t owner = 0;
   };
   Workers *workers = nullptr;
 
+  static void copy_bytes(char *dst, const char *src, size_t lo, size_t len, size_t width, size_t pitch,
+                         size_t base) {
+    if (width == 0) {
+      memcpy(dst + lo, src + lo, len);
+      return;
+    }
+    const char *s = src + lo;
+    for (size_t f = base + lo, end = base + lo + len; f < end;) {
+      const size_t row = f / width, col = f - row * width;
+      const size_t run = std::min(width - col, end - f);
+      memcpy(dst + row * pitch + col, s, run);
+      s += run;
+      f += run;
+    }
+  }
   static void copy_part(Workers *w, int part) {
     const size_t lo = w->per * (size_t)part;
-    if (lo < w->bytes) memcpy(w->dst + lo, w->src + lo, std::min(w->per, w->bytes - lo));
+    if (lo < w->bytes) copy_bytes(w->dst, w->src, lo, std::min(w->per, w->bytes - lo), w->width, w->pitch, w->base);
   }
   static void worker_main(Workers *w, int index) {
     long seen = 0;
@@ -347,16 +365,17 @@ struct StagingPool {
       if (--w->pending == 0) w->done.notify_one();
     }
   }
-  void parallel_copy(char *dst, const char *src, size_t bytes, int threads) {
+  void parallel_copy(char *dst, const char *src, size_t bytes, int threads, size_t width = 0, size_t pitch = 0,
+                     size_t base = 0) {
     if (threads <= 1 || bytes < (4u << 20)) {
-      memcpy(dst, src, bytes);
+      copy_bytes(dst, src, 0, bytes, width, pitch, base);
       return;
     }
     // (a forked child has the parent's pool object but none of its threads)
     if (!workers || workers->owner != getpid() || (int)workers->threads.size() + 1 < threads) {
       Workers *w = new (std::nothrow) Workers();
       if (!w) {
-        memcpy(dst, src, bytes);
+        copy_bytes(dst, src, 0, bytes, width, pitch, base);
         return;
       }
       w->owner = getpid();
@@ -375,6 +394,9 @@ struct StagingPool {
       w->dst = dst;
       w->src = src;
       w->bytes = bytes;
+      w->width = width;
+      w->pitch = pitch;
+      w->base = base;
       w->per = ((bytes + parts - 1) / parts + 4095) & ~(size_t)4095;
       w->parts = parts;
       w->pending = nworkers;
@@ -447,7 +469,12 @@ struct StagingPool {
   }
 
   // The way back: the DMA engine fills one buffer while host threads copy the other out.
-  int download(int dev, hipStream_t stream, void *dst, const void *src, size_t bytes) {
+  // width != 0: the device bytes are a dense [bytes / width][width] matrix whose rows go to
+  // dst `pitch` bytes apart (a batch of columns of a wider host matrix). ready: the event
+  // after the kernels that produce src, when the stream has later work queued that the
+  // download need not wait for.
+  int download(int dev, hipStream_t stream, void *dst, const void *src, size_t bytes, size_t width = 0,
+               size_t pitch = 0, hipEvent_t ready = nullptr) {
     if (dev < 0 || dev >= MAX_DEV || bytes < MIN_STAGED) return 1;
     std::lock_guard<std::mutex> lock(mu);
     if (!ensure(dev)) return 1;
@@ -457,7 +484,8 @@ struct StagingPool {
     if (threads < 1) threads = 1;
     const size_t piece = piece_size(bytes);
     const size_t chunks = (bytes + piece - 1) / piece;
-    KM_HIP_TRY(hipStreamSynchronize(stream));  // the kernels that produce src
+    if (ready) KM_HIP_TRY(hipEventSynchronize(ready));
+    else KM_HIP_TRY(hipStreamSynchronize(stream));  // the kernels that produce src
     for (size_t c = 0; c <= chunks; c++) {
       const int b = (int)(c & 1);
       if (c < chunks) {
@@ -469,8 +497,12 @@ struct StagingPool {
       if (c >= 1) {  // chunk c-1 sits in the other buffer
         const size_t off = (c - 1) * piece, len = std::min(piece, bytes - off);
         KM_HIP_TRY(hipEventSynchronize(done[dev][b ^ 1]));
-        parallel_copy(static_cast<char *>(dst) + off, static_cast<const char *>(buf[dev][b ^ 1]), len,
-                      threads);
+        if (width == 0)
+          parallel_copy(static_cast<char *>(dst) + off, static_cast<const char *>(buf[dev][b ^ 1]), len,
+                        threads);
+        else
+          parallel_copy(static_cast<char *>(dst), static_cast<const char *>(buf[dev][b ^ 1]), len, threads,
+                        width, pitch, off);
       }
     }
     return 0;
@@ -498,6 +530,18 @@ static int download_rows(int dev, hipStream_t stream, void *dst, const void *src
   const int rc = g_staging.download(dev, stream, dst, src, bytes);
   if (rc <= 0) return rc;
   KM_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, stream));
+  return 0;
+}
+
+// A dense device matrix of `height` rows of `width` bytes into host rows `pitch` bytes apart;
+// `ready` as in StagingPool::download. Returns after the bytes have arrived.
+static int download_matrix(int dev, hipStream_t stream, void *dst, size_t pitch, const void *src, size_t width,
+                           size_t height, hipEvent_t ready) {
+  const int rc = g_staging.download(dev, stream, dst, src, width * height, width, pitch, ready);
+  if (rc <= 0) return rc;
+  if (ready) KM_HIP_TRY(hipEventSynchronize(ready));
+  else KM_HIP_TRY(hipStreamSynchronize(stream));
+  KM_HIP_TRY(hipMemcpy2D(dst, pitch, src, width, width, height, hipMemcpyDeviceToHost));
   return 0;
 }
 
@@ -1459,7 +1503,11 @@ struct Engine : h2o4gpu_kmeans_handle {
 
   // The n x k result is produced in row batches of at most ~4 GB so the device
   // buffer stays bounded; the reference materialises it whole ("TODO batch
-  // this", kmeans_h2o4gpu.cu:936).
+  // this", kmeans_h2o4gpu.cu:936). With more than one batch there are two sets of device
+  // buffers: the kernels of batch i + 1 are queued before the host starts to bring batch i
+  // back, so they run under that download, and a batch's [k][its rows] block goes through
+  // the pinned staging buffers into its columns of the caller's [k][rows] matrix (a strided
+  // copy straight into pageable memory moved a quarter of the bytes per second).
   int transform_host(size_t rows, const void *hX, void *hD) override {
     KM_HIP_TRY(hipSetDevice(dev));
     if (!have_centroids || sets > 1) return H2O4GPU_KMEANS_ESTATE;
@@ -1468,37 +1516,59 @@ struct Engine : h2o4gpu_kmeans_handle {
     batch = batch / 128 * 128;
     if (batch < 128) batch = 128;
     if (batch > rows) batch = rows;
-    T *dX = nullptr, *dxn = nullptr, *dD = nullptr;
-    int rc = dalloc(&dX, batch * d);
-    if (rc == 0) rc = dalloc(&dxn, batch);
-    if (rc == 0) rc = dalloc(&dD, batch * k);
-    for (size_t lo = 0; rc == 0 && lo < rows; lo += batch) {
-      const size_t cur_rows = std::min(batch, rows - lo);
-      rc = run_transform_batch(lo, cur_rows, rows, hX, hD, dX, dxn, dD);
+    const size_t nbatch = (rows + batch - 1) / batch;
+    const int nbuf = nbatch > 1 ? 2 : 1;
+    T *dX[2] = {nullptr, nullptr}, *dxn[2] = {nullptr, nullptr}, *dD[2] = {nullptr, nullptr};
+    hipEvent_t ready[2] = {nullptr, nullptr};
+    int rc = ensure_cnorm();
+    for (int b = 0; b < nbuf && rc == 0; b++) {
+      rc = dalloc(&dX[b], batch * d);
+      if (rc == 0) rc = dalloc(&dxn[b], batch);
+      if (rc == 0) rc = dalloc(&dD[b], batch * k);
+      if (rc == 0 && hipEventCreateWithFlags(&ready[b], hipEventDisableTiming) != hipSuccess) {
+        (void)hipGetLastError();
+        rc = H2O4GPU_KMEANS_EDEVICE;
+      }
+    }
+    const SplitScratch scratch = rc == 0 ? split_scratch() : SplitScratch();
+    // upload + kernels of batch i, left running
+    auto queue_batch = [&](size_t i) -> int {
+      const size_t lo = i * batch, cur_rows = std::min(batch, rows - lo);
+      const int b = (int)(i % (size_t)nbuf);
+      // (nothing on the stream touches this buffer: its last kernels ended before the
+      // download of batch i - 2 returned)
+      KM_TRY(upload_rows(dev, stream, dX[b], static_cast<const T *>(hX) + lo * d, cur_rows * d * sizeof(T),
+                         false));
+      PROFILED("row_norms", launch_row_norms<T>(stream, dX[b], dxn[b], (int64_t)cur_rows, d));
+      PROFILED("transform", launch_transform<T>(stream, dX[b], dxn[b], C[cur], cnorm, dD[b],
+                                                (int64_t)cur_rows, (int64_t)cur_rows, d, k, num_cu,
+                                                opt_split, scratch));
+      KM_HIP_TRY(hipEventRecord(ready[b], stream));
+      return 0;
+    };
+    if (rc == 0) rc = queue_batch(0);
+    for (size_t i = 0; rc == 0 && i < nbatch; i++) {
+      if (i + 1 < nbatch) rc = queue_batch(i + 1);
+      if (rc != 0) break;
+      const size_t lo = i * batch, cur_rows = std::min(batch, rows - lo);
+      const int b = (int)(i % (size_t)nbuf);
+      T *dst = static_cast<T *>(hD) + lo;
+      if (nbatch == 1) {  // one contiguous [k][rows] block
+        rc = download_rows(dev, stream, dst, dD[b], (size_t)k * rows * sizeof(T));
+        if (rc == 0 && hipStreamSynchronize(stream) != hipSuccess) rc = H2O4GPU_KMEANS_EDEVICE;
+      } else {
+        rc = download_matrix(dev, stream, dst, rows * sizeof(T), dD[b], cur_rows * sizeof(T), (size_t)k,
+                             ready[b]);
+      }
     }
     (void)hipStreamSynchronize(stream);
-    if (dX) (void)hipFree(dX);
-    if (dxn) (void)hipFree(dxn);
-    if (dD) (void)hipFree(dD);
+    for (int b = 0; b < 2; b++) {
+      if (dX[b]) (void)hipFree(dX[b]);
+      if (dxn[b]) (void)hipFree(dxn[b]);
+      if (dD[b]) (void)hipFree(dD[b]);
+      if (ready[b]) (void)hipEventDestroy(ready[b]);
+    }
     return rc;
-  }
-  int run_transform_batch(size_t lo, size_t cur_rows, size_t rows, const void *hX, void *hD,
-                          T *dX, T *dxn, T *dD) {
-    const T *src = static_cast<const T *>(hX) + lo * d;
-    KM_TRY(ensure_cnorm());
-    KM_TRY(upload_rows(dev, stream, dX, src, cur_rows * d * sizeof(T)));
-    PROFILED("row_norms", launch_row_norms<T>(stream, dX, dxn, (int64_t)cur_rows, d));
-    PROFILED("transform", launch_transform<T>(stream, dX, dxn, C[cur], cnorm, dD,
-                                              (int64_t)cur_rows, (int64_t)cur_rows, d, k, num_cu,
-                                              opt_split, split_scratch()));
-    T *dst = static_cast<T *>(hD) + lo;
-    if (cur_rows == rows)  // a single batch is one contiguous [k][rows] block
-      KM_TRY(download_rows(dev, stream, dst, dD, (size_t)k * rows * sizeof(T)));
-    else
-      KM_HIP_TRY(hipMemcpy2DAsync(dst, rows * sizeof(T), dD, cur_rows * sizeof(T),
-                                  cur_rows * sizeof(T), (size_t)k, hipMemcpyDeviceToHost, stream));
-    KM_HIP_TRY(hipStreamSynchronize(stream));
-    return 0;
   }
   int transform_resident(void *d_dist) override {
     KM_HIP_TRY(hipSetDevice(dev));
