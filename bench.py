@@ -193,6 +193,22 @@ def c_abi_fit(X, C0, iters):
                     "malloc'ed results out"}
 
 
+def seeding_seconds(X, k, seed=7):
+    """The reference's default start (k-means||, then its host k-means++ over the candidates)
+    on rows already resident: not part of a step, reported beside it."""
+    from h2o4gpu_amd.libs import kmeans_hip
+    n, d = X.shape
+    with kmeans_hip.Handle(n, d, k, X.dtype) as h:
+        h.set_data(X)
+        h.init_parallel(seed)  # (first call: lazy set-up)
+        t0 = time.perf_counter()
+        h.init_parallel(seed + 1)
+        dt = time.perf_counter() - t0
+        info = h.parallel_seed_info()
+    return {"seconds": dt, "candidates": int(len(info["cand_rows"])),
+            "note": "init_from_data=1 on resident rows: rounds of k-means||, weights, k picks"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -394,6 +410,7 @@ def main():
         out["cpu_reference_path"] = sklearn_baseline(X, C0, args.sklearn_rows)
     if args.end_to_end:
         out["c_abi_fit"] = c_abi_fit(X, C0, datasets.SHAPES[args.workload][4])
+        out["kmeans_parallel_seeding"] = seeding_seconds(X, k)
     print(json.dumps(out), flush=True)
     return 0
 
