@@ -155,6 +155,29 @@ def test_transform_in_several_batches(hip, dtype):
     assert np.max(np.abs(whole[:, rows].astype(np.float64) - want)) <= 64 * np.finfo(dtype).eps * scale
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_transform_batches_through_the_staging_buffers(hip, dtype):
+    """Batches of 24 MB and more come back through the pinned staging buffers, each batch's
+    [k][its rows] block scattered into its columns of the [k][rows] result while the next
+    batch is computed: the result must be the single-batch one, bit for bit (ragged last batch,
+    batch widths that do not divide the 16 MB staging chunk)."""
+    n, d, k = 200003, 16, 130
+    rng = np.random.default_rng(5)
+    X = rng.standard_normal((n, d)).astype(dtype)
+    C = rng.standard_normal((k, d)).astype(dtype)
+    with hip.Handle(k, d, k, dtype) as h:
+        h.set_centroids(C)
+        whole = h.transform(X)
+        for mb in (32, 40):
+            h.set_option("transform_batch_mb", mb)
+            assert n * k * np.dtype(dtype).itemsize > 2 * (mb << 20)  # three batches or more
+            assert np.array_equal(h.transform(X), whole)
+    rows = rng.choice(n, size=100, replace=False)
+    want = ((X[rows][:, None, :].astype(np.float64) - C[None].astype(np.float64)) ** 2).sum(-1).T
+    scale = 2 * (X.astype(np.float64) ** 2).sum(1).max()
+    assert np.max(np.abs(whole[:, rows].astype(np.float64) - want)) <= 64 * np.finfo(dtype).eps * scale
+
+
 @pytest.mark.parametrize("dtype,n,d,k", [(np.float32, 301234, 128, 200), (np.float64, 150001, 120, 20),
                                          (np.float32, 2100000, 16, 8)])
 def test_predict_of_a_large_input_goes_up_in_pieces(hip, dtype, n, d, k):
