@@ -946,8 +946,20 @@ struct Engine : h2o4gpu_kmeans_handle {
     // whether `recent` has been through a pass yet.
     int recent_off = 0;
     bool measured = false;
+    // A round that adds no candidate leaves `recent` as it was: the next round would measure
+    // the same candidates again, find the same costs, the same potential and, the thresholds
+    // depending on (seed, row) alone, the same empty selection. Such rounds are not run; their
+    // potential and count are the previous round's.
+    bool settled = false;
     for (int counter = 0; counter < rounds; counter++) {
       log_msg(verbose, LOG_VERBOSE, "KMeans|| - Iteration %d.", counter);
+      if (settled) {
+        seed_info.phi[counter] = seed_info.phi[counter - 1];
+        seed_info.round_count[counter] = 0;
+        log_msg(verbose, LOG_VERBOSE, "KMeans|| - Total min cost from centers %g.", seed_info.phi[counter]);
+        if (seed_info.phi[counter] != 0) log_msg(verbose, LOG_VERBOSE, "KMeans|| - New potential centroids %d.", 0);
+        continue;
+      }
       KM_TRY(stage(recent));
       // minimum distance to this round's candidates, compared as floats (no integer keys)
       PROFILED("seed_assign", launch_assign<T>(stream, opt_assign, X, xnorm, *Cc, *ccn, labels, mindist,
@@ -964,7 +976,10 @@ struct Engine : h2o4gpu_kmeans_handle {
       const T total = (T)sum;
       seed_info.phi[counter] = (double)total;
       log_msg(verbose, LOG_VERBOSE, "KMeans|| - Total min cost from centers %g.", (double)total);
-      if (total == (T)0) continue;
+      if (total == (T)0) {
+        settled = true;
+        continue;
+      }
       KM_HIP_TRY(hipMemsetAsync(*dcount, 0, sizeof(int), stream));
       PROFILED("seed_select", launch_select_rows<T>(stream, *cost, total, state0, k, *list, *dcount,
                                                     list_cap, n));
@@ -974,6 +989,7 @@ struct Engine : h2o4gpu_kmeans_handle {
       if (count > list_cap) count = list_cap;  // (cannot happen: one entry per row at most)
       seed_info.round_count[counter] = count;
       log_msg(verbose, LOG_VERBOSE, "KMeans|| - New potential centroids %d.", count);
+      if (count == 0) settled = true;
       if (count > 0) {
         recent.resize((size_t)count);
         KM_HIP_TRY(hipMemcpyAsync(recent.data(), *list, (size_t)count * sizeof(int), hipMemcpyDeviceToHost,
