@@ -183,6 +183,7 @@ struct h2o4gpu_kmeans_handle {
   int opt_buckets = 1;  // 1: bucketed centroid sums where the sums do not fit LDS
   int opt_exact = 0;    // 1: float32 MFMA argmin on the float distances, not on 16-ulp keys
   int opt_split = 0;    // 6 or 9: float32 matrix-core kernels as that many bfloat16 products per feature pair
+  int opt_transform_buffers = 2;  // sets of device buffers of a transform in several batches
   int opt_seed_matrix = 1;  // k-means||: distances between candidates as one matrix (0: a kernel per pick)
   int opt_transform_batch_mb = 4096;  // device buffer of transform_host's output, per batch of rows
   int last_variant = ASSIGN_AUTO;
@@ -1533,18 +1534,30 @@ struct Engine : h2o4gpu_kmeans_handle {
     if (batch < 128) batch = 128;
     if (batch > rows) batch = rows;
     const size_t nbatch = (rows + batch - 1) / batch;
-    const int nbuf = nbatch > 1 ? 2 : 1;
+    int nbuf = nbatch > 1 && opt_transform_buffers == 2 ? 2 : 1;
     T *dX[2] = {nullptr, nullptr}, *dxn[2] = {nullptr, nullptr}, *dD[2] = {nullptr, nullptr};
     hipEvent_t ready[2] = {nullptr, nullptr};
     int rc = ensure_cnorm();
     for (int b = 0; b < nbuf && rc == 0; b++) {
-      rc = dalloc(&dX[b], batch * d);
-      if (rc == 0) rc = dalloc(&dxn[b], batch);
-      if (rc == 0) rc = dalloc(&dD[b], batch * k);
-      if (rc == 0 && hipEventCreateWithFlags(&ready[b], hipEventDisableTiming) != hipSuccess) {
+      int arc = dalloc(&dX[b], batch * d);
+      if (arc == 0) arc = dalloc(&dxn[b], batch);
+      if (arc == 0) arc = dalloc(&dD[b], batch * k);
+      if (arc == 0 && hipEventCreateWithFlags(&ready[b], hipEventDisableTiming) != hipSuccess) {
         (void)hipGetLastError();
-        rc = H2O4GPU_KMEANS_EDEVICE;
+        arc = H2O4GPU_KMEANS_EDEVICE;
       }
+      if (arc != 0 && b == 1) {
+        // no room for the second set: one batch at a time, each downloaded before the next is computed
+        if (dX[1]) (void)hipFree(dX[1]);
+        if (dxn[1]) (void)hipFree(dxn[1]);
+        if (dD[1]) (void)hipFree(dD[1]);
+        if (ready[1]) (void)hipEventDestroy(ready[1]);
+        dX[1] = dxn[1] = dD[1] = nullptr;
+        ready[1] = nullptr;
+        nbuf = 1;
+        break;
+      }
+      rc = arc;
     }
     const SplitScratch scratch = rc == 0 ? split_scratch() : SplitScratch();
     // upload + kernels of batch i, left running
@@ -1564,7 +1577,8 @@ struct Engine : h2o4gpu_kmeans_handle {
     };
     if (rc == 0) rc = queue_batch(0);
     for (size_t i = 0; rc == 0 && i < nbatch; i++) {
-      if (i + 1 < nbatch) rc = queue_batch(i + 1);
+      if (i > 0 && nbuf == 1) rc = queue_batch(i);  // (the only buffers are free again)
+      if (nbuf == 2 && i + 1 < nbatch && rc == 0) rc = queue_batch(i + 1);
       if (rc != 0) break;
       const size_t lo = i * batch, cur_rows = std::min(batch, rows - lo);
       const int b = (int)(i % (size_t)nbuf);
@@ -2149,6 +2163,11 @@ KM_API int h2o4gpu_kmeans_set_option(h2o4gpu_kmeans_handle *h, const char *name,
   if (strcmp(name, "fuse") == 0) {
     if (value != 0 && value != 1) return H2O4GPU_KMEANS_EARG;
     h->opt_fuse = value;
+    return 0;
+  }
+  if (strcmp(name, "transform_buffers") == 0) {
+    if (value != 1 && value != 2) return H2O4GPU_KMEANS_EARG;
+    h->opt_transform_buffers = value;
     return 0;
   }
   if (strcmp(name, "seed_matrix") == 0) {

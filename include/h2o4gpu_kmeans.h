@@ -244,6 +244,9 @@ int h2o4gpu_kmeans_transform_resident(h2o4gpu_kmeans_handle *h, void *d_dist);
  * h2o4gpu_kmeans_assign_variant() names what runs ("mfma_tiled_bf16x6", ...). The
  * environment variable H2O4GPU_KMEANS_FP32_SPLIT=6|9 sets it for every handle created
  * afterwards, the reference's four entry points included.
+ * "transform_buffers" = 2 (default) gives a transform in several batches two sets of device
+ * buffers, so that a batch is computed while the previous one is downloaded (this is also
+ * what happens with 1, one batch at a time, when the second set cannot be allocated).
  * "seed_matrix" = 1 (default) lets init_parallel compute the distances between its
  * candidates as one matrix (while it fits 1 GiB) and pick the centres on the host from it;
  * 0 runs one small kernel per pick, as "assign" = 1 always does.

@@ -172,6 +172,9 @@ def test_transform_batches_through_the_staging_buffers(hip, dtype):
             h.set_option("transform_batch_mb", mb)
             assert n * k * np.dtype(dtype).itemsize > 2 * (mb << 20)  # three batches or more
             assert np.array_equal(h.transform(X), whole)
+        # one set of device buffers (what a failed allocation of the second set falls back to)
+        h.set_option("transform_buffers", 1)
+        assert np.array_equal(h.transform(X), whole)
     rows = rng.choice(n, size=100, replace=False)
     want = ((X[rows][:, None, :].astype(np.float64) - C[None].astype(np.float64)) ** 2).sum(-1).T
     scale = 2 * (X.astype(np.float64) ** 2).sum(1).max()
