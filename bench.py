@@ -410,7 +410,10 @@ def main():
         out["cpu_reference_path"] = sklearn_baseline(X, C0, args.sklearn_rows)
     if args.end_to_end:
         out["c_abi_fit"] = c_abi_fit(X, C0, datasets.SHAPES[args.workload][4])
-        out["kmeans_parallel_seeding"] = seeding_seconds(X, k)
+        try:
+            out["kmeans_parallel_seeding"] = seeding_seconds(X, k)
+        except Exception as e:  # an extra: never the reason a bench line is missing
+            out["kmeans_parallel_seeding"] = {"error": repr(e)}
     print(json.dumps(out), flush=True)
     return 0
 
