@@ -1351,6 +1351,13 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
       const vec_t *ap = reinterpret_cast<const vec_t *>(As + buf * A_ELEMS);
       const vec_t *bp = reinterpret_cast<const vec_t *>(Bs + buf * B_ELEMS);
       const int nq_st = DTAIL ? stage_nq(st) : NV;
+      // Whole stages are one basic block of matrix instructions and operand reads: the
+      // compiler's interleaving strategy for such blocks spreads the reads between the matrix
+      // instructions instead of bunching them in front (256-centroid block, 500k x 784,
+      // k = 4096: 25.71 -> 24.51 ms, 200k x 784: 11.32 -> 10.94 ms; the 128-centroid block and the
+      // double kernels measured the same with and without it, the per-step blocks of the DTAIL
+      // kernels do not benefit).
+      if constexpr (!DTAIL && SPLIT == 0 && sizeof(T) == 4) __builtin_amdgcn_iglp_opt(0);
 #pragma unroll
       for (int q = 0; q < (SPLIT ? 0 : NV); q++) {
         if (DTAIL && q >= nq_st) continue;  // nothing of this stage there
