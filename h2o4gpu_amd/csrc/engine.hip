@@ -629,9 +629,12 @@ struct Engine : h2o4gpu_kmeans_handle {
     hipError_t e = hipMalloc(reinterpret_cast<void **>(p), count * sizeof(U));
     if (e != hipSuccess) {
       (void)hipGetLastError();
-      log_msg(verbose ? verbose : LOG_ERROR, LOG_ERROR,
-              "device allocation of %zu bytes failed: %s", count * sizeof(U),
-              hipGetErrorString(e));
+      // the reference's message and level (log_error(verbose, ...), kmeans_impl.h:81-94):
+      // printed when verbose >= 200, and the call returns -1
+      log_msg(verbose, LOG_ERROR,
+              "Unable to allocate memory for gpu: %d | n: %lld | k: %d | d: %d | error: %s "
+              "(%zu bytes)",
+              dev, (long long)n, k, d, hipGetErrorString(e), count * sizeof(U));
       return H2O4GPU_KMEANS_EALLOC;
     }
     return 0;
@@ -827,9 +830,12 @@ struct Engine : h2o4gpu_kmeans_handle {
     std::vector<double> bs((size_t)nb);
     std::vector<T> blk(KPP_BLOCK);
     idx[0] = first(gen);
+    // per-row scratch of the seeding: the selected set's own block of a stacked handle
+    T *const md = mindist + row_off();
+    int *const lb = labels + row_off();
     for (int c = 1; c <= k; c++) {
       PROFILED("min_dist_update",
-               launch_min_dist_update<T>(stream, X, xnorm, idx[c - 1], mindist, labels,
+               launch_min_dist_update<T>(stream, X, xnorm, idx[c - 1], md, lb,
                                          kpp_rows, kpp_dcc, c - 1, kpp_bsums, n, d));
       if (c == k) break;
       KM_HIP_TRY(hipMemcpyAsync(bs.data(), kpp_bsums, (size_t)nb * sizeof(double),
@@ -852,7 +858,7 @@ struct Engine : h2o4gpu_kmeans_handle {
         }
         const int64_t lo = b * KPP_BLOCK;
         const int cntb = (int)std::min<int64_t>(KPP_BLOCK, n - lo);
-        KM_HIP_TRY(hipMemcpyAsync(blk.data(), mindist + lo, (size_t)cntb * sizeof(T),
+        KM_HIP_TRY(hipMemcpyAsync(blk.data(), md + lo, (size_t)cntb * sizeof(T),
                                   hipMemcpyDeviceToHost, stream));
         KM_HIP_TRY(hipStreamSynchronize(stream));
         int i = 0, last_pos = 0;
@@ -922,6 +928,10 @@ struct Engine : h2o4gpu_kmeans_handle {
     const int64_t nb = (n + KPP_BLOCK - 1) / KPP_BLOCK;
     size_t cap_model = 0, cap_norm = 0, cap_idx = 0, cap_best = 0;
     const int list_cap = (int)n;
+    // per-row scratch of the rounds: the selected set's own block of a stacked handle (the
+    // block that init_parallel clears afterwards)
+    T *const md = mindist + row_off();
+    int *const lb = labels + row_off();
     KM_TRY(dalloc(cost, n));
     KM_TRY(dalloc(near, n));
     KM_TRY(dalloc(list, list_cap));
@@ -963,10 +973,10 @@ struct Engine : h2o4gpu_kmeans_handle {
       }
       KM_TRY(stage(recent));
       // minimum distance to this round's candidates, compared as floats (no integer keys)
-      PROFILED("seed_assign", launch_assign<T>(stream, opt_assign, X, xnorm, *Cc, *ccn, labels, mindist,
+      PROFILED("seed_assign", launch_assign<T>(stream, opt_assign, X, xnorm, *Cc, *ccn, lb, md,
                                                n, d, (int)recent.size(), num_cu, nullptr, true, StackShape(),
                                                opt_split, split_scratch((int)recent.size())));
-      PROFILED("seed_fold", launch_fold_min<T>(stream, mindist, *cost, kpp_bsums, n, counter == 0, labels, *near,
+      PROFILED("seed_fold", launch_fold_min<T>(stream, md, *cost, kpp_bsums, n, counter == 0, lb, *near,
                                                recent_off));
       measured = true;
       KM_HIP_TRY(hipMemcpyAsync(bs.data(), kpp_bsums, (size_t)nb * sizeof(double), hipMemcpyDeviceToHost,
@@ -1022,10 +1032,10 @@ struct Engine : h2o4gpu_kmeans_handle {
     // not been through a pass yet.
     if (!measured) {
       KM_TRY(stage(recent));
-      PROFILED("seed_weights", launch_assign<T>(stream, opt_assign, X, xnorm, *Cc, *ccn, labels, mindist, n, d,
+      PROFILED("seed_weights", launch_assign<T>(stream, opt_assign, X, xnorm, *Cc, *ccn, lb, md, n, d,
                                                 (int)recent.size(), num_cu, nullptr, true, StackShape(),
                                                 opt_split, split_scratch((int)recent.size())));
-      PROFILED("seed_fold", launch_fold_min<T>(stream, mindist, *cost, kpp_bsums, n, 0, labels, *near, recent_off));
+      PROFILED("seed_fold", launch_fold_min<T>(stream, md, *cost, kpp_bsums, n, 0, lb, *near, recent_off));
     }
     KM_TRY(stage(all));  // the picks below read all candidates
     int *dhist = nullptr;
@@ -1738,7 +1748,8 @@ static int fit_entry(int verbose, int seed, int gpu_id, size_t rows, size_t cols
   if (rc != 0) {
     free(oc);
     free(ol);
-    log_msg(verbose ? verbose : LOG_ERROR, LOG_ERROR, "KMeans algorithm failed (%d).", rc);
+    // kmeans_h2o4gpu.cu:758-761
+    log_msg(verbose, LOG_ERROR, "KMeans algorithm failed (%d).", rc);
     return rc;
   }
   *pred_centroids = oc;

@@ -14,7 +14,12 @@ on top of the gfx950 engine. Differences, all additive:
     that name); `'k-means||'` is accepted as a second name for it and `'d2-sampling'`
     selects textbook k-means++ (one centre per pass, drawn proportionally to the squared
     distance to the nearest chosen centre);
-  * `n_init` restarts, `n_iter_` and a native `score`;
+  * `n_init` restarts, `n_iter_` and a native `score`. Restarts run stacked through the
+    matrix-core kernel wherever the shape allows; a single fit of a small model (k <= 16,
+    d <= 64) runs the scalar-order kernels instead, so restart r of an `n_init` fit equals
+    the `n_init=1` fit with `random_state + r` up to rows whose two nearest centroids are a
+    near-tie (1e-5 relative), not bit for bit; `labels_` always come from an ordinary relabel
+    against the returned centroids, so they equal `predict` on the same rows;
   * fit / predict / score / transform accept rows that already live on the GPU (any
     object with `__cuda_array_interface__`, e.g. a PyTorch-ROCm tensor): the engine adopts
     the pointer, nothing crosses PCIe (the reference re-uploads the rows on every call,

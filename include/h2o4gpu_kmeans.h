@@ -294,8 +294,14 @@ int h2o4gpu_kmeans_copy_probe(int gpu_id, size_t bytes, int reps,
  * more returns H2O4GPU_KMEANS_ESCRATCH and queues nothing. All calls on one
  * device share that array: calls that overlap in time on one device (other
  * threads, other streams) race; serialise them. The first call on a device
- * looks up the array's address and the device's properties and should be made
- * outside graph capture.
+ * looks up the array's address and the device's properties, and the first call
+ * of a process for a new kind of shape (a kernel instance that needs more than
+ * 64 KB of LDS: wide rows, large models) sets that kernel's LDS limit once
+ * (hipFuncSetAttribute): make one call per shape that will be used outside
+ * graph capture first. The float32 arithmetic is always the float32 matrix
+ * instructions': the environment variable H2O4GPU_KMEANS_FP32_SPLIT, which
+ * switches handles to bfloat16 parts, is not read here, so with it set the
+ * labels can differ from h2o4gpu_kmeans_predict_host's on near-tie rows.
  * ------------------------------------------------------------------------- */
 #define H2O4GPU_KMEANS_NOALLOC_SCRATCH_BYTES (16u << 20)
 int h2o4gpu_kmeans_predict_device_noalloc(int elem_size, size_t rows, size_t cols,

@@ -24,3 +24,24 @@ def hip():
     from h2o4gpu_amd.libs import kmeans_hip
     kmeans_hip.lib()
     return kmeans_hip
+
+
+_FULL_DATA = {}
+
+
+@pytest.fixture(scope="session")
+def full_data():
+    """full_data(name, dtype) -> (X, k, iterations) of a benchmark shape at its full size,
+    generated once per session (the five shapes take 1.5 minutes to draw; both full-size test
+    files use them). About 11 GB of host memory when every shape has been asked for."""
+    import numpy as np
+    from h2o4gpu_amd import datasets
+
+    def get(name, dtype):
+        key = (name, np.dtype(dtype).name)
+        if key not in _FULL_DATA:
+            X, k, iters = datasets.make(name, 1.0, dtype)
+            X.setflags(write=False)
+            _FULL_DATA[key] = (X, k, iters)
+        return _FULL_DATA[key]
+    return get

@@ -214,12 +214,12 @@ FULL = [
 
 @pytest.mark.timeout(900)
 @pytest.mark.parametrize("name,dtype,iters,e2e_iters", FULL)
-def test_full_shape(hip, oracle, name, dtype, iters, e2e_iters):
+def test_full_shape(hip, oracle, full_data, name, dtype, iters, e2e_iters):
     """A benchmark configuration at its full size: lock-step against the oracle on all rows
     at the start and at the fitted centroids, end to end for a fixed number of iterations,
     and the size-independent properties of a fit (monotone objective, predict reproduces
     the labels, counts add up, centroids are means). C5 also transforms 100,000 held-out rows."""
-    X, k, _ = datasets.make(name, 1.0, dtype)
+    X, k, _ = full_data(name, dtype)
     n, d = X.shape
     tag = "%s %s" % (name, np.dtype(dtype).name)
     rng = np.random.default_rng(99)

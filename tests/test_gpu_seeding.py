@@ -140,6 +140,37 @@ def test_picks_from_the_distance_matrix_and_from_a_kernel_per_pick_agree(hip, n,
     assert abs(val[ca[p]] - val[cb[p]]) <= tol * val.max(), (p, val[ca[p]], val[cb[p]], val.max())
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n,d,k,seed", [(40000, 32, 64, 3), (9000, 200, 300, 4), (25000, 16, 24, 6),
+                                        (15000, 100, 600, 2)])
+def test_default_path_weights_equal_one_pass_over_all_candidates(hip, oracle, n, d, k, seed, dtype):
+    """The weights come from the nearest candidate noted round by round, and with the default
+    (matrix-core) kernels every round's model has another size and may run another kernel family,
+    so a row's distances to candidates of different rounds need not be summed alike. The
+    reference counts the rows per nearest candidate in ONE pass over all candidates
+    (count_pts_per_centroid, kmeans_h2o4gpu.h:90-126): the engine's weights may differ from that
+    pass only by rows whose two nearest candidates are a near-tie (1e-5 relative gap, or the
+    rounding floor 8 eps (|x|^2 + |c|^2) of the expanded form), each of which moves one unit
+    of weight from one candidate to another."""
+    X = blobs(n, d, k, dtype, seed=n + d + 1, spread=6.0)
+    with hip.Handle(n, d, k, dtype) as h:
+        h.set_data(X)
+        h.init_parallel(seed)
+        info = h.parallel_seed_info()
+    cand = np.ascontiguousarray(X[info["cand_rows"]])
+    M = cand.shape[0]
+    assert M > k and info["weights"] is not None
+    assert info["weights"].sum() == n
+    one_pass = oracle.assign(X, cand, threads=8)
+    want = np.bincount(one_pass, minlength=M).astype(np.float64)
+    moved = np.abs(info["weights"] - want).sum()
+    best, d1, d2 = oracle.top2_exact(X, cand, threads=8)
+    xx = (X.astype(np.float64) ** 2).sum(1)
+    floor = 8 * float(np.finfo(dtype).eps) * 2 * xx            # (candidates are rows: |c|^2 ~ |x|^2)
+    near_tie = ((d2 - d1) <= 1e-5 * d2) | ((d2 - d1) <= floor)
+    assert moved <= 2 * int(near_tie.sum()), (moved, int(near_tie.sum()))
+
+
 def test_fit_entry_point_seeds_with_kmeans_parallel(hip, oracle):
     """init_from_data == 1 through make_ptr_float_kmeans; zero iterations return the seeds."""
     from h2o4gpu_amd.libs import ch2o4gpu_gpu

@@ -130,3 +130,57 @@ def test_estimator_restarts_keep_the_best(hip):
     assert abs(best.inertia_ - min(inertias)) <= 1e-6 * min(inertias)
     assert best.cluster_centers_.shape == (k, d) and best.labels_.shape == (n,)
     assert best.n_iter_ == 15
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n,d,k,sets", [(60000, 16, 8, 4), (30000, 40, 12, 3), (20000, 5, 16, 5)])
+def test_small_shapes_stacked_restarts_against_the_default_single_fit(hip, oracle, n, d, k, sets, dtype):
+    """For k <= 16 and d <= 64 a single fit runs the scalar-order kernels (bit-identical to the
+    oracle) while stacked restarts always run the matrix-core kernel with its own summation order
+    (and 16-ulp keys in float32): restart r of an n_init fit is then the single fit from the same
+    start only up to near-tie rows. Checked here by the usual bars, per iteration in lock-step
+    (same centroids in: labels equal except near-ties, the update of the set's own labels equal
+    to the oracle's) and end to end on the objective."""
+    from parity import label_report
+    X = blobs(n, d, k, dtype, seed=n + d + k)
+    assert hip.stack_width(n, d, k, dtype, sets) >= sets
+    rng = np.random.default_rng(17)
+    starts = [np.ascontiguousarray(X[rng.choice(n, size=k, replace=False)]) for _ in range(sets)]
+    tol = 1e-5 if dtype == np.float32 else 1e-12
+    with hip.Handle(n, d, k, dtype, sets=sets) as h:
+        h.set_data(X)
+        for s in range(sets):
+            h.select_set(s)
+            h.set_centroids(starts[s])
+        h.iterate(1)
+        flips = 0
+        for s in range(sets):
+            h.select_set(s)
+            L, C1 = h.labels(), h.centroids()
+            wL = oracle.assign(X, starts[s], threads=4)
+            flips += label_report(oracle, X, starts[s], L, wL)["mismatch"]
+            wC, _ = oracle.update(X, L, starts[s], threads=4)
+            assert np.allclose(C1, wC, rtol=tol, atol=tol * np.abs(wC).max())
+        for s in range(sets):
+            h.select_set(s)
+            h.set_centroids(starts[s])
+        assert h.fit(25, 0.0) == 25
+        stacked = []
+        for s in range(sets):
+            h.select_set(s)
+            stacked.append((h.centroids(), h.labels(), h.inertia()))
+    for s in range(sets):
+        with hip.Handle(n, d, k, dtype) as h1:
+            h1.set_data(X)
+            assert h1.assign_variant() == "valu"
+            h1.set_centroids(starts[s])
+            assert h1.fit(25, 0.0) == 25
+            C, L, inertia = h1.centroids(), h1.labels(), h1.inertia()
+        sC, sL, sinertia = stacked[s]
+        # labels_ of a stacked set come from an ordinary relabel (the default family) against
+        # the set's own centroids
+        assert np.array_equal(sL, oracle.assign(X, sC, threads=4))
+        assert abs(sinertia - inertia) <= 1e-5 * inertia
+        if flips == 0 and np.array_equal(sL, L):
+            assert np.allclose(sC, C, rtol=1e-4 if dtype == np.float32 else 1e-9,
+                               atol=(1e-4 if dtype == np.float32 else 1e-9) * np.abs(C).max())

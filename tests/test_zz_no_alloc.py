@@ -27,8 +27,15 @@ def hiprt():
         rt.hipStreamCreateWithFlags.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_uint]
         rt.hipStreamSynchronize.argtypes = [ctypes.c_void_p]
         rt.hipStreamDestroy.argtypes = [ctypes.c_void_p]
+        rt.hipMemGetInfo.argtypes = [ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]
         _hip = rt
     return _hip
+
+
+def free_device_bytes():
+    fr, tot = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    assert hiprt().hipMemGetInfo(ctypes.byref(fr), ctypes.byref(tot)) == 0
+    return fr.value
 
 
 class DeviceBuffer:
@@ -89,6 +96,15 @@ def test_noalloc_predict_equals_predict_host(hip, oracle, first, second, dtype):
                                            stream.value)
                 assert hiprt().hipStreamSynchronize(stream) == 0
                 got = dL.download(n, np.int32)
+                # the same call again (the shape's one-time set-up is behind it): the device's
+                # free memory is the same before, while the work is queued, and after
+                before = free_device_bytes()
+                hip.predict_device_noalloc(dtype, n, d, k, dX.ptr.value, dC.ptr.value, dL.ptr.value,
+                                           stream.value)
+                queued = free_device_bytes()
+                assert hiprt().hipStreamSynchronize(stream) == 0
+                assert before == queued == free_device_bytes(), "the call changed the device's free memory"
+                assert np.array_equal(dL.download(n, np.int32), got)
             finally:
                 dX.free(); dC.free(); dL.free()
             where = "call %d: n=%d d=%d k=%d %s" % (call, n, d, k, np.dtype(dtype).name)
