@@ -1675,6 +1675,35 @@ __global__ void copy_probe_kernel(const float4 *__restrict__ src, float4 *__rest
     dst[i] = src[i];
 }
 
+// Read-only stream: every thread keeps four 16-byte loads in flight and adds what arrives;
+// one value per thread leaves at the end (so the loads cannot be dropped).
+__global__ __launch_bounds__(256) void read_probe_kernel(const float4 *__restrict__ src,
+                                                         float *__restrict__ out, size_t nvec) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  float4 a0 = {0, 0, 0, 0}, a1 = a0, a2 = a0, a3 = a0;
+  for (; i + 3 * stride < nvec; i += 4 * stride) {
+    const float4 v0 = src[i], v1 = src[i + stride], v2 = src[i + 2 * stride], v3 = src[i + 3 * stride];
+    a0.x += v0.x; a0.y += v0.y; a0.z += v0.z; a0.w += v0.w;
+    a1.x += v1.x; a1.y += v1.y; a1.z += v1.z; a1.w += v1.w;
+    a2.x += v2.x; a2.y += v2.y; a2.z += v2.z; a2.w += v2.w;
+    a3.x += v3.x; a3.y += v3.y; a3.z += v3.z; a3.w += v3.w;
+  }
+  for (; i < nvec; i += stride) {
+    const float4 v0 = src[i];
+    a0.x += v0.x; a0.y += v0.y; a0.z += v0.z; a0.w += v0.w;
+  }
+  out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] =
+      (a0.x + a0.y + a0.z + a0.w) + (a1.x + a1.y + a1.z + a1.w) + (a2.x + a2.y + a2.z + a2.w) +
+      (a3.x + a3.y + a3.z + a3.w);
+}
+// Write-only stream.
+__global__ __launch_bounds__(256) void fill_probe_kernel(float4 *__restrict__ dst, size_t nvec, float v) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  const float4 val = {v, v, v, v};
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += stride) dst[i] = val;
+}
+
 // ---------------------------------------------------------------------------
 // C ABI, part 1: the reference's entry points
 // ---------------------------------------------------------------------------
@@ -2239,15 +2268,19 @@ KM_API const char *h2o4gpu_kmeans_assign_variant(h2o4gpu_kmeans_handle *h) {
   return assign_variant_name(v);
 }
 
-KM_API int h2o4gpu_kmeans_copy_probe(int gpu_id, size_t bytes, int reps, float *ms) {
-  if (!ms || reps < 1 || bytes < 16) return H2O4GPU_KMEANS_EARG;
+KM_API int h2o4gpu_kmeans_bandwidth_probe(int gpu_id, int kind, size_t bytes, int reps, float *ms) {
+  if (!ms || reps < 1 || bytes < 16 || kind < 0 || kind > 3) return H2O4GPU_KMEANS_EARG;
   const int nvis = visible_devices();
   if (nvis < 1) return H2O4GPU_KMEANS_EDEVICE;
   KM_HIP_TRY(hipSetDevice((gpu_id < 0 ? 0 : gpu_id) % nvis));
+  const unsigned grid = 256 * 8, block = 256;
   void *a = nullptr, *b = nullptr;
-  if (hipMalloc(&a, bytes) != hipSuccess || hipMalloc(&b, bytes) != hipSuccess) {
+  float *sink = nullptr;
+  if (hipMalloc(&a, bytes) != hipSuccess || hipMalloc(&b, bytes) != hipSuccess ||
+      hipMalloc(reinterpret_cast<void **>(&sink), (size_t)grid * block * sizeof(float)) != hipSuccess) {
     (void)hipGetLastError();
     if (a) (void)hipFree(a);
+    if (b) (void)hipFree(b);
     return H2O4GPU_KMEANS_EALLOC;
   }
   hipEvent_t e0, e1;
@@ -2257,13 +2290,23 @@ KM_API int h2o4gpu_kmeans_copy_probe(int gpu_id, size_t bytes, int reps, float *
     (void)hipMemset(a, 1, bytes);
     (void)hipMemset(b, 0, bytes);
     const size_t nvec = bytes / 16;
-    hipLaunchKernelGGL(copy_probe_kernel, dim3(256 * 8), dim3(256), 0, 0, (const float4 *)a, (float4 *)b, nvec);
+    auto once = [&]() {
+      if (kind == H2O4GPU_KMEANS_PROBE_COPY)
+        hipLaunchKernelGGL(copy_probe_kernel, dim3(grid), dim3(block), 0, 0, (const float4 *)a, (float4 *)b, nvec);
+      else if (kind == H2O4GPU_KMEANS_PROBE_READ)
+        hipLaunchKernelGGL(read_probe_kernel, dim3(grid), dim3(block), 0, 0, (const float4 *)a, sink, nvec);
+      else if (kind == H2O4GPU_KMEANS_PROBE_WRITE)
+        hipLaunchKernelGGL(fill_probe_kernel, dim3(grid), dim3(block), 0, 0, (float4 *)b, nvec, 1.0f);
+      else
+        (void)hipMemcpyAsync(b, a, bytes, hipMemcpyDeviceToDevice, 0);
+    };
+    once();
     (void)hipDeviceSynchronize();
     (void)hipEventRecord(e0, 0);
-    for (int r = 0; r < reps; r++)
-      hipLaunchKernelGGL(copy_probe_kernel, dim3(256 * 8), dim3(256), 0, 0, (const float4 *)a, (float4 *)b, nvec);
+    for (int r = 0; r < reps; r++) once();
     (void)hipEventRecord(e1, 0);
     if (hipEventSynchronize(e1) != hipSuccess) rc = H2O4GPU_KMEANS_EDEVICE;
+    if (rc == 0 && hipGetLastError() != hipSuccess) rc = H2O4GPU_KMEANS_EDEVICE;
     float t = 0;
     if (rc == 0 && hipEventElapsedTime(&t, e0, e1) == hipSuccess) *ms = t / reps;
     (void)hipEventDestroy(e0);
@@ -2271,7 +2314,11 @@ KM_API int h2o4gpu_kmeans_copy_probe(int gpu_id, size_t bytes, int reps, float *
   }
   (void)hipFree(a);
   (void)hipFree(b);
+  (void)hipFree(sink);
   return rc;
+}
+KM_API int h2o4gpu_kmeans_copy_probe(int gpu_id, size_t bytes, int reps, float *ms) {
+  return h2o4gpu_kmeans_bandwidth_probe(gpu_id, H2O4GPU_KMEANS_PROBE_COPY, bytes, reps, ms);
 }
 
 KM_API int h2o4gpu_kmeans_predict_device_noalloc(int elem_size, size_t rows, size_t cols, int k,

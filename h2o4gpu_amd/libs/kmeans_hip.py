@@ -78,6 +78,7 @@ PROTOTYPES = {
     "h2o4gpu_kmeans_kernel_time": (c_int, [c_void_p, c_char_p, P(c_int), P(c_double)]),
     "h2o4gpu_kmeans_assign_variant": (c_char_p, [c_void_p]),
     "h2o4gpu_kmeans_copy_probe": (c_int, [c_int, c_size_t, c_int, P(c_float)]),
+    "h2o4gpu_kmeans_bandwidth_probe": (c_int, [c_int, c_int, c_size_t, c_int, P(c_float)]),
     "h2o4gpu_kmeans_predict_device_noalloc": (c_int, [c_int, c_size_t, c_size_t, c_int, c_void_p,
                                                       c_void_p, c_void_p, c_void_p]),
 }
@@ -332,6 +333,19 @@ def copy_probe(nbytes, reps=10, gpu_id=0):
     """Average milliseconds of one device-to-device copy of nbytes."""
     ms = c_float(0.0)
     _check("copy_probe", lib().h2o4gpu_kmeans_copy_probe(gpu_id, nbytes, reps, ctypes.byref(ms)))
+    return ms.value
+
+
+PROBE_KINDS = {"copy": 0, "read": 1, "write": 2, "memcpy": 3}
+
+
+def bandwidth_probe(kind, nbytes, reps=10, gpu_id=0):
+    """Average milliseconds of one streaming pass over nbytes: kind "read" (read only), "write"
+    (write only), "copy" (a kernel that reads and writes nbytes) or "memcpy" (hipMemcpy device
+    to device)."""
+    ms = c_float(0.0)
+    _check("bandwidth_probe", lib().h2o4gpu_kmeans_bandwidth_probe(gpu_id, PROBE_KINDS[kind], nbytes, reps,
+                                                                    ctypes.byref(ms)))
     return ms.value
 
 

@@ -275,6 +275,21 @@ const char *h2o4gpu_kmeans_assign_variant(h2o4gpu_kmeans_handle *h);
 int h2o4gpu_kmeans_copy_probe(int gpu_id, size_t bytes, int reps,
                               float *milliseconds);
 
+/* The same measurement for the other streaming patterns a Lloyd step is made of,
+ * so that a kernel's bytes per second can be put beside what this device
+ * delivers for its own mix of reads and writes and not only beside the
+ * datasheet figure. kind: COPY = the kernel above (reads `bytes`, writes
+ * `bytes`); READ = a kernel that only reads `bytes` (four 16-byte loads in
+ * flight per thread, one float per thread written at the end); WRITE = a
+ * kernel that only writes `bytes`; MEMCPY = hipMemcpyAsync device to device
+ * (reads and writes `bytes`). Returns the average milliseconds of one pass. */
+#define H2O4GPU_KMEANS_PROBE_COPY 0
+#define H2O4GPU_KMEANS_PROBE_READ 1
+#define H2O4GPU_KMEANS_PROBE_WRITE 2
+#define H2O4GPU_KMEANS_PROBE_MEMCPY 3
+int h2o4gpu_kmeans_bandwidth_probe(int gpu_id, int kind, size_t bytes, int reps,
+                                   float *milliseconds);
+
 /* ---------------------------------------------------------------------------
  * Part 4 - assignment without any allocation.
  * No counterpart in the reference. For callers that cannot allocate device
