@@ -209,6 +209,62 @@ def seeding_seconds(X, k, seed=7):
             "note": "init_from_data=1 on resident rows: rounds of k-means||, weights, k picks"}
 
 
+def hbm_probes(nbytes=1 << 30, reps=10):
+    """What this device's memory system delivers for plain streaming kernels over 1 GiB: the
+    measured roof beside the 8 TB/s datasheet figure."""
+    out = {"bytes": nbytes}
+    for kind, moved in (("read", 1.0), ("write", 1.0), ("copy", 2.0), ("memcpy", 2.0)):
+        ms = kmeans_hip.bandwidth_probe(kind, nbytes, reps)
+        out[kind + "_gbps"] = moved * nbytes / (ms * 1e-3) / 1e9
+    return out
+
+
+def extra_step(workload, scale, steps, warmup=2):
+    """One more shape timed in this process after the headline one, the same way: `steps`
+    Lloyd steps (assign + update) on resident rows between stream events, then again with an
+    event pair round every launch for the dominant kernel's average. float32."""
+    t0 = time.perf_counter()
+    X, k, _ = datasets.make(workload, scale, np.float32)
+    n, d = X.shape
+    gen_s = time.perf_counter() - t0
+    seed = datasets.SHAPES[workload][3]
+    with kmeans_hip.Handle(n, d, k, np.float32) as h:
+        h.set_data(X)
+        if workload == "C4":
+            h.init_plusplus(seed)   # the benchmark's start for this shape: k-means++, fixed seed
+        else:
+            h.set_centroids(datasets.seeded_row_init(X, k, seed))
+        variant = h.assign_variant()
+        h.iterate(warmup)
+        h.timer_start()
+        h.iterate(steps)
+        ms_step = h.timer_stop() / steps
+        h.profile(True)
+        h.iterate(steps)
+        kern = {}
+        for name in ("assign", "accumulate", "assign_accumulate", "finalize"):
+            cnt, ms = h.kernel_time(name)
+            if cnt:
+                kern[name] = ms / cnt
+        h.profile(False)
+    dom = "assign_accumulate" if "assign_accumulate" in kern else "assign"
+    out = {"workload": "%s generator: %d x %d f32, k=%d" % (workload, n, d, k), "assign_variant": variant,
+           "steps": steps, "ms_per_step": ms_step, "kernel": "%s (%s)" % (dom, variant),
+           "kernel_avg_ms": kern[dom], "kernels_avg_ms": {a: round(b, 5) for a, b in kern.items()},
+           "generation_seconds": gen_s}
+    if variant == "valu":
+        # the iteration's algorithmic bytes: rows read once, labels written once, centroids in and out
+        nbytes = float(n) * d * 4 + 4.0 * n + 2.0 * k * d * 4
+        gbps = nbytes / (kern[dom] * 1e-3) / 1e9
+        out.update({"bound": "hbm", "algorithmic_bytes": nbytes, "achieved": gbps, "peak": PEAK_HBM_GBPS,
+                    "unit": "GB/s", "frac": gbps / PEAK_HBM_GBPS})
+    else:
+        tf = 2.0 * n * k * d / (kern[dom] * 1e-3) / 1e12
+        out.update({"bound": "mfma", "algorithmic_flops": 2.0 * n * k * d, "achieved": tf,
+                    "peak": PEAK_MFMA_TFLOPS["f32"], "unit": "TFLOP/s", "frac": tf / PEAK_MFMA_TFLOPS["f32"]})
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -238,6 +294,10 @@ def main():
                     help="skip the whole fit through make_ptr_*_kmeans (upload included, field c_abi_fit)")
     ap.add_argument("--end-to-end", dest="end_to_end", action="store_true", help=argparse.SUPPRESS)
     ap.set_defaults(end_to_end=True)
+    ap.add_argument("--no-extras", dest="extras", action="store_false",
+                    help="skip the two extra shapes timed after the headline one (the compute-bound "
+                         "distance step at 2M x 256, k = 1024 and the bandwidth-bound step at 10M x 16, k = 8)")
+    ap.set_defaults(extras=True)
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -332,14 +392,19 @@ def main():
         roofline = {"bound": "mfma", "kernel": "%s (%s)" % (dom, variant), "achieved": tflops,
                     "peak": peak, "unit": "TFLOP/s", "frac": tflops / peak, "traffic": traffic}
     else:
-        # per row: the row and its squared norm read, label and minimum distance written
-        gbps = float(n) * (d * s + s + 4 + s) / (assign_ms * 1e-3) / 1e9
+        # per row: the row read, the label written (inside a fit loop the fused step neither reads
+        # the stored row norms nor writes the minimum distances)
+        gbps = float(n) * (d * s + 4) / (assign_ms * 1e-3) / 1e9
         roofline = {"bound": "hbm", "kernel": "%s (valu)" % dom, "achieved": gbps,
                     "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": gbps / PEAK_HBM_GBPS,
                     "traffic": traffic}
     iter_gbps = bytes_per_iter / (ms_step * 1e-3) / 1e9
     copy_bytes = 1 << 30
     copy_ms = kmeans_hip.copy_probe(copy_bytes, 10)
+    try:
+        probes = hbm_probes()
+    except Exception as e:  # an extra: never the reason a bench line is missing
+        probes = {"error": repr(e)}
 
     inertia = None
     h.assign()
@@ -397,6 +462,7 @@ def main():
                       "mfma_frac": flops_per_iter / (ms_step * 1e-3) / 1e12 / peak},
         "kernels_avg_ms": {kname: round(v["avg_ms"], 5) for kname, v in kern.items()},
         "copy_probe_gbps": 2.0 * copy_bytes / (copy_ms * 1e-3) / 1e9,
+        "hbm_probes": probes,
         "h2d_seconds": h2d_s,
         "h2d_seconds_first_call": h2d_first_s,
         "inertia": inertia,
@@ -405,6 +471,20 @@ def main():
         out["transform"] = transform
     if split_leg:
         out["fp32_split"] = split_leg
+    if args.extras and args.workload == "C3" and args.scale == 1.0 and args.dtype == "f32":
+        # the north star's two regimes under the same clock as the headline shape; extras, never
+        # the reason a bench line is missing
+        for key, wl, scale in (("c4_distance_step", "C4", 1.0), ("hbm_bound_step", "C1", 100.0)):
+            try:
+                t0 = time.perf_counter()
+                out[key] = extra_step(wl, scale, 5 if wl == "C4" else 20)
+                if key == "hbm_bound_step" and "read_gbps" in probes:
+                    out[key]["frac_of_read_probe"] = out[key]["achieved"] / probes["read_gbps"]
+                    out[key]["frac_of_copy_probe"] = out[key]["achieved"] / probes["copy_gbps"]
+                log("%s: %.4f ms per launch, %.3f of peak (%.1f s)" % (key, out[key]["kernel_avg_ms"],
+                                                                         out[key]["frac"], time.perf_counter() - t0))
+            except Exception as e:
+                out[key] = {"error": repr(e)}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(X, C0, args.cpu_iters)
         out["cpu_reference_path"] = sklearn_baseline(X, C0, args.sklearn_rows)

@@ -154,41 +154,50 @@ template <typename T>
 struct BlockLoad<T, 1> {
   typedef T type;
 };
+// Layout of the per-centroid sums of the two fused kernels in LDS: `ncopy` copies (1, 2 or 4),
+// copy (lane / 16) % ncopy for the lanes of a wavefront, [copy][centroid][sxs] doubles, sxs =
+// d rounded up to 16 (d itself below 16). A lane adds its row starting at feature lane % 16,
+// so at any moment the 16 lanes of a group add 16 consecutive features, and with a centroid
+// stride of 0 or 16 (mod 32) doubles those are 16 different bank pairs whatever the labels
+// are; the groups of a wavefront add into copies of their own. Measured on the LDS pipe
+// alone (8 labels, 16 features): 6.7 lane additions per clock and CU against 2.6 for one
+// copy with an odd centroid stride (7.6 with no conflict at all).
+__host__ __device__ static inline int sums_stride(int d) { return d < 16 ? d : (d + 15) / 16 * 16; }
+
 template <typename T, int DREG, bool SUMS>
 __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
     const T *__restrict__ X, const T *__restrict__ xnorm, const T *__restrict__ C,
     const T *__restrict__ cnorm, int *__restrict__ labels, T *__restrict__ mindist,
     double *__restrict__ psums, int *__restrict__ pcounts, int64_t n, int k,
-    T *__restrict__ D, int64_t ldn) {
+    T *__restrict__ D, int64_t ldn, int ncopy) {
 #pragma clang fp contract(off)
   extern __shared__ __align__(16) unsigned char smem_raw[];
   constexpr int d = DREG;
   // D (assignment-only form): write every distance to D[c * ldn + row] instead of labels
   const bool full = !SUMS && D != nullptr;
   constexpr int VEC = Mfma<T>::VW;
-  const int sx = staged_row_stride(d);                           // row stride of the staged block
+  // Rows are staged with a stride of d + one 16-byte vector: every staged vector and every
+  // row start stays 16-byte aligned (one ds_write_b128 per fetched vector, d / VEC
+  // ds_read_b128 per row), and the 8 lanes such an access serves per clock fall on
+  // different banks for every d here (d = VEC needs no padding: the rows are lane-linear).
+  constexpr int SXT = DREG == VEC ? DREG : DREG + VEC;
+  constexpr int sxs = DREG;  // = sums_stride(DREG): DREG is a power of two
   // SUMS false: assignment only (predict, final relabel, inertia): no sums, no counts
-  double *sums = reinterpret_cast<double *>(smem_raw);           // [k][sx]
-  int *cnt = reinterpret_cast<int *>(sums + (SUMS ? (size_t)k * sx : 0));  // [k]
-  T *ccs = reinterpret_cast<T *>(cnt + (SUMS ? k + (k & 1) : 0));          // [k] centroid norms
-  T *Xs = ccs + k + (k & 1);                                     // [WG][sx]
+  const int kq = (k + 3) & ~3;
+  double *sums = reinterpret_cast<double *>(smem_raw);                      // [ncopy][k][sxs]
+  int *cnt = reinterpret_cast<int *>(sums + (SUMS ? (size_t)ncopy * k * sxs : 0));  // [kq]
+  T *ccs = reinterpret_cast<T *>(cnt + (SUMS ? kq : 0));                    // [kq] centroid norms
+  T *Xs = ccs + kq;                                                         // [WG][SXT], 16-byte aligned
   typedef typename BlockLoad<T, VEC>::type ld_t;
-  constexpr int NLD = DREG / VEC;  // loads per thread and block
+  constexpr int NLD = DREG / VEC;  // 16-byte vectors per row = loads per thread and block
   const int tid = threadIdx.x;
   if (SUMS) {
-    for (int e = tid; e < k * sx; e += WG) sums[e] = 0.0;
+    for (int e = tid; e < ncopy * k * sxs; e += WG) sums[e] = 0.0;
     for (int c = tid; c < k; c += WG) cnt[c] = 0;
   }
-  // LDS offset of the i-th load of this thread: element (tid + i*WG)*VEC of the block
-  int off[NLD];
-#pragma unroll
-  for (int i = 0; i < NLD; i++) {
-    const int el = (tid + i * WG) * VEC;
-    const int r = el / d;
-    off[i] = r * sx + (el - r * d);
-  }
+  // vector tid + i*WG of the block is vector tid % NLD of row tid / NLD + i * (WG / NLD)
+  const int st_off = (tid / NLD) * SXT + (tid % NLD) * VEC;
   ld_t pre[NLD];
-  T pre_xx = 0;  // squared norm of this thread's row in the fetched block
   // Loads are never predicated: indices past the end of the data set are
   // clamped instead, which keeps the loop free of divergent branches and lets
   // the fetched block stay in flight across the processing of the current one.
@@ -200,8 +209,6 @@ __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
       const int64_t e = tid + i * WG;
       pre[i] = src[e < last ? e : last];
     }
-    const int64_t r = base + tid;
-    pre_xx = xnorm[r < n ? r : n - 1];
   };
   const int64_t stride = (int64_t)gridDim.x * WG;
   int64_t base = (int64_t)blockIdx.x * WG;
@@ -209,26 +216,33 @@ __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
   fetch(base);
   // centroid norms while the first block travels (visible after the barrier below)
   for (int c = tid; c < k; c += WG) ccs[c] = cnorm ? cnorm[c] : row_sqnorm<T>(C + (size_t)c * d, d);
-  const int jrot = (tid & 63) % d;
+  const int l16 = tid & 15;
+  double *const my_sums = sums + (size_t)((tid >> 4) & (ncopy - 1)) * k * sxs;
   for (; base < n; base += stride) {
     const int rows = (int)min<int64_t>(WG, n - base);
     __syncthreads();  // the previous block has been consumed
 #pragma unroll
-    for (int i = 0; i < NLD; i++) {  // rows past the end of a last, partial block hold clamped copies
-#pragma unroll
-      for (int q = 0; q < VEC; q++) Xs[off[i] + q] = pre[i][q];
-    }
-    const T xx = pre_xx;
+    for (int i = 0; i < NLD; i++)  // rows past the end of a last, partial block hold clamped copies
+      *reinterpret_cast<ld_t *>(Xs + st_off + i * (WG / NLD) * SXT) = pre[i];
     __syncthreads();
     // the next block travels while this one is processed: no other vector
     // load is issued below, so nothing waits for these until the next round
     fetch(base + stride < n ? base + stride : base);
     const int64_t row = base + tid;
     if (tid < rows) {
-      const T *xrow = Xs + tid * sx;
+      const T *xrow = Xs + tid * SXT;
       T xr[DREG];
 #pragma unroll
-      for (int j = 0; j < DREG; j++) xr[j] = xrow[j];
+      for (int q = 0; q < NLD; q++) {
+        const ld_t v = *reinterpret_cast<const ld_t *>(xrow + q * VEC);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) xr[q * VEC + e] = v[e];
+      }
+      // the row's squared norm, j ascending, multiply and add rounded separately: the value
+      // row_norms stores (kmeans_labels.h:187-199), without reading it back from memory
+      T xx = 0;
+#pragma unroll
+      for (int j = 0; j < DREG; j++) xx = xx + xr[j] * xr[j];
       T best = argmin_start<T>();
       int bidx = -1;
 #pragma unroll 2
@@ -250,14 +264,11 @@ __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
         if (mindist) mindist[row] = best;
       }
       if (SUMS && bidx >= 0) {
-        // Lane l starts at feature l mod d: with only a handful of centroids the
-        // lanes of a wavefront would otherwise all add to the same few addresses
-        // at once, and same-address LDS atomics are served one lane at a time.
-        double *srow = sums + (size_t)bidx * sx;
-        int j = jrot;
+        double *srow = my_sums + (size_t)bidx * sxs;
+#pragma unroll 4
         for (int q = 0; q < d; q++) {
+          const int j = (l16 + q) & (d - 1);
           unsafeAtomicAdd(srow + j, (double)xrow[j]);
-          j = (j + 1 == d) ? 0 : j + 1;
         }
         atomicAdd(&cnt[bidx], 1);
       }
@@ -268,7 +279,9 @@ __global__ __launch_bounds__(WG) void lloyd_valu_fused_kernel(
   double *dst = psums + (size_t)blockIdx.x * k * d;
   for (int e = tid; e < k * d; e += WG) {
     const int c = e / d, j = e - c * d;
-    dst[e] = sums[(size_t)c * sx + j];
+    double v = sums[(size_t)c * sxs + j];
+    for (int cp = 1; cp < ncopy; cp++) v += sums[((size_t)cp * k + c) * sxs + j];  // copy order
+    dst[e] = v;
   }
   int *cdst = pcounts + (size_t)blockIdx.x * k;
   for (int c = tid; c < k; c += WG) cdst[c] = cnt[c];
@@ -295,21 +308,22 @@ __global__ __launch_bounds__(WG) void lloyd_valu_anyd_kernel(
     const T *__restrict__ X, const T *__restrict__ xnorm, const T *__restrict__ C,
     const T *__restrict__ cnorm, int *__restrict__ labels, T *__restrict__ mindist,
     double *__restrict__ psums, int *__restrict__ pcounts, int64_t n, int d, int k,
-    T *__restrict__ D, int64_t ldn) {
+    T *__restrict__ D, int64_t ldn, int ncopy) {
 #pragma clang fp contract(off)
   extern __shared__ __align__(16) unsigned char smem_raw[];
   const bool full = !SUMS && D != nullptr;  // as in lloyd_valu_fused_kernel
   const int sx = staged_row_stride(d);
   const int pad = sx - d;                                        // 0 or 1
-  double *sums = reinterpret_cast<double *>(smem_raw);           // [k][sx]; SUMS false: none
-  int *cnt = reinterpret_cast<int *>(sums + (SUMS ? (size_t)k * sx : 0));  // [k]
+  const int sxs = sums_stride(d);
+  double *sums = reinterpret_cast<double *>(smem_raw);           // [ncopy][k][sxs]; SUMS false: none
+  int *cnt = reinterpret_cast<int *>(sums + (SUMS ? (size_t)ncopy * k * sxs : 0));  // [k]
   T *ccs = reinterpret_cast<T *>(cnt + (SUMS ? k + (k & 1) : 0));          // [k]
   T *Xs = ccs + k + (k & 1);                                     // [WG][sx]
   typedef typename BlockLoad<T, VEC>::type ld_t;
   constexpr int NLD = (DMAX + VEC - 1) / VEC;
   const int tid = threadIdx.x;
   if (SUMS) {
-    for (int e = tid; e < k * sx; e += WG) sums[e] = 0.0;
+    for (int e = tid; e < ncopy * k * sxs; e += WG) sums[e] = 0.0;
     for (int c = tid; c < k; c += WG) cnt[c] = 0;
   }
   const int nld = (d + VEC - 1) / VEC;  // loads per thread and block
@@ -354,7 +368,8 @@ __global__ __launch_bounds__(WG) void lloyd_valu_anyd_kernel(
   int coff[KREG];
 #pragma unroll
   for (int c = 0; c < KREG; c++) coff[c] = (c < k ? c : k - 1) * d;
-  const int jrot = (tid & 63) % d;
+  const int jrot = (tid & 15) % d;  // sums_stride: the 16 lanes of a group add 16 consecutive features
+  double *const my_sums = sums + (size_t)((tid >> 4) & (ncopy - 1)) * k * sxs;
   for (; base < n; base += stride) {
     const int rows = (int)min<int64_t>(WG, n - base);
     __syncthreads();  // the previous block has been consumed
@@ -444,7 +459,7 @@ __global__ __launch_bounds__(WG) void lloyd_valu_anyd_kernel(
         if (mindist) mindist[row] = best;
       }
       if (SUMS && bidx >= 0) {
-        double *srow = sums + (size_t)bidx * sx;
+        double *srow = my_sums + (size_t)bidx * sxs;
         int jj = jrot;  // rotated start, as in lloyd_valu_fused_kernel
         for (int q = 0; q < d; q++) {
           unsafeAtomicAdd(srow + jj, (double)xrow[jj]);
@@ -459,7 +474,9 @@ __global__ __launch_bounds__(WG) void lloyd_valu_anyd_kernel(
   double *dst = psums + (size_t)blockIdx.x * k * d;
   for (int e = tid; e < k * d; e += WG) {
     const int c = e / d, jx = e - c * d;
-    dst[e] = sums[(size_t)c * sx + jx];
+    double v = sums[(size_t)c * sxs + jx];
+    for (int cp = 1; cp < ncopy; cp++) v += sums[((size_t)cp * k + c) * sxs + jx];  // copy order
+    dst[e] = v;
   }
   int *cdst = pcounts + (size_t)blockIdx.x * k;
   for (int c = tid; c < k; c += WG) cdst[c] = cnt[c];
@@ -1763,14 +1780,36 @@ struct RowstatDispatch<double, FUSE> {
 #undef KM_ROWSTAT_CASE
 
 static bool valu_fused_applies(int d, int k) { return k <= 16 && d <= 64; }
+// LDS of the two fused kernels for a shape: `reg` = the register variant (d one of 4, 8, 16,
+// 32, 64 and 16-byte aligned rows), otherwise the any-d variant.
 template <typename T>
-static size_t valu_fused_lds(int d, int k, bool sums = true) {
+static size_t valu_fused_lds(int d, int k, bool sums, bool reg, int ncopy) {
+  const int vw = Mfma<T>::VW;
+  const size_t sum_bytes = sums ? (size_t)ncopy * k * sums_stride(d) * sizeof(double) : 0;
+  if (reg) {
+    const int kq = (k + 3) & ~3;
+    const int sxt = d == vw ? d : d + vw;
+    return sum_bytes + (sums ? (size_t)kq * sizeof(int) : 0) + (size_t)kq * sizeof(T) +
+           (size_t)WG * sxt * sizeof(T);
+  }
   const int sx = staged_row_stride(d);
-  return (sums ? (size_t)k * sx * sizeof(double) + ((size_t)k + 1) * sizeof(int) : 0) +
-         ((size_t)k + 1) * sizeof(T) + (size_t)WG * sx * sizeof(T) + 16;
+  return sum_bytes + (sums ? ((size_t)k + 1) * sizeof(int) : 0) + ((size_t)k + 1) * sizeof(T) +
+         (size_t)WG * sx * sizeof(T) + 16;
 }
-static int valu_fused_grid(int64_t n, size_t lds, int num_cu) {
-  int per_cu = (int)((160 * 1024) / lds);  // a CU has 160 KB of LDS
+// Copies of the sums (see sums_stride): as many of 4, 2, 1 as leave the workgroups per CU that
+// one copy allows (by LDS; at most 8 are used).
+template <typename T>
+static int valu_fused_copies(int d, int k, bool reg) {
+  auto per_cu = [&](int nc) {
+    const int v = (int)((160 * 1024) / valu_fused_lds<T>(d, k, true, reg, nc));
+    return v > 8 ? 8 : v;
+  };
+  for (int nc = 4; nc > 1; nc >>= 1)
+    if (per_cu(nc) >= per_cu(1) && per_cu(nc) >= 1) return nc;
+  return 1;
+}
+static int valu_fused_grid(int64_t n, int resident, int num_cu) {
+  int per_cu = resident;  // what a CU holds at once of this kernel instance
   if (per_cu > 8) per_cu = 8;
   if (per_cu < 1) per_cu = 1;
   int64_t grid = (int64_t)num_cu * per_cu;
@@ -1798,19 +1837,24 @@ static int launch_valu_fused(hipStream_t s, const T *X, const T *xnorm, const T 
                              const T *cnorm, int *labels, T *mindist, int64_t n, int d, int k,
                              int num_cu, double *psums, int *pcounts, int *slots, T *D = nullptr,
                              int64_t ldn = 0) {
-  const size_t lds = valu_fused_lds<T>(d, k, SUMS);
-  const int grid = valu_fused_grid(n, lds, num_cu);
-  if (slots) *slots = grid;
+  int grid = 1;
   const int vw = Mfma<T>::VW;
   const bool aligned = (reinterpret_cast<uintptr_t>(X) & 15) == 0;
-#define KM_VF_SETUP(kern) KM_TRY(ensure_dynamic_lds(reinterpret_cast<const void *>(kern), lds))
+  const bool reg = aligned && (d == 4 || d == 8 || d == 16 || d == 32 || d == 64) && d >= vw;
+  const int ncopy = SUMS ? valu_fused_copies<T>(d, k, reg) : 1;
+  const size_t lds = valu_fused_lds<T>(d, k, SUMS, reg, ncopy);
+  // the grid is what the device holds at once of the chosen instance (its registers count too)
+#define KM_VF_SETUP(kern)                                                                      \
+  KM_TRY(ensure_dynamic_lds(reinterpret_cast<const void *>(kern), lds));                       \
+  grid = valu_fused_grid(n, resident_blocks_per_cu(reinterpret_cast<const void *>(kern), WG, lds), num_cu); \
+  if (slots) *slots = grid
   // d is one of the register sizes: the row lives in registers
 #define KM_VF(DREG)                                                                        \
   do {                                                                                     \
     auto kern = lloyd_valu_fused_kernel<T, DREG, SUMS>;                                    \
     KM_VF_SETUP(kern);                                                                     \
     hipLaunchKernelGGL(kern, dim3(grid), dim3(WG), lds, s, X, xnorm, C, cnorm, labels,     \
-                       mindist, psums, pcounts, n, k, D, ldn);                             \
+                       mindist, psums, pcounts, n, k, D, ldn, ncopy);                      \
   } while (0)
   // any other d: dot products in registers, KREG >= k of them
 #define KM_VA_LAUNCH(DMAX, VEC, KREG)                                                      \
@@ -1818,7 +1862,7 @@ static int launch_valu_fused(hipStream_t s, const T *X, const T *xnorm, const T 
     auto kern = lloyd_valu_anyd_kernel<T, DMAX, VEC, KREG, SUMS>;                          \
     KM_VF_SETUP(kern);                                                                     \
     hipLaunchKernelGGL(kern, dim3(grid), dim3(WG), lds, s, X, xnorm, C, cnorm, labels,     \
-                       mindist, psums, pcounts, n, d, k, D, ldn);                          \
+                       mindist, psums, pcounts, n, d, k, D, ldn, ncopy);                   \
   } while (0)
 #define KM_VA_K(DMAX, VEC)                       \
   do {                                           \
@@ -1831,11 +1875,11 @@ static int launch_valu_fused(hipStream_t s, const T *X, const T *xnorm, const T 
     if (aligned && d >= vw) KM_VA_K(DMAX, Mfma<T>::VW);     \
     else KM_VA_K(DMAX, 1);                                  \
   } while (0)
-  if (aligned && d == 4) KM_VF(4);
-  else if (aligned && d == 8) KM_VF(8);
-  else if (aligned && d == 16) KM_VF(16);
-  else if (aligned && d == 32) KM_VF(32);
-  else if (aligned && d == 64) KM_VF(64);
+  if (reg && d == 4) KM_VF(4);
+  else if (reg && d == 8) KM_VF(8);
+  else if (reg && d == 16) KM_VF(16);
+  else if (reg && d == 32) KM_VF(32);
+  else if (reg && d == 64) KM_VF(64);
   else if (d <= 16) KM_VA(16);
   else if (d <= 32) KM_VA(32);
   else if (d <= 48) KM_VA(48);

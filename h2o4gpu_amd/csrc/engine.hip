@@ -17,6 +17,7 @@
 #include <ctime>
 #include <limits>
 #include <map>
+#include <tuple>
 #include <memory>
 #include <mutex>
 #include <new>
@@ -141,10 +142,31 @@ int ensure_dynamic_lds(const void *kernel, size_t bytes) {
   granted = bytes;
   return 0;
 }
+// (kernel, device, dynamic LDS) -> workgroups of `block` threads one CU holds at once
+static std::map<std::tuple<const void *, int, size_t>, int> g_resident;
+int resident_blocks_per_cu(const void *kernel, int block, size_t lds) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 1;
+  std::lock_guard<std::mutex> lock(g_lds_mu);
+  auto key = std::make_tuple(kernel, dev, lds);
+  auto it = g_resident.find(key);
+  if (it != g_resident.end()) return it->second;
+  int nb = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, kernel, block, lds) != hipSuccess || nb < 1) {
+    (void)hipGetLastError();
+    nb = 1;
+  }
+  g_resident[key] = nb;
+  return nb;
+}
 void forget_dynamic_lds(int dev) {
   std::lock_guard<std::mutex> lock(g_lds_mu);
   for (auto it = g_lds_granted.begin(); it != g_lds_granted.end();) {
     if (it->first.second == dev) it = g_lds_granted.erase(it);
+    else ++it;
+  }
+  for (auto it = g_resident.begin(); it != g_resident.end();) {
+    if (std::get<1>(it->first) == dev) it = g_resident.erase(it);
     else ++it;
   }
 }
@@ -1209,7 +1231,9 @@ struct Engine : h2o4gpu_kmeans_handle {
 
   // one Lloyd step: labels against the current centroids, then the update.
   // want_shift: the caller will read the convergence scalar of this step.
-  int step_async(bool want_shift) {
+  // want_mindist false: the step need not leave the rows' minimum distances behind (a later
+  // assignment pass will, before anyone reads them): one store per row less in the fused step.
+  int step_async(bool want_shift, bool want_mindist = true) {
     // (the exact-compare argmin exists in the assignment-only kernels)
     const bool exact_mfma = opt_exact && sizeof(T) == 4 &&
                             pick_assign_variant<T>(opt_assign, n, d, k) != ASSIGN_VALU;
@@ -1217,9 +1241,10 @@ struct Engine : h2o4gpu_kmeans_handle {
       int slots = 0;
       PROFILED("assign_accumulate",
                launch_assign_accumulate<T>(stream, opt_assign, X, xnorm, C[cur], (const T *)nullptr,
-                                           labels, mindist, n, d, k, num_cu, psums, pcounts, &slots,
-                                           &last_variant, shape(), opt_split));
-      have_mindist = true;
+                                           labels, (want_mindist || sets > 1) ? mindist : (T *)nullptr, n, d,
+                                           k, num_cu, psums, pcounts, &slots, &last_variant, shape(),
+                                           opt_split));
+      have_mindist = want_mindist || sets > 1;
       return finish_update(slots, want_shift);
     }
     if (sets > 1) return H2O4GPU_KMEANS_ESTATE;  // a stacked handle has no other step
@@ -1293,7 +1318,7 @@ struct Engine : h2o4gpu_kmeans_handle {
     } else {
       for (int i = 0; i < max_iterations; i++) {
         log_msg(verbose, LOG_VERBOSE, "KMeans - Iteration %d/%d", i, max_iterations);
-        KM_TRY(step_async(false));
+        KM_TRY(step_async(false, false));  // (the final relabel below leaves the minimum distances)
         updates++;
         bool done = false;
         if (g_stop_flag) {
@@ -1448,7 +1473,8 @@ struct Engine : h2o4gpu_kmeans_handle {
   int iterate(int steps) override {
     KM_HIP_TRY(hipSetDevice(dev));
     if (!have_data || !have_centroids) return H2O4GPU_KMEANS_ESTATE;
-    for (int i = 0; i < steps; i++) KM_TRY(step_async(false));
+    // only the last step's minimum distances can be read afterwards
+    for (int i = 0; i < steps; i++) KM_TRY(step_async(false, i == steps - 1));
     return 0;
   }
 

@@ -47,6 +47,11 @@ void log_msg(int verbose, int level, const char *fmt, ...)
 // remembered) instead of on every launch; forget_dynamic_lds drops what is remembered for
 // a device whose context was reset.
 int ensure_dynamic_lds(const void *kernel, size_t bytes);
+// How many workgroups of `block` threads with `lds` bytes of dynamic LDS one CU holds at once
+// (registers, LDS and wave slots all counted; asked of the runtime once per kernel instance,
+// device and size): the grid of a persistent kernel must not exceed this times the CUs, or its
+// last workgroups start only when the first ones have finished.
+int resident_blocks_per_cu(const void *kernel, int block, size_t lds);
 void forget_dynamic_lds(int dev);
 
 // Assign-kernel variants (value of the "assign" option).
