@@ -1521,6 +1521,374 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
 }
 
 // ---------------------------------------------------------------------------
+// Tiled kernel, operands staged by the memory system itself.
+//
+// The same tiling as assign_tiled_kernel for the shapes that need none of its special cases
+// (rows and centroids whole numbers of stages, 16-byte aligned rows, float32 instructions or
+// float64): here no operand passes through a register on its way to LDS. gfx950's
+// global_load_lds_dwordx4 lets every lane name a 16-byte source and writes the 64 vectors of a
+// wavefront to 64 consecutive 16-byte LDS slots, which is exactly one [tile][vector][lane]
+// block of the operand-order layout when lane (group g, row i) asks for vector q * KL + g of
+// the stage from row i of the tile. The stages form a ring of NBUF buffers and the loads run
+// NBUF - 1 stages ahead of the matrix instructions; a wavefront waits for its own loads of a
+// stage with s_waitcnt vmcnt (the loads of later stages stay in flight), the workgroup's
+// barrier then covers everybody else's, and the loads of the stage NBUF - 1 ahead are
+// issued right behind the barrier, into the buffer the stage before this one was read from.
+// All (centroid block, stage) pairs of a workgroup run as one pipeline, so a new centroid
+// block starts with its first stages already in LDS.
+//
+// The accumulators start at zero and -(xx + cc)/2 is added when a block is complete (the order
+// of a GEMM with beta = 1, which is what the reference runs, kmeans_labels.cu:158-165): the
+// partial sums of the dot product are then rounded at their own size instead of at the size
+// of xx + cc, which measured 1.5 times less rounding noise in the minimum distance at 256
+// features than accumulators that start at -(xx + cc)/2.
+// ---------------------------------------------------------------------------
+template <typename T, int BCW, bool WIDE, int BK, int NBUF>
+struct DmaCfg {
+  typedef Mfma<T> M;
+  static constexpr int TPB = 2 * BCW * 64;
+  static constexpr int BC = 64 * BCW * (WIDE ? 2 : 1);
+  static constexpr int BR = 128;
+  static constexpr int STAGE_ELEMS = (BC + BR) * BK;
+  // ring of stages + two copies of the block's centroid norms
+  static constexpr size_t LDS_BYTES = ((size_t)NBUF * STAGE_ELEMS + 2 * BC) * sizeof(T);
+};
+
+// One direct-to-LDS load: every lane's 16 bytes (4 for the narrow form) from its own global
+// address, the wavefront's 64 results to consecutive LDS slots starting at `lds` (the same
+// address in every lane). The builtin exists for the gfx950 target only; the host pass of the
+// compiler, which has to see the kernel's body to emit its launch stub, gets an empty function.
+__device__ __forceinline__ void dma_to_lds_16(const void *gsrc, void *lds) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __builtin_amdgcn_global_load_lds(gsrc, (__attribute__((address_space(3))) void *)(lds), 16, 0, 0);
+#else
+  (void)gsrc;
+  (void)lds;
+#endif
+}
+// s_waitcnt vmcnt(N) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, the other counters at
+// "do not wait")
+#define KM_WAIT_VMCNT(N) __builtin_amdgcn_s_waitcnt(0x0F70 | ((N) & 15) | (((N) >> 4) << 14))
+
+template <typename T, int MODE, int BCW, bool EXACT, bool WIDE, int BK, int NBUF, bool SPREAD>
+__global__ __launch_bounds__(2 * BCW * 64, 2) void assign_tiled_dma_kernel(
+    const T *__restrict__ X, const T *__restrict__ xnorm,
+    const T *__restrict__ C, const T *__restrict__ cnorm,
+    int *__restrict__ labels, T *__restrict__ mindist, T *__restrict__ D,
+    int64_t n, int64_t ldn, int d, int k) {
+  typedef Mfma<T> M;
+  typedef DmaCfg<T, BCW, WIDE, BK, NBUF> Cfg;
+  constexpr int MT = M::MT, KL = M::KL, NACC = M::NACC, VW = M::VW;
+  constexpr int BC = Cfg::BC, BR = Cfg::BR, NWAVE = Cfg::TPB / 64;
+  constexpr int NV = BK / KL / VW;   // 16-byte vectors per lane per tile per stage
+  constexpr int CT = BC / BCW / MT;  // centroid tiles per wavefront
+  constexpr int RT = BR / 2 / MT;    // row tiles per wavefront
+  constexpr int TILE_ELEMS = MT * BK;
+  constexpr int A_TILES = BC / MT, B_TILES = BR / MT;
+  constexpr int A_TPW = A_TILES / NWAVE, B_TPW = B_TILES / NWAVE;  // tiles a wavefront fetches
+  constexpr int A_ELEMS = A_TILES * TILE_ELEMS;  // the A part of a stage
+  constexpr int STAGE_ELEMS = Cfg::STAGE_ELEMS;
+  static_assert(A_TILES % NWAVE == 0 && B_TILES % NWAVE == 0, "tiles are dealt evenly to the wavefronts");
+  static_assert(BK % (KL * VW) == 0 && NBUF >= 2 && NBUF <= 4, "whole vectors per lane group");
+  constexpr int LPW = (A_TPW + B_TPW) * NV;  // loads per wavefront and stage
+  constexpr int AHEAD = NBUF - 1;
+  static_assert((AHEAD - 1) * LPW < 64, "vmcnt is a 6-bit counter");
+  typedef typename M::acc_t acc_t;
+  typedef typename M::vec_t vec_t;
+
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wc = wave % BCW;
+  const int wr = wave / BCW;
+  const int r = lane % MT;
+  const int g = lane / MT;
+  T *ring = reinterpret_cast<T *>(smem_raw);   // [NBUF][A tiles | B tiles]
+  T *cns = ring + (size_t)NBUF * STAGE_ELEMS;  // [2][BC]: squared norms of the current block's centroids
+  const int ncb = (k + BC - 1) / BC;
+  const int64_t rt_id = MODE == 1 ? (int64_t)blockIdx.x / ncb : (int64_t)blockIdx.x;
+  const int cb_id = MODE == 1 ? (int)((int64_t)blockIdx.x - rt_id * ncb) : 0;
+  const int64_t row0 = rt_id * BR;
+  const int nstage = d / BK;
+  const int c_begin = MODE == 1 ? cb_id * BC : 0;
+  const int nblk = MODE == 1 ? 1 : ncb;
+  const int total = nblk * nstage;  // stages of this workgroup's pipeline
+
+  // What this lane fetches: vector g (+ q * KL) of the stage from row r of each tile the
+  // wavefront is responsible for, as a byte offset from a base that is the same for the whole
+  // workgroup (the block's first centroid, the workgroup's first row): the loads then take
+  // their address as scalar base + 32-bit lane offset and cost no vector arithmetic.
+  unsigned aoff[A_TPW], boff[B_TPW];
+#pragma unroll
+  for (int t = 0; t < A_TPW; t++)
+    aoff[t] = (unsigned)((((wave * A_TPW + t) * MT + r) * (size_t)d + g * VW) * sizeof(T));
+#pragma unroll
+  for (int t = 0; t < B_TPW; t++) {
+    const int64_t row = min(row0 + (wave * B_TPW + t) * MT + r, n - 1);  // clamped: stays inside X
+    boff[t] = (unsigned)(((row - row0) * (int64_t)d + g * VW) * sizeof(T));
+  }
+  const char *const xbase = reinterpret_cast<const char *>(X + row0 * (int64_t)d);
+  // the pipeline's fetch position: stage ist of block iblk goes to ring slot ibuf
+  int iblk = 0, ist = 0, ibuf = 0, issued = 0;
+  // The burst form takes the tiles one after the other, the NV vectors of a tile in a row:
+  // they ask for adjacent pieces of the same 32 (16) rows, i.e. of the same cache lines.
+  // vector q of every tile the wavefront fetches (the order the 256-centroid block of a fit
+  // prefers when the loads are spread over the stage: 500k x 784, k = 4096 23.7 against 24.5 ms)
+  auto issue_part = [&](int q) {
+    T *dst = ring + (size_t)ibuf * STAGE_ELEMS;
+    const char *abase = reinterpret_cast<const char *>(C + ((size_t)(c_begin + iblk * BC) * d + (size_t)ist * BK));
+    const char *bbase = xbase + (size_t)ist * BK * sizeof(T);
+#pragma unroll
+    for (int t = 0; t < A_TPW; t++)
+      dma_to_lds_16(abase + q * KL * VW * sizeof(T) + aoff[t], dst + ((wave * A_TPW + t) * NV + q) * 64 * VW);
+#pragma unroll
+    for (int t = 0; t < B_TPW; t++)
+      dma_to_lds_16(bbase + q * KL * VW * sizeof(T) + boff[t],
+                    dst + A_ELEMS + ((wave * B_TPW + t) * NV + q) * 64 * VW);
+  };
+  auto issue_done = [&]() {
+    issued++;
+    ibuf = ibuf + 1 == NBUF ? 0 : ibuf + 1;
+    if (++ist == nstage) {
+      ist = 0;
+      iblk++;
+    }
+  };
+  // all of a stage's loads, tile by tile
+  auto issue_all = [&]() {
+    T *dst = ring + (size_t)ibuf * STAGE_ELEMS;
+    const char *abase = reinterpret_cast<const char *>(C + ((size_t)(c_begin + iblk * BC) * d + (size_t)ist * BK));
+    const char *bbase = xbase + (size_t)ist * BK * sizeof(T);
+#pragma unroll
+    for (int t = 0; t < A_TPW; t++) {
+#pragma unroll
+      for (int q = 0; q < NV; q++)
+        dma_to_lds_16(abase + q * KL * VW * sizeof(T) + aoff[t], dst + ((wave * A_TPW + t) * NV + q) * 64 * VW);
+    }
+#pragma unroll
+    for (int t = 0; t < B_TPW; t++) {
+#pragma unroll
+      for (int q = 0; q < NV; q++)
+        dma_to_lds_16(bbase + q * KL * VW * sizeof(T) + boff[t],
+                      dst + A_ELEMS + ((wave * B_TPW + t) * NV + q) * 64 * VW);
+    }
+  };
+  auto issue = [&]() {
+    issue_all();
+    issue_done();
+  };
+
+  T xxh[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; rt++)
+    xxh[rt] = (T)-0.5 * xnorm[min(row0 + (wr * RT + rt) * MT + r, n - 1)];
+  T best[RT];
+  int bidx[RT];
+  unsigned bkey[RT];
+  int bblk[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; rt++) {
+    best[rt] = (T)0.5 * argmin_start<T>();  // the start value FLT_MAX on the accumulators' scale
+    bidx[rt] = -1;
+    bkey[rt] = 0x7EFFFFF0u;  // FLT_MAX / 2 with the index bits cleared
+    bblk[rt] = -1;
+  }
+
+#pragma unroll
+  for (int a = 0; a < AHEAD; a++)
+    if (issued < total) issue();
+  // the row norms are in their registers before the loop starts (the loads above, issued
+  // after them, stay in flight): no wait for them can end up inside the pipeline
+#pragma unroll
+  for (int rt = 0; rt < RT; rt++) asm volatile("" : "+v"(xxh[rt]));
+
+  int buf = 0, done = 0;
+  for (int blk = 0; blk < nblk; blk++) {
+    const int c0 = c_begin + blk * BC;
+    // This block's centroid norms for the epilogue, fetched the same way (64 lanes x 16 bytes
+    // cover the block); they have landed and are visible to everybody at the latest after the
+    // second barrier below. The copy of the block before stays readable for wavefronts that
+    // are still in its epilogue.
+    T *cn = cns + (blk & 1) * BC;
+    static_assert(BC / VW <= 64, "one wavefront fetches the block's norms");
+    if (wave == 0 && lane < BC / VW) dma_to_lds_16(cnorm + c0 + lane * VW, cn);
+    acc_t acc[CT][RT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ct++) {
+#pragma unroll
+      for (int rt = 0; rt < RT; rt++) {
+#pragma unroll
+        for (int v = 0; v < NACC; v++) acc[ct][rt][v] = (T)0;
+      }
+    }
+    for (int st = 0; st < nstage; st++) {
+      // this wavefront's loads of the stage have landed (those of the AHEAD - 1 stages after it
+      // may still be under way), then everybody's
+      if (AHEAD > 1 && issued - done >= AHEAD) KM_WAIT_VMCNT((AHEAD - 1) * LPW);
+      else KM_WAIT_VMCNT(0);
+      __syncthreads();
+      const bool more = issued < total;  // the next stage to fetch goes into the slot read one stage ago
+      // SPREAD: a part of the next stage's loads in front of every step's matrix instructions
+      // instead of all of them in front of the stage.
+      if constexpr (!SPREAD) {
+        if (more) issue_all();
+      }
+      __builtin_amdgcn_s_setprio(3);
+      const vec_t *ap = reinterpret_cast<const vec_t *>(ring + (size_t)buf * STAGE_ELEMS) + lane;
+      const vec_t *bp = ap + A_ELEMS / VW;
+      if constexpr (sizeof(T) == 4) __builtin_amdgcn_iglp_opt(0);
+#pragma unroll
+      for (int q = 0; q < NV; q++) {
+        if constexpr (SPREAD) {
+          if (more) issue_part(q);
+        }
+        vec_t a[CT], b[RT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ct++) a[ct] = ap[((wc * CT + ct) * NV + q) * 64];
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) b[rt] = bp[((wr * RT + rt) * NV + q) * 64];
+#pragma unroll
+        for (int e = 0; e < VW; e++) {
+#pragma unroll
+          for (int ct = 0; ct < CT; ct++) {
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++)
+              acc[ct][rt] = M::mma(a[ct][e], b[rt][e], acc[ct][rt]);
+          }
+        }
+      }
+      __builtin_amdgcn_s_setprio(0);
+      if (more) issue_done();
+      done++;
+      buf = buf + 1 == NBUF ? 0 : buf + 1;
+    }
+    if (nstage < NBUF) {  // too few waits since the norms were asked for: wait for them here
+      KM_WAIT_VMCNT(0);
+      __syncthreads();
+    }
+    // epilogue of the block: a = x.c - (xx + cc)/2, i.e. -1/2 of the reference's value with its
+    // rounding order ((xx + cc) first, then the product term); -(xx + cc)/2 as one fused
+    // multiply-add of exact terms, i.e. rounded once like xx + cc itself
+    if (MODE == 1) {
+#pragma unroll
+      for (int ct = 0; ct < CT; ct++) {
+#pragma unroll
+        for (int v = 0; v < NACC; v++) {
+          const int cl = (wc * CT + ct) * MT + M::acc_row(v, g);
+          const T cc = cn[cl];
+#pragma unroll
+          for (int rt = 0; rt < RT; rt++) {
+            const int64_t row = row0 + (wr * RT + rt) * MT + r;
+            const T a = acc[ct][rt][v] + fma((T)-0.5, cc, xxh[rt]);
+            if (c0 + cl < k && row < n) D[(size_t)(c0 + cl) * ldn + row] = (T)2 * fabs(a);
+          }
+        }
+      }
+    } else if constexpr (sizeof(T) == 4 && !EXACT) {
+#pragma unroll
+      for (int ct = 0; ct < CT; ct++) {
+        T ccv[NACC];
+#pragma unroll
+        for (int v = 0; v < NACC; v++) ccv[v] = cn[(wc * CT + ct) * MT + M::acc_row(v, g)];
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) {
+          unsigned key[NACC];
+#pragma unroll
+          for (int v = 0; v < NACC; v++)
+            key[v] = (__float_as_uint(acc[ct][rt][v] + fmaf(-0.5f, ccv[v], xxh[rt])) & 0x7FFFFFF0u) | (unsigned)v;
+          unsigned m = umin3(key[0], key[1], key[2]);
+#pragma unroll
+          for (int v = 3; v + 1 < NACC; v += 2) m = umin3(m, key[v], key[v + 1]);
+          if ((NACC & 1) == 0) m = min(m, key[NACC - 1]);
+          if ((m | 15u) < bkey[rt]) {
+            bkey[rt] = m;
+            bblk[rt] = c0 + (wc * CT + ct) * MT;
+          }
+        }
+      }
+    } else {
+      int loc[RT];
+#pragma unroll
+      for (int rt = 0; rt < RT; rt++) loc[rt] = -1;
+#pragma unroll
+      for (int ct = 0; ct < CT; ct++) {
+#pragma unroll
+        for (int v = 0; v < NACC; v++) {
+          const T cc = cn[(wc * CT + ct) * MT + M::acc_row(v, g)];
+#pragma unroll
+          for (int rt = 0; rt < RT; rt++) {
+            const T a = acc[ct][rt][v] + fma((T)-0.5, cc, xxh[rt]);
+            if (fabs(a) < fabs(best[rt])) {
+              best[rt] = a;
+              loc[rt] = ct * NACC + v;
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int rt = 0; rt < RT; rt++) {
+        if (loc[rt] >= 0) {
+          bblk[rt] = c0;
+          bidx[rt] = loc[rt];
+        }
+      }
+    }
+  }
+  if (MODE == 0) {
+    if constexpr (sizeof(T) == 4 && !EXACT) {
+#pragma unroll
+      for (int rt = 0; rt < RT; rt++) {
+        best[rt] = __uint_as_float(bkey[rt] & 0xFFFFFFF0u);
+        bidx[rt] = bblk[rt] < 0 ? -1 : bblk[rt] + key_row(bkey[rt] & 15u, g);
+      }
+    } else {
+#pragma unroll
+      for (int rt = 0; rt < RT; rt++) {
+        best[rt] = fabs(best[rt]);
+        if (bblk[rt] >= 0)
+          bidx[rt] = bblk[rt] + (wc * CT + bidx[rt] / NACC) * MT + M::acc_row(bidx[rt] % NACC, g);
+      }
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++) {
+#pragma unroll
+      for (int off = MT; off < 64; off <<= 1) {
+        const T ob = __shfl_xor(best[rt], off, 64);
+        const int oi = __shfl_xor(bidx[rt], off, 64);
+        argmin_merge(best[rt], bidx[rt], ob, oi);
+      }
+    }
+    __syncthreads();  // all waves are past their last LDS operand read
+    T *mb = reinterpret_cast<T *>(smem_raw);                   // [BCW-1][BR]
+    int *mi = reinterpret_cast<int *>(mb + (BCW - 1) * BR);    // [BCW-1][BR]
+    if (wc > 0 && g == 0) {
+#pragma unroll
+      for (int rt = 0; rt < RT; rt++) {
+        const int lr = (wr * RT + rt) * MT + r;
+        mb[(wc - 1) * BR + lr] = best[rt];
+        mi[(wc - 1) * BR + lr] = bidx[rt];
+      }
+    }
+    __syncthreads();
+    if (wc == 0 && g == 0) {
+#pragma unroll
+      for (int rt = 0; rt < RT; rt++) {
+        const int lr = (wr * RT + rt) * MT + r;
+#pragma unroll
+        for (int w = 0; w < BCW - 1; w++)
+          argmin_merge(best[rt], bidx[rt], mb[w * BR + lr], mi[w * BR + lr]);
+        const int64_t row = row0 + lr;
+        if (row < n) {
+          labels[row] = bidx[rt];
+          if (mindist) mindist[row] = (T)2 * best[rt];
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 const char *assign_variant_name(int variant) {
@@ -1911,6 +2279,39 @@ int launch_assign_accumulate(hipStream_t s, int variant, const T *X, const T *xn
                                        num_cu, psums, pcounts, slots, 0, 0, false, st, split);
 }
 
+// The kernel whose operands are staged by direct-to-LDS loads: rows and centroids whole
+// numbers of BK-feature stages and 16-byte aligned. Returns 1 when the shape is not its.
+template <typename T, int MODE, int BCW, bool WIDE, int BK, int NBUF, bool SPREAD>
+static int launch_tiled_dma(hipStream_t s, const T *X, const T *xnorm, const T *C, const T *cnorm,
+                            int *labels, T *mindist, T *D, int64_t n, int64_t ldn, int d, int k,
+                            bool exact) {
+  typedef DmaCfg<T, BCW, WIDE, BK, NBUF> Cfg;
+  const uintptr_t bits = reinterpret_cast<uintptr_t>(X) | reinterpret_cast<uintptr_t>(C) |
+                         reinterpret_cast<uintptr_t>(cnorm);
+  if (d % BK != 0 || (bits & 15) != 0 || ((size_t)d * sizeof(T)) % 16 != 0) return 1;
+  const int64_t row_tiles = (n + Cfg::BR - 1) / Cfg::BR;
+  const int64_t tiles = MODE == 1 ? row_tiles * ((k + Cfg::BC - 1) / Cfg::BC) : row_tiles;
+  if (tiles > 2147483647ll) return H2O4GPU_KMEANS_EARG;
+  const size_t lds = Cfg::LDS_BYTES;
+#define KM_DMA_X(EXACT)                                                                      \
+  do {                                                                                       \
+    auto kern = assign_tiled_dma_kernel<T, MODE, BCW, EXACT, WIDE, BK, NBUF, SPREAD>;        \
+    KM_TRY(ensure_dynamic_lds(reinterpret_cast<const void *>(kern), lds));                   \
+    hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(Cfg::TPB), lds, s, X, xnorm, C,     \
+                       cnorm, labels, mindist, D, n, ldn, d, k);                             \
+  } while (0)
+  if (d >= 128) exact = true;  // as in launch_tiled_bcw
+  if constexpr (MODE == 0 && sizeof(T) == 4) {
+    if (exact) KM_DMA_X(true);
+    else KM_DMA_X(false);
+  } else {
+    KM_DMA_X(false);
+  }
+#undef KM_DMA_X
+  KM_HIP_TRY(hipGetLastError());
+  return 0;
+}
+
 template <typename T, int MODE, int BCW, bool WIDE = false, int SPLIT = 0>
 static int launch_tiled_bcw(hipStream_t s, const T *X, const T *xnorm, const T *C,
                             const T *cnorm, int *labels, T *mindist, T *D, int64_t n,
@@ -1925,6 +2326,26 @@ static int launch_tiled_bcw(hipStream_t s, const T *X, const T *xnorm, const T *
     hipLaunchKernelGGL(split_centroids_kernel, dim3((unsigned)std::min<int64_t>((items + 255) / 256, 4096)),
                        dim3(256), 0, s, reinterpret_cast<const float *>(C), static_cast<uintx4 *>(cparts), k,
                        d, Cfg::BC, nstage, nblocks);
+  }
+  if constexpr (SPLIT == 0 && BCW == 2) {
+    // Stage depth, ring size and issue order per shape, each measured against the others and
+    // against the kernel that stages through registers in alternating runs on one machine:
+    // 128-centroid block, float32: 32 features, 2 buffers (2M x 256, k = 1024: 8.16 against 8.20 ms;
+    // 16 features with 3 buffers 8.28); 256-centroid block in a fit: 16 features, 2 buffers, loads
+    // spread over the stage (500k x 784, k = 4096: 23.9 against 24.6 ms; in one go 24.4); its
+    // transform: in one go (100,000 rows: 5.46 against 5.59 ms; spread 5.57); float64: 16
+    // features, 2 buffers (2M x 256, k = 1024: 15.8 against 16.1 ms; 3 buffers 17.6).
+    int rc = 1;
+    if constexpr (sizeof(T) == 8)
+      rc = launch_tiled_dma<T, MODE, BCW, WIDE, 16, 2, false>(s, X, xnorm, C, cnorm, labels, mindist, D, n, ldn,
+                                                              d, k, exact);
+    else if constexpr (!WIDE)
+      rc = launch_tiled_dma<T, MODE, BCW, WIDE, 32, 2, false>(s, X, xnorm, C, cnorm, labels, mindist, D, n, ldn,
+                                                              d, k, exact);
+    else
+      rc = launch_tiled_dma<T, MODE, BCW, WIDE, 16, 2, MODE == 0>(s, X, xnorm, C, cnorm, labels, mindist, D, n,
+                                                                  ldn, d, k, exact);
+    if (rc != 1) return rc;
   }
   const int64_t row_tiles = (n + Cfg::BR - 1) / Cfg::BR;
   const int64_t tiles = MODE == 1 ? row_tiles * ((k + Cfg::BC - 1) / Cfg::BC) : row_tiles;
