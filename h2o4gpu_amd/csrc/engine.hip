@@ -1703,20 +1703,24 @@ __global__ void copy_probe_kernel(const float4 *__restrict__ src, float4 *__rest
 
 // Read-only stream: every thread keeps four 16-byte loads in flight and adds what arrives;
 // one value per thread leaves at the end (so the loads cannot be dropped).
-__global__ __launch_bounds__(256) void read_probe_kernel(const float4 *__restrict__ src,
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void read_probe_kernel(const floatx4 *__restrict__ src,
                                                          float *__restrict__ out, size_t nvec) {
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  float4 a0 = {0, 0, 0, 0}, a1 = a0, a2 = a0, a3 = a0;
+  floatx4 a0 = {0, 0, 0, 0}, a1 = a0, a2 = a0, a3 = a0;
   for (; i + 3 * stride < nvec; i += 4 * stride) {
-    const float4 v0 = src[i], v1 = src[i + stride], v2 = src[i + 2 * stride], v3 = src[i + 3 * stride];
+    // (loads that do not displace cached lines: 6.0 against 5.5 TB/s with plain ones)
+    const floatx4 v0 = __builtin_nontemporal_load(&src[i]), v1 = __builtin_nontemporal_load(&src[i + stride]),
+                  v2 = __builtin_nontemporal_load(&src[i + 2 * stride]),
+                  v3 = __builtin_nontemporal_load(&src[i + 3 * stride]);
     a0.x += v0.x; a0.y += v0.y; a0.z += v0.z; a0.w += v0.w;
     a1.x += v1.x; a1.y += v1.y; a1.z += v1.z; a1.w += v1.w;
     a2.x += v2.x; a2.y += v2.y; a2.z += v2.z; a2.w += v2.w;
     a3.x += v3.x; a3.y += v3.y; a3.z += v3.z; a3.w += v3.w;
   }
   for (; i < nvec; i += stride) {
-    const float4 v0 = src[i];
+    const floatx4 v0 = src[i];
     a0.x += v0.x; a0.y += v0.y; a0.z += v0.z; a0.w += v0.w;
   }
   out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] =
@@ -2303,7 +2307,7 @@ KM_API int h2o4gpu_kmeans_bandwidth_probe(int gpu_id, int kind, size_t bytes, in
   void *a = nullptr, *b = nullptr;
   float *sink = nullptr;
   if (hipMalloc(&a, bytes) != hipSuccess || hipMalloc(&b, bytes) != hipSuccess ||
-      hipMalloc(reinterpret_cast<void **>(&sink), (size_t)grid * block * sizeof(float)) != hipSuccess) {
+      hipMalloc(reinterpret_cast<void **>(&sink), (size_t)2 * grid * block * sizeof(float)) != hipSuccess) {
     (void)hipGetLastError();
     if (a) (void)hipFree(a);
     if (b) (void)hipFree(b);
@@ -2320,7 +2324,7 @@ KM_API int h2o4gpu_kmeans_bandwidth_probe(int gpu_id, int kind, size_t bytes, in
       if (kind == H2O4GPU_KMEANS_PROBE_COPY)
         hipLaunchKernelGGL(copy_probe_kernel, dim3(grid), dim3(block), 0, 0, (const float4 *)a, (float4 *)b, nvec);
       else if (kind == H2O4GPU_KMEANS_PROBE_READ)
-        hipLaunchKernelGGL(read_probe_kernel, dim3(grid), dim3(block), 0, 0, (const float4 *)a, sink, nvec);
+        hipLaunchKernelGGL(read_probe_kernel, dim3(grid * 2), dim3(block), 0, 0, (const floatx4 *)a, sink, nvec);
       else if (kind == H2O4GPU_KMEANS_PROBE_WRITE)
         hipLaunchKernelGGL(fill_probe_kernel, dim3(grid), dim3(block), 0, 0, (float4 *)b, nvec, 1.0f);
       else

@@ -248,8 +248,11 @@ int h2o4gpu_kmeans_transform_resident(h2o4gpu_kmeans_handle *h, void *d_dist);
  * buffers, so that a batch is computed while the previous one is downloaded (this is also
  * what happens with 1, one batch at a time, when the second set cannot be allocated).
  * "seed_matrix" = 1 (default) lets init_parallel compute the distances between its
- * candidates as one matrix (while it fits 1 GiB) and pick the centres on the host from it;
- * 0 runs one small kernel per pick, as "assign" = 1 always does.
+ * candidates as one matrix (while it fits 1 GiB) and pick the centres on the host from it:
+ * for the duration of the seeding that takes up to 1 GiB of device memory and as much host
+ * memory for the downloaded copy (M x M values for M candidates; when either allocation
+ * fails the picks fall back to the other form); 0 runs one small kernel per pick, as
+ * "assign" = 1 always does.
  * Unknown names return EARG. */
 int h2o4gpu_kmeans_set_option(h2o4gpu_kmeans_handle *h, const char *name,
                               int value);
