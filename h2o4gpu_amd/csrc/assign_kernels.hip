@@ -2317,7 +2317,8 @@ static int launch_tiled_dma(hipStream_t s, const T *X, const T *xnorm, const T *
 template <typename T, int MODE, int BCW, bool WIDE = false, int SPLIT = 0>
 static int launch_tiled_bcw(hipStream_t s, const T *X, const T *xnorm, const T *C,
                             const T *cnorm, int *labels, T *mindist, T *D, int64_t n,
-                            int64_t ldn, int d, int k, bool exact, void *cparts = nullptr) {
+                            int64_t ldn, int d, int k, bool exact, void *cparts = nullptr,
+                            bool direct = true) {
   typedef TiledCfg<T, BCW, WIDE, SPLIT> Cfg;
   const size_t lds = Cfg::LDS_BYTES;
   if constexpr (SPLIT != 0) {
@@ -2329,7 +2330,7 @@ static int launch_tiled_bcw(hipStream_t s, const T *X, const T *xnorm, const T *
                        dim3(256), 0, s, reinterpret_cast<const float *>(C), static_cast<uintx4 *>(cparts), k,
                        d, Cfg::BC, nstage, nblocks);
   }
-  if constexpr (SPLIT == 0 && BCW == 2) {
+  if constexpr (SPLIT == 0 && BCW == 2) if (direct) {
     // Stage depth, ring size and issue order per shape, each measured against the others and
     // against the kernel that stages through registers in alternating runs on one machine:
     // 128-centroid block, float32: 32 features, 2 buffers (2M x 256, k = 1024: 8.16 against 8.20 ms;
@@ -2415,6 +2416,7 @@ static int launch_tiled(hipStream_t s, const T *X, const T *xnorm, const T *C,
                         const T *cnorm, int *labels, T *mindist, T *D, int64_t n,
                         int64_t ldn, int d, int k, bool exact = false, int split = 0,
                         SplitScratch scratch = SplitScratch()) {
+  const bool direct = !scratch.through_registers;
   if constexpr (sizeof(T) == 4) {
     const bool wide = tiled_split_wide(k);
     const size_t need = tiled_split_scratch_bytes<T>(split, d, k);
@@ -2444,9 +2446,21 @@ static int launch_tiled(hipStream_t s, const T *X, const T *xnorm, const T *C,
   // L2 miss path); while the model fits L2 it is behind (2M x 256, k = 1024: 8.37 -> 8.53 ms).
   if constexpr (sizeof(T) == 4) {
     if ((size_t)k * d * sizeof(T) > ((size_t)4 << 20))
-      return launch_tiled_bcw<T, MODE, 2, true>(s, X, xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k, exact);
+      return launch_tiled_bcw<T, MODE, 2, true>(s, X, xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k, exact,
+                                                nullptr, direct);
+    // With the operands staged by direct loads the 256-centroid block is ahead for models that
+    // stay in L2 as well (2M x 256, k = 1024: 7.95 against 8.11 ms in alternating runs): half as
+    // many bytes fetched and read back from LDS per matrix instruction. Taken whenever its
+    // padding of the model costs nothing (or next to nothing) over the 128-centroid block's.
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(X) | reinterpret_cast<uintptr_t>(C) |
+                           reinterpret_cast<uintptr_t>(cnorm);
+    const int64_t pad256 = ((int64_t)k + 255) / 256 * 256, pad128 = ((int64_t)k + 127) / 128 * 128;
+    if (direct && MODE == 0 && d % 16 == 0 && (bits & 15) == 0 && pad256 * 50 <= pad128 * 51)
+      return launch_tiled_bcw<T, MODE, 2, true>(s, X, xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k, exact,
+                                                nullptr, true);
   }
-  return launch_tiled_bcw<T, MODE, 2>(s, X, xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k, exact);
+  return launch_tiled_bcw<T, MODE, 2>(s, X, xnorm, C, cnorm, labels, mindist, D, n, ldn, d, k, exact, nullptr,
+                                      direct);
 }
 
 template <typename T>

@@ -207,6 +207,7 @@ struct h2o4gpu_kmeans_handle {
   int opt_split = 0;    // 6 or 9: float32 matrix-core kernels as that many bfloat16 products per feature pair
   int opt_transform_buffers = 2;  // sets of device buffers of a transform in several batches
   int opt_seed_matrix = 1;  // k-means||: distances between candidates as one matrix (0: a kernel per pick)
+  int opt_tiled_direct = 1;  // tiled kernels: operands by direct-to-LDS loads where the shape allows
   int opt_transform_batch_mb = 4096;  // device buffer of transform_host's output, per batch of rows
   int last_variant = ASSIGN_AUTO;
 
@@ -620,6 +621,7 @@ struct Engine : h2o4gpu_kmeans_handle {
   SplitScratch split_scratch() { return split_scratch(k); }
   SplitScratch split_scratch(int model_rows) {  // (the seeding runs models of other sizes)
     SplitScratch sc;
+    sc.through_registers = opt_tiled_direct == 0;
     const size_t need = opt_split ? tiled_split_scratch_bytes<T>(opt_split, d, model_rows) : 0;
     if (need == 0) return sc;
     if (need > split_bytes) {
@@ -2238,6 +2240,11 @@ KM_API int h2o4gpu_kmeans_set_option(h2o4gpu_kmeans_handle *h, const char *name,
   if (strcmp(name, "transform_buffers") == 0) {
     if (value != 1 && value != 2) return H2O4GPU_KMEANS_EARG;
     h->opt_transform_buffers = value;
+    return 0;
+  }
+  if (strcmp(name, "tiled_direct") == 0) {
+    if (value != 0 && value != 1) return H2O4GPU_KMEANS_EARG;
+    h->opt_tiled_direct = value;
     return 0;
   }
   if (strcmp(name, "seed_matrix") == 0) {

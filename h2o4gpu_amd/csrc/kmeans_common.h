@@ -84,6 +84,9 @@ struct StackShape {
 struct SplitScratch {
   void *ptr = nullptr;
   size_t bytes = 0;
+  // tiled kernels: stage the operands through registers also where the direct-to-LDS form
+  // applies (handle option "tiled_direct" = 0)
+  bool through_registers = false;
 };
 
 // Fused distance + argmin. labels[i] = argmin_c |(xx_i + cc_c) - 2 x_i.c_c|,

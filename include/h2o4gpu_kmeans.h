@@ -247,6 +247,11 @@ int h2o4gpu_kmeans_transform_resident(h2o4gpu_kmeans_handle *h, void *d_dist);
  * "transform_buffers" = 2 (default) gives a transform in several batches two sets of device
  * buffers, so that a batch is computed while the previous one is downloaded (this is also
  * what happens with 1, one batch at a time, when the second set cannot be allocated).
+ * "tiled_direct" = 1 (default) lets the tiled matrix-core kernels fetch their operands with
+ * direct-to-LDS loads wherever rows and centroids are whole stages and 16-byte aligned; 0
+ * stages them through registers everywhere (the form that serves every other shape). Same
+ * labels up to near-ties: the two forms add the norms to the dot product at different ends
+ * of the sum.
  * "seed_matrix" = 1 (default) lets init_parallel compute the distances between its
  * candidates as one matrix (while it fits 1 GiB) and pick the centres on the host from it:
  * for the duration of the seeding that takes up to 1 GiB of device memory and as much host
