@@ -283,6 +283,10 @@ def main():
                     help="keep assignment and accumulation as separate kernels")
     ap.add_argument("--transform-rows", type=int, default=0,
                     help="also time transform (full distance matrix) on this many held-out rows (C5)")
+    ap.add_argument("--operands", default="generator", choices=["generator", "zeros", "ones", "normal"],
+                    help="replace the values of the workload's rows (same shape, same kernels, same "
+                         "instruction stream) by zeros, ones or unit-variance noise: shows how far the "
+                         "chip's clock, and with it the kernel's time, follows the bit patterns it works on")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-iters", type=int, default=0, help="CPU baseline iterations (0 = about 12 s worth)")
     ap.add_argument("--sklearn-rows", type=int, default=10_000_000,
@@ -326,6 +330,11 @@ def main():
     X, k, _ = datasets.make(args.workload, args.scale, dtype)
     n, d = X.shape
     seed = datasets.SHAPES[args.workload][3]
+    if args.operands != "generator":
+        if args.operands == "normal":
+            X = np.random.default_rng(seed).standard_normal(X.shape, dtype=dtype)
+        else:
+            X = np.full(X.shape, 0.0 if args.operands == "zeros" else 1.0, dtype)
     C0 = datasets.seeded_row_init(X, k, seed)
     log("generated %s: %d x %d %s, k=%d in %.1f s" % (args.workload, n, d, X.dtype, k,
                                                     time.perf_counter() - t0))
@@ -340,7 +349,7 @@ def main():
     t0 = time.perf_counter()
     h.set_data(X)
     h2d_s = time.perf_counter() - t0
-    if args.workload == "C4":  # the benchmark text starts this shape from k-means++
+    if args.workload == "C4" and args.operands == "generator":  # the benchmark text starts this shape from k-means++
         h.init_plusplus(seed)
         C0 = h.centroids()
     h.set_centroids(C0)
@@ -453,7 +462,8 @@ def main():
         "dtype": args.dtype, "data": "synthetic",
         "config": {"workload": "%s: %d x %d %s, k=%d, %s; one step = assign + centroid update"
                                % (args.workload, n, d, args.dtype, k, WORKLOAD_TEXT[args.workload]),
-                   "rows": n, "cols": d, "k": k, "assign_variant": variant},
+                   "rows": n, "cols": d, "k": k, "assign_variant": variant,
+                   "operands": args.operands},
         "roofline": roofline,
         "traffic_measurement": traffic_details,
         "iteration": {"algorithmic_bytes": bytes_per_iter, "algorithmic_flops": flops_per_iter,
