@@ -91,3 +91,46 @@ def test_unaligned_rows_fall_back_to_registers(hip, oracle):
     finally:
         rt.hipFree(buf)
     label_report(oracle, X, C, L, oracle.assign(X, C, threads=4))
+
+
+@pytest.mark.parametrize("n,d,k,direct", [
+    (20000, 256, 1024, 1),    # direct loads
+    (20000, 256, 1024, 0),    # the same shape staged through registers
+    (20000, 298, 1000, 1),    # rows that are not whole stages: through registers whatever the option says
+    (20000, 142, 40, 1),      # the 64-centroid block
+])
+def test_float32_distances_carry_the_rounding_noise_of_a_scalar_loop(hip, oracle, n, d, k, direct):
+    """Both forms of the tiled kernel sum the dot product from zero and add -(xx + cc)/2 when a
+    block of centroids is complete, which is the order of the reference's GEMM with beta = 1
+    (kmeans_labels.cu:158-165) and of the oracle's scalar loop. Accumulators that start at
+    -(xx + cc)/2 round every partial sum at the size of xx + cc and carry 1.5 times the noise
+    (rms 3.0 against 2.0 eps (xx + cc) at 256 features), which flips near-tie rows that a scalar
+    loop decides the other way. Measured here: the error of every returned distance against
+    float64, in units of eps (xx + cc), for the engine's transform and for the oracle's."""
+    rng = np.random.default_rng(d + k)
+    X = (rng.standard_normal((n, d)) * 3 + rng.integers(0, 20, (n, 1))).astype(np.float32)
+    C = np.ascontiguousarray(X[rng.choice(n, size=k, replace=False)] + rng.standard_normal((k, d)).astype(np.float32))
+    m = 4000
+    with hip.Handle(n, d, k, np.float32) as h:
+        h.set_data(X)
+        h.set_option("assign", "mfma_tiled")
+        h.set_option("tiled_direct", direct)
+        h.set_centroids(C)
+        D = h.transform(X[:m]).T.astype(np.float64)           # [m][k]
+        h.set_option("exact_argmin", 1)
+        h.assign()
+        L, md = h.labels()[:m], h.min_distances()[:m].astype(np.float64)
+    wD = oracle.distances(np.ascontiguousarray(X[:m]), C, threads=4).T.astype(np.float64)
+    X64, C64 = X[:m].astype(np.float64), C.astype(np.float64)
+    xx, cc = (X64 * X64).sum(1)[:, None], (C64 * C64).sum(1)[None, :]
+    truth = np.abs(xx + cc - 2.0 * X64 @ C64.T)
+    unit = float(np.finfo(np.float32).eps) * (xx + cc)
+    e_engine, e_oracle = (D - truth) / unit, (wD - truth) / unit
+    rms_e, rms_o = np.sqrt((e_engine ** 2).mean()), np.sqrt((e_oracle ** 2).mean())
+    print("d=%d k=%d direct=%d: engine rms %.2f max %.1f, oracle rms %.2f max %.1f" % (
+        d, k, direct, rms_e, np.abs(e_engine).max(), rms_o, np.abs(e_oracle).max()))
+    assert abs(e_engine.mean()) <= 0.2
+    assert rms_e <= 1.25 * rms_o + 0.1, (rms_e, rms_o)
+    # the assignment pass returns the same numbers as the transform for the rows' own minima
+    e_min = (md - truth[np.arange(m), L]) / unit[np.arange(m), L]
+    assert np.sqrt((e_min ** 2).mean()) <= 1.25 * rms_o + 0.1
