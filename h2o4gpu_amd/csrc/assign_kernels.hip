@@ -1122,10 +1122,10 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
   // LATE: the accumulators start at zero and -(xx + cc)/2 is added when a block is complete, as
   // in assign_tiled_dma_kernel and for its reason (the partial sums of the dot product are then
   // rounded at their own size: 1.5 times less rounding noise in the minimum distance at 256
-  // features), wherever the distances themselves are compared or returned in float32; the
-  // 16-ulp keys (rows of fewer than 128 features) and float64 keep the start value, which
-  // saves them an instruction per distance. The block's norms wait in LDS for the epilogue.
-  constexpr bool LATE = sizeof(T) == 4 && (MODE == 1 || EXACT);
+  // features) in float32; float64, whose rounding noise is nine orders of magnitude below the
+  // near-tie allowance, keeps the start value, which saves it an instruction per distance.
+  // The block's norms wait in LDS for the epilogue.
+  constexpr bool LATE = sizeof(T) == 4;
   T *cns = reinterpret_cast<T *>(smem_raw + Cfg::OPERAND_BYTES);  // [2][BC]
   static_assert(BC <= WG, "one thread per centroid of a block fetches its norm");
 
@@ -1442,12 +1442,17 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
       // or block replaces the running key only from a lower bucket)
 #pragma unroll
       for (int ct = 0; ct < CT; ct++) {
+        T ccv[NACC];
+#pragma unroll
+        for (int v = 0; v < NACC; v++) ccv[v] = LATE ? cn[(wc * CT + ct) * MT + M::acc_row(v, g)] : (T)0;
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
           unsigned key[NACC];
 #pragma unroll
-          for (int v = 0; v < NACC; v++)
-            key[v] = (__float_as_uint(acc[ct][rt][v]) & 0x7FFFFFF0u) | (unsigned)v;
+          for (int v = 0; v < NACC; v++) {
+            const float a = LATE ? (float)(acc[ct][rt][v] + fma((T)-0.5, ccv[v], xx[rt])) : (float)acc[ct][rt][v];
+            key[v] = (__float_as_uint(a) & 0x7FFFFFF0u) | (unsigned)v;
+          }
           unsigned m = umin3(key[0], key[1], key[2]);
 #pragma unroll
           for (int v = 3; v + 1 < NACC; v += 2) m = umin3(m, key[v], key[v + 1]);
