@@ -2,7 +2,7 @@
 (tests/test_gpu_configs.py, tests/test_gpu_entry_points_full_size.py) into the markdown tables of
 the parity summary. Numbers only; nothing here touches a GPU.
 
-    python tests/parity_report_table.py gpurun_out/parity_report.jsonl
+    python tests/parity_report_table.py parity_report.jsonl
 """
 import json
 import sys
@@ -81,4 +81,6 @@ def main(path):
 
 
 if __name__ == "__main__":
-    main(sys.argv[1] if len(sys.argv) > 1 else "gpurun_out/parity_report.jsonl")
+    if len(sys.argv) != 2:
+        sys.exit("usage: python tests/parity_report_table.py <file the tests wrote to $H2O4GPU_PARITY_REPORT>")
+    main(sys.argv[1])
