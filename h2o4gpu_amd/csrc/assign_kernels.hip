@@ -1119,13 +1119,12 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
   constexpr int NSB = SPLIT ? NV / 2 : 1;  // 16-feature steps per stage
   constexpr int A_BYTES = BC * BK * 6, B_BYTES = BR * BK * 6;
   unsigned char *Ab = smem_raw, *Bb = smem_raw + 2 * A_BYTES;
-  // LATE: the accumulators start at zero and -(xx + cc)/2 is added when a block is complete, as
-  // in assign_tiled_dma_kernel and for its reason (the partial sums of the dot product are then
+  // The accumulators start at zero and -(xx + cc)/2 is added when a block is complete, as in
+  // assign_tiled_dma_kernel and for its reason (the partial sums of the dot product are then
   // rounded at their own size: 1.5 times less rounding noise in the minimum distance at 256
-  // features) in float32; float64, whose rounding noise is nine orders of magnitude below the
-  // near-tie allowance, keeps the start value, which saves it an instruction per distance.
-  // The block's norms wait in LDS for the epilogue.
-  constexpr bool LATE = sizeof(T) == 4;
+  // float32 features); the two kernels add the same products in the same order and close a
+  // block with the same expression, so a shape gives the same bits through either, whatever
+  // its alignment or the tiled_direct option. The block's norms wait in LDS for the epilogue.
   T *cns = reinterpret_cast<T *>(smem_raw + Cfg::OPERAND_BYTES);  // [2][BC]
   static_assert(BC <= WG, "one thread per centroid of a block fetches its norm");
 
@@ -1211,8 +1210,8 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
   // matrix cores add +x.c with the centroids staged as they are, which spares the staging of
   // every tile a multiplication by -2. Halving and doubling are exact, so every accumulator
   // is bit for bit -1/2 of (xx + cc) - 2 x.c accumulated in the same order; the comparisons
-  // are unaffected and the distance that leaves the kernel is 2 |acc|. (LATE: they start at
-  // zero and -(xx + cc)/2 joins them in the epilogue.)
+  // are unaffected and the distance that leaves the kernel is 2 |acc|. (They start at zero
+  // and -(xx + cc)/2 joins them in the epilogue.)
   T xx[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; rt++)
@@ -1320,21 +1319,17 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
   const int c_end = MODE == 1 ? min(k, c_begin + BC) : k;
   for (int c0 = c_begin; c0 < c_end; c0 += BC) {
     acc_t acc[CT][RT];
-    // (LATE) the copy of the norms this block's epilogue reads; the other copy may still be
+    // the copy of the norms this block's epilogue reads; the other copy may still be
     // read by wavefronts in the epilogue of the block before. Visible to everybody after the
     // barriers below.
     const T *cn = cns + (((c0 - c_begin) / BC) & 1) * BC;
-    (void)cn;
-    if constexpr (LATE) {
-      if (tid < BC) cns[(((c0 - c_begin) / BC) & 1) * BC + tid] = cnorm[c0 + tid];
-    }
+    if (tid < BC) cns[(((c0 - c_begin) / BC) & 1) * BC + tid] = cnorm[c0 + tid];
 #pragma unroll
     for (int ct = 0; ct < CT; ct++) {
 #pragma unroll
-      for (int v = 0; v < NACC; v++) {
-        const T cc = LATE ? (T)0 : (T)-0.5 * cnorm[c0 + (wc * CT + ct) * MT + M::acc_row(v, g)];
+      for (int rt = 0; rt < RT; rt++) {
 #pragma unroll
-        for (int rt = 0; rt < RT; rt++) acc[ct][rt][v] = LATE ? (T)0 : xx[rt] + cc;
+        for (int v = 0; v < NACC; v++) acc[ct][rt][v] = (T)0;
       }
     }
     if (DTAIL && nstage == 1) gload(c0, 0, std::true_type{});
@@ -1428,11 +1423,11 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
 #pragma unroll
         for (int v = 0; v < NACC; v++) {
           const int c = c0 + (wc * CT + ct) * MT + M::acc_row(v, g);
-          const T cc = LATE ? cn[c - c0] : (T)0;
+          const T cc = cn[c - c0];
 #pragma unroll
           for (int rt = 0; rt < RT; rt++) {
             const int64_t row = row0 + (wr * RT + rt) * MT + r;
-            const T a = LATE ? acc[ct][rt][v] + fma((T)-0.5, cc, xx[rt]) : acc[ct][rt][v];
+            const T a = acc[ct][rt][v] + fma((T)-0.5, cc, xx[rt]);
             if (c < k && row < n) D[(size_t)c * ldn + row] = (T)2 * fabs(a);
           }
         }
@@ -1444,13 +1439,13 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
       for (int ct = 0; ct < CT; ct++) {
         T ccv[NACC];
 #pragma unroll
-        for (int v = 0; v < NACC; v++) ccv[v] = LATE ? cn[(wc * CT + ct) * MT + M::acc_row(v, g)] : (T)0;
+        for (int v = 0; v < NACC; v++) ccv[v] = cn[(wc * CT + ct) * MT + M::acc_row(v, g)];
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
           unsigned key[NACC];
 #pragma unroll
           for (int v = 0; v < NACC; v++) {
-            const float a = LATE ? (float)(acc[ct][rt][v] + fma((T)-0.5, ccv[v], xx[rt])) : (float)acc[ct][rt][v];
+            const float a = (float)(acc[ct][rt][v] + fma((T)-0.5, ccv[v], xx[rt]));
             key[v] = (__float_as_uint(a) & 0x7FFFFFF0u) | (unsigned)v;
           }
           unsigned m = umin3(key[0], key[1], key[2]);
@@ -1476,10 +1471,10 @@ __global__ __launch_bounds__(2 * BCW * 64, BCW == 4 ? 1 : 2) void assign_tiled_k
       for (int ct = 0; ct < CT; ct++) {
 #pragma unroll
         for (int v = 0; v < NACC; v++) {
-          const T cc = LATE ? cn[(wc * CT + ct) * MT + M::acc_row(v, g)] : (T)0;
+          const T cc = cn[(wc * CT + ct) * MT + M::acc_row(v, g)];
 #pragma unroll
           for (int rt = 0; rt < RT; rt++) {
-            const T a = LATE ? acc[ct][rt][v] + fma((T)-0.5, cc, xx[rt]) : acc[ct][rt][v];
+            const T a = acc[ct][rt][v] + fma((T)-0.5, cc, xx[rt]);
             if (fabs(a) < fabs(best[rt])) {
               best[rt] = a;
               loc[rt] = ct * NACC + v;
