@@ -89,15 +89,29 @@ def measure_traffic(argv_tail, timeout_s=240):
     return total, details
 
 
+def load_workload(args, dtype):
+    """Rows, k, seed and the benchmark's iteration count of the workload the arguments name: one of
+    the five configurations, or (--shape) unit-variance noise of any shape, drawn once as a block of
+    16M values and repeated (a sweep over shapes should not wait for a generator)."""
+    if args.shape:
+        n, d, k = (int(v) for v in args.shape.lower().split("x"))
+        base = np.random.default_rng(1).standard_normal(1 << 24).astype(np.float32)
+        reps = -(-(n * d) // base.size)
+        X = np.ascontiguousarray(np.tile(base, reps)[:n * d].reshape(n, d).astype(dtype))
+        return X, k, 1, 5
+    X, k, _ = datasets.make(args.workload, args.scale, dtype)
+    return X, k, datasets.SHAPES[args.workload][3], datasets.SHAPES[args.workload][4]
+
+
 def traffic_child(args):
     """The run the counters are read from: a few Lloyd steps of the workload plus the copy
     kernel that calibrates the counter."""
     dtype = np.float32 if args.dtype == "f32" else np.float64
-    X, k, _ = datasets.make(args.workload, args.scale, dtype)
+    X, k, seed, _ = load_workload(args, dtype)
     n, d = X.shape
     h = kmeans_hip.Handle(n, d, k, dtype)
     h.set_data(X)
-    h.set_centroids(datasets.seeded_row_init(X, k, datasets.SHAPES[args.workload][3]))
+    h.set_centroids(datasets.seeded_row_init(X, k, seed))
     h.set_option("assign", args.assign)
     if args.no_fuse:
         h.set_option("fuse", 0)
@@ -272,6 +286,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="C3", choices=sorted(datasets.SHAPES))
     ap.add_argument("--scale", type=float, default=1.0, help="row-count scale (1.0 = full shape)")
+    ap.add_argument("--shape", default=None, metavar="ROWSxCOLSxK",
+                    help="instead of a configuration: unit-variance noise of this shape, seeded-random row start "
+                         "(for sweeps over shapes; the bench line then names the shape as its workload)")
     ap.add_argument("--dtype", default="f32", choices=["f32", "f64"])
     ap.add_argument("--assign", default="auto", choices=sorted(kmeans_hip.ASSIGN_VARIANTS))
     ap.add_argument("--exact-argmin", action="store_true",
@@ -314,7 +331,8 @@ def main():
     traffic, traffic_details = None, {"skipped": "--no-traffic"}
     if not args.no_traffic:
         tail = ["--workload", args.workload, "--scale", str(args.scale), "--dtype", args.dtype,
-                "--assign", args.assign] + (["--no-fuse"] if args.no_fuse else []) + \
+                "--assign", args.assign] + (["--shape", args.shape] if args.shape else []) + \
+               (["--no-fuse"] if args.no_fuse else []) + \
                (["--exact-argmin"] if args.exact_argmin else []) + \
                (["--fp32-split", str(args.fp32_split)] if args.fp32_split is not None else [])
         t0 = time.perf_counter()
@@ -327,17 +345,16 @@ def main():
 
     dtype = np.float32 if args.dtype == "f32" else np.float64
     t0 = time.perf_counter()
-    X, k, _ = datasets.make(args.workload, args.scale, dtype)
+    X, k, seed, fit_iters = load_workload(args, dtype)
     n, d = X.shape
-    seed = datasets.SHAPES[args.workload][3]
     if args.operands != "generator":
         if args.operands == "normal":
             X = np.random.default_rng(seed).standard_normal(X.shape, dtype=dtype)
         else:
             X = np.full(X.shape, 0.0 if args.operands == "zeros" else 1.0, dtype)
     C0 = datasets.seeded_row_init(X, k, seed)
-    log("generated %s: %d x %d %s, k=%d in %.1f s" % (args.workload, n, d, X.dtype, k,
-                                                    time.perf_counter() - t0))
+    wname = "noise %s" % args.shape if args.shape else args.workload
+    log("generated %s: %d x %d %s, k=%d in %.1f s" % (wname, n, d, X.dtype, k, time.perf_counter() - t0))
     s = X.dtype.itemsize
     flops_per_iter = 2.0 * n * k * d
     bytes_per_iter = float(n) * d * s + 4.0 * n + 2.0 * k * d * s
@@ -349,7 +366,7 @@ def main():
     t0 = time.perf_counter()
     h.set_data(X)
     h2d_s = time.perf_counter() - t0
-    if args.workload == "C4" and args.operands == "generator":  # the benchmark text starts this shape from k-means++
+    if args.workload == "C4" and args.operands == "generator" and not args.shape:  # the benchmark text starts this shape from k-means++
         h.init_plusplus(seed)
         C0 = h.centroids()
     h.set_centroids(C0)
@@ -461,7 +478,9 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic",
         "config": {"workload": "%s: %d x %d %s, k=%d, %s; one step = assign + centroid update"
-                               % (args.workload, n, d, args.dtype, k, WORKLOAD_TEXT[args.workload]),
+                               % (wname, n, d, args.dtype, k,
+                                  "unit-variance noise, seeded-random row start" if args.shape
+                                  else WORKLOAD_TEXT[args.workload]),
                    "rows": n, "cols": d, "k": k, "assign_variant": variant,
                    "operands": args.operands},
         "roofline": roofline,
@@ -481,7 +500,7 @@ def main():
         out["transform"] = transform
     if split_leg:
         out["fp32_split"] = split_leg
-    if args.extras and args.workload == "C3" and args.scale == 1.0 and args.dtype == "f32":
+    if args.extras and args.workload == "C3" and args.scale == 1.0 and args.dtype == "f32" and not args.shape:
         # the north star's two regimes under the same clock as the headline shape; extras, never
         # the reason a bench line is missing
         for key, wl, scale in (("c4_distance_step", "C4", 1.0), ("hbm_bound_step", "C1", 100.0)):
@@ -501,7 +520,7 @@ def main():
         out["cpu_baseline"] = cpu_baseline(X, C0, args.cpu_iters)
         out["cpu_reference_path"] = sklearn_baseline(X, C0, args.sklearn_rows)
     if args.end_to_end:
-        out["c_abi_fit"] = c_abi_fit(X, C0, datasets.SHAPES[args.workload][4])
+        out["c_abi_fit"] = c_abi_fit(X, C0, fit_iters)
         try:
             out["kmeans_parallel_seeding"] = seeding_seconds(X, k)
         except Exception as e:  # an extra: never the reason a bench line is missing
