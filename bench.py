@@ -75,7 +75,7 @@ def measure_traffic(argv_tail, timeout_s=240):
             shutil.rmtree(tmp, ignore_errors=True)
         copy = [v for name, v in per_kernel.items() if "copy_probe_kernel" in name]
         step = [(len(v), name, v) for name, v in per_kernel.items()
-                if ("assign_" in name or "lloyd_valu" in name)]
+                if ("assign_" in name or "lloyd_valu" in name or "lloyd_longrow" in name)]
         if not copy or not step:
             return None, {"skipped": "%s pass: kernels not found" % counter}
         # the Lloyd-step kernel is the assign/step kernel with the most dispatches
@@ -405,7 +405,7 @@ def main():
     assign_ms = kern[dom]["avg_ms"]
     tflops = flops_per_iter / (assign_ms * 1e-3) / 1e12
     peak = PEAK_MFMA_TFLOPS[args.dtype]
-    mfma_bound = variant != "valu"
+    mfma_bound = variant not in ("valu", "wave_row")   # (the kernels without matrix instructions stream X)
     if mfma_bound and "_bf16x" in variant:
         # the option that forms each float32 product from bfloat16 parts: the kernel executes
         # 6 or 9 times the algorithmic flop, on the bfloat16 matrix pipe, and is priced there
@@ -421,7 +421,7 @@ def main():
         # per row: the row read, the label written (inside a fit loop the fused step neither reads
         # the stored row norms nor writes the minimum distances)
         gbps = float(n) * (d * s + 4) / (assign_ms * 1e-3) / 1e9
-        roofline = {"bound": "hbm", "kernel": "%s (valu)" % dom, "achieved": gbps,
+        roofline = {"bound": "hbm", "kernel": "%s (%s)" % (dom, variant), "achieved": gbps,
                     "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": gbps / PEAK_HBM_GBPS,
                     "traffic": traffic}
     iter_gbps = bytes_per_iter / (ms_step * 1e-3) / 1e9

@@ -7,7 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libh2o4gpu_kmeans_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ["engine.hip", "assign_kernels.hip", "update_kernels.hip", "seed_kernels.hip"]
+SOURCES = ["engine.hip", "assign_kernels.hip", "longrow_kernels.hip", "update_kernels.hip", "seed_kernels.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",

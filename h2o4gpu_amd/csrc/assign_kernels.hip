@@ -1921,6 +1921,7 @@ const char *assign_variant_name(int variant) {
     case ASSIGN_VALU: return "valu";
     case ASSIGN_ROWSTAT: return "mfma_rowstat";
     case ASSIGN_TILED: return "mfma_tiled";
+    case ASSIGN_LONGROW: return "wave_row";
     default: return "auto";
   }
 }
@@ -1961,6 +1962,7 @@ int pick_assign_variant(int requested, int64_t n, int d, int k) {
   // any model can be swept in LDS-sized chunks of centroids (one launch per chunk)
   if (requested == ASSIGN_ROWSTAT) return dp != 0 ? ASSIGN_ROWSTAT : -1;
   if (requested == ASSIGN_VALU || requested == ASSIGN_TILED) return requested;
+  if (requested == ASSIGN_LONGROW) return longrow_applies<T>(d, k) ? ASSIGN_LONGROW : -1;
   // the reference switches to its hand-written small kernel at k<=16 && d<=64
   // (kmeans_labels.cu:140,207); same boundary here
   if (k <= 16 && d <= 64) return ASSIGN_VALU;
@@ -1971,6 +1973,14 @@ int pick_assign_variant(int requested, int64_t n, int d, int k) {
   // register slice exactly (measured, chunked vs tiled: 2M x 128 f32 k=2048 0.83 vs 0.78 of
   // peak, 4M x 64 f64 k=2048 0.78 vs 0.68; with d = 96 padded to 128 it is 0.58 vs 0.71).
   if (dp != 0 && (dp * (int)sizeof(T) <= 256 || d == dp)) return ASSIGN_ROWSTAT;
+  // Long rows and a handful of centroids: the tiled kernel would pad the model to 64 centroids
+  // and need a second pass over the rows for the sums; one wavefront along the features of
+  // four rows reads them once.
+  // (float64 from 256 features on: its exchanges between lanes cost twice the float32 ones, and
+  // below that the two passes are as fast or faster: 1M x 192, k = 16: 0.87 against 0.85 ms,
+  // 500k x 256, k = 8: 0.40 against 0.64 ms; float32 from the first shape the row-stationary kernel
+  // does not take: 1M x 132, k = 8: 0.33 against 0.37 ms, 500k x 784, k = 10: 0.52 against 0.86 ms)
+  if (longrow_applies<T>(d, k) && (sizeof(T) == 4 || d >= 256)) return ASSIGN_LONGROW;
   return ASSIGN_TILED;
 }
 
@@ -2218,6 +2228,7 @@ template <typename T>
 int fused_slots(int requested_variant, int64_t n, int d, int k, int num_cu) {
   const int v = pick_assign_variant<T>(requested_variant, n, d, k);
   if (v == ASSIGN_VALU && valu_fused_applies(d, k)) return 8 * num_cu;
+  if (v == ASSIGN_LONGROW) return longrow_max_slots<T>(d, k, num_cu);
   if (v != ASSIGN_ROWSTAT) return 0;
   const size_t lds = rowstat_fused_lds<T>(d, k);
   if (lds > ROWSTAT_FUSED_LDS_MAX) return 0;
@@ -2299,6 +2310,9 @@ int launch_assign_accumulate(hipStream_t s, int variant, const T *X, const T *xn
   if (v == ASSIGN_VALU && valu_fused_applies(d, k))
     return launch_valu_fused<T, true>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu,
                                       psums, pcounts, slots);
+  if (v == ASSIGN_LONGROW)
+    return launch_longrow<T, true>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu, psums, pcounts,
+                                   slots);
   if (v != ASSIGN_ROWSTAT) return H2O4GPU_KMEANS_EARG;
   return RowstatDispatch<T, true>::run(s, X, xnorm, C, cnorm, labels, mindist, n, d, k,
                                        num_cu, psums, pcounts, slots, 0, 0, false, st, split);
@@ -2531,6 +2545,9 @@ int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
     case ASSIGN_TILED:
       return launch_tiled<T, 0>(s, X, xnorm, C, cnorm, labels, mindist, nullptr, n, n, d, k, exact, split,
                                 split_scratch);
+    case ASSIGN_LONGROW:
+      return launch_longrow<T, false>(s, X, xnorm, C, cnorm, labels, mindist, n, d, k, num_cu, nullptr,
+                                      nullptr, nullptr);
   }
   return H2O4GPU_KMEANS_EARG;
 }

@@ -701,6 +701,8 @@ struct Engine : h2o4gpu_kmeans_handle {
     int slots = plan.row_blocks;
     const int fs = fused_slots<T>(ASSIGN_AUTO, n, d, k, num_cu);
     if (fs > slots) slots = fs;
+    // (a shape the long-row kernel takes only when asked to writes more slots than the default kernel's)
+    if (sets == 1 && longrow_applies<T>(d, k)) slots = std::max(slots, longrow_max_slots<T>(d, k, num_cu));
     KM_TRY(dalloc(&psums, (size_t)slots * kd));
     KM_TRY(dalloc(&pcounts, (size_t)slots * k));
     use_buckets = bucketed_update_applies(plan.k_chunks, k, d);
@@ -1237,8 +1239,8 @@ struct Engine : h2o4gpu_kmeans_handle {
   // assignment pass will, before anyone reads them): one store per row less in the fused step.
   int step_async(bool want_shift, bool want_mindist = true) {
     // (the exact-compare argmin exists in the assignment-only kernels)
-    const bool exact_mfma = opt_exact && sizeof(T) == 4 &&
-                            pick_assign_variant<T>(opt_assign, n, d, k) != ASSIGN_VALU;
+    const int fam = pick_assign_variant<T>(opt_assign, n, d, k);
+    const bool exact_mfma = opt_exact && sizeof(T) == 4 && fam != ASSIGN_VALU && fam != ASSIGN_LONGROW;
     if ((opt_fuse || sets > 1) && !exact_mfma && fused_slots<T>(opt_assign, n, d, k, num_cu) > 0) {
       int slots = 0;
       PROFILED("assign_accumulate",
@@ -2208,7 +2210,7 @@ KM_API int h2o4gpu_kmeans_set_option(h2o4gpu_kmeans_handle *h, const char *name,
   KM_CHECK_HANDLE(h);
   if (!name) return H2O4GPU_KMEANS_EARG;
   if (strcmp(name, "assign") == 0) {
-    if (value < ASSIGN_AUTO || value > ASSIGN_TILED) return H2O4GPU_KMEANS_EARG;
+    if (value < ASSIGN_AUTO || value > ASSIGN_LONGROW) return H2O4GPU_KMEANS_EARG;
     h->opt_assign = value;
     return 0;
   }

@@ -59,7 +59,8 @@ enum AssignVariant {
   ASSIGN_AUTO = 0,
   ASSIGN_VALU = 1,     // one thread per row, centroids broadcast from LDS
   ASSIGN_ROWSTAT = 2,  // MFMA, row tile stationary in registers, all centroids in LDS
-  ASSIGN_TILED = 3     // MFMA, both operands staged through LDS over a d-loop
+  ASSIGN_TILED = 3,    // MFMA, both operands staged through LDS over a d-loop
+  ASSIGN_LONGROW = 4   // no MFMA: a wavefront along the features of four rows (k <= 16, rows beyond 64 features)
 };
 
 // Rows the centroid buffer C (zeros) and entries the norm buffer cnorm (+inf) must
@@ -102,6 +103,18 @@ int launch_assign(hipStream_t s, int variant, const T *X, const T *xnorm,
                   StackShape st = StackShape(), int split = 0, SplitScratch split_scratch = SplitScratch());
 template <typename T>
 int pick_assign_variant(int requested, int64_t n, int d, int k);
+// The one-pass kernel for long rows and at most 16 centroids (longrow_kernels.hip): whether a
+// shape is its (rows of whole 16-byte vectors, centroids and double-precision sums within one
+// CU's LDS), the largest number of partial-sum slots its fused form writes, and the launch
+// (SUMS false: labels and minimum distances only; cnorm may be null as for the fused kernels).
+template <typename T>
+bool longrow_applies(int d, int k);
+template <typename T>
+int longrow_max_slots(int d, int k, int num_cu);
+template <typename T, bool SUMS>
+int launch_longrow(hipStream_t s, const T *X, const T *xnorm, const T *C, const T *cnorm, int *labels,
+                   T *mindist, int64_t n, int d, int k, int num_cu, double *psums, int *pcounts,
+                   int *slots);
 const char *assign_variant_name(int variant);
 // split (float32 matrix-core kernels; 0, 6 or 9): run the dot products on the bfloat16
 // matrix pipe as that many products of bfloat16 parts per feature pair (9: every product

@@ -140,7 +140,7 @@ def stack_width(rows, cols, k, dtype, max_sets):
                                                 int(max_sets)))
 
 
-ASSIGN_VARIANTS = {"auto": 0, "valu": 1, "mfma_rowstat": 2, "mfma_tiled": 3}
+ASSIGN_VARIANTS = {"auto": 0, "valu": 1, "mfma_rowstat": 2, "mfma_tiled": 3, "wave_row": 4}
 
 
 class Handle:

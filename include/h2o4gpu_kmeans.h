@@ -226,7 +226,9 @@ int h2o4gpu_kmeans_transform_host(h2o4gpu_kmeans_handle *h, size_t rows,
 int h2o4gpu_kmeans_transform_resident(h2o4gpu_kmeans_handle *h, void *d_dist);
 
 /* Kernel selection: "assign" = 0 auto, 1 VALU, 2 MFMA row-stationary,
- * 3 MFMA tiled; "fuse" = 1 (default) lets fit/iterate run assignment and the
+ * 3 MFMA tiled, 4 the one-pass kernel for rows beyond 64 features and at most 16
+ * centroids (a wavefront along the features of four rows; a shape outside its range
+ * reports "unsupported"); "fuse" = 1 (default) lets fit/iterate run assignment and the
  * per-centroid accumulation as one kernel where the shape allows, 0 keeps them
  * separate; "buckets" = 1 (default) sums the centroids of shapes whose sums do not
  * fit LDS by bucketing rows by label, 0 uses the chunked LDS kernel for them too;
