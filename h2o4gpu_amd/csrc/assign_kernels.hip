@@ -1966,6 +1966,10 @@ int pick_assign_variant(int requested, int64_t n, int d, int k) {
   // the reference switches to its hand-written small kernel at k<=16 && d<=64
   // (kmeans_labels.cu:140,207); same boundary here
   if (k <= 16 && d <= 64) return ASSIGN_VALU;
+  // Up to four centroids and rows beyond 64 features: the one-pass kernel of longrow_kernels.hip is
+  // ahead of the matrix-core kernels on every such shape (2M x 128, k = 4: 0.34 against 0.62 ms per
+  // step, 2M x 72: 0.32 against 0.37; float64 1M x 128: 0.26 against 0.52, 1M x 200: 0.33 against 0.86).
+  if (k <= 4 && longrow_applies<T>(d, k)) return ASSIGN_LONGROW;
   if (rowstat_ok) return ASSIGN_ROWSTAT;
   // Short rows with a large model: the tiled kernel's d-loop has one or two stages and
   // cannot hide its loads; chunked row-stationary sweeps re-read X once per chunk, which
@@ -1976,8 +1980,8 @@ int pick_assign_variant(int requested, int64_t n, int d, int k) {
   // Long rows and a handful of centroids: the tiled kernel would pad the model to 64 centroids
   // and need a second pass over the rows for the sums; one wavefront along the features of
   // four rows reads them once.
-  // (float64 from 256 features on: its exchanges between lanes cost twice the float32 ones, and
-  // below that the two passes are as fast or faster: 1M x 192, k = 16: 0.87 against 0.85 ms,
+  // (5 to 16 centroids in float64 from 256 features on: its exchanges between lanes cost twice the
+  // float32 ones, and below that the two passes are as fast or faster: 1M x 192, k = 16: 0.87 against 0.85 ms,
   // 500k x 256, k = 8: 0.40 against 0.64 ms; float32 from the first shape the row-stationary kernel
   // does not take: 1M x 132, k = 8: 0.33 against 0.37 ms, 500k x 784, k = 10: 0.52 against 0.86 ms)
   if (longrow_applies<T>(d, k) && (sizeof(T) == 4 || d >= 256)) return ASSIGN_LONGROW;

@@ -43,7 +43,7 @@ def test_assign_and_fused_step_against_the_oracle(hip, oracle, n, d, k, dtype):
     with hip.Handle(n, d, k, dtype) as h:
         h.set_data(X)
         h.set_centroids(C)
-        h.set_option("assign", "wave_row")             # (the default beyond 128 float32 / from 256 float64 features)
+        h.set_option("assign", "wave_row")   # (the default for up to 4 centroids, and beyond 128 float32 / from 256 float64 features)
         assert h.assign_variant() == "wave_row"
         h.assign()
         L, m = h.labels(), h.min_distances()
@@ -134,6 +134,7 @@ def test_which_shapes_take_it_by_default(hip):
                                  (2000, 1028, 8, np.float32, "mfma_tiled"), (2000, 786, 8, np.float32, "mfma_tiled"),
                                  (2000, 96, 8, np.float32, "mfma_rowstat"), (2000, 96, 8, np.float64, "mfma_tiled"), (2000, 256, 8, np.float64, "wave_row"),
                                  (2000, 784, 10, np.float32, "wave_row"), (2000, 256, 16, np.float32, "wave_row"),
-                                 (2000, 516, 4, np.float64, "mfma_tiled")]:
+                                 (2000, 516, 4, np.float64, "mfma_tiled"), (2000, 96, 4, np.float32, "wave_row"),
+                                 (2000, 96, 5, np.float32, "mfma_rowstat"), (2000, 72, 2, np.float64, "wave_row")]:
         with hip.Handle(n, d, k, dtype) as h:
             assert h.assign_variant() == want, (n, d, k, h.assign_variant())
