@@ -1980,11 +1980,12 @@ int pick_assign_variant(int requested, int64_t n, int d, int k) {
   // Long rows and a handful of centroids: the tiled kernel would pad the model to 64 centroids
   // and need a second pass over the rows for the sums; one wavefront along the features of
   // four rows reads them once.
-  // (5 to 16 centroids in float64 from 256 features on: its exchanges between lanes cost twice the
-  // float32 ones, and below that the two passes are as fast or faster: 1M x 192, k = 16: 0.87 against 0.85 ms,
-  // 500k x 256, k = 8: 0.40 against 0.64 ms; float32 from the first shape the row-stationary kernel
-  // does not take: 1M x 132, k = 8: 0.33 against 0.37 ms, 500k x 784, k = 10: 0.52 against 0.86 ms)
-  if (longrow_applies<T>(d, k) && (sizeof(T) == 4 || d >= 256)) return ASSIGN_LONGROW;
+  // (float64, whose exchanges between lanes cost twice the float32 ones: 5 to 8 centroids from 96
+  // features on, 1M x 96, k = 8: 0.33 against 0.40 ms, 1M x 128: 0.35 against 0.52; 9 to 16 from 224 on,
+  // 1M x 128, k = 16: 0.66 against 0.53, 1M x 192: 0.86 against 0.85, 1M x 252, k = 12: 0.82 against 1.03,
+  // 500k x 256, k = 8: 0.30 against 0.64; float32 from the first shape the row-stationary kernel does
+  // not take: 1M x 132, k = 8: 0.27 against 0.37 ms, 500k x 784, k = 10: 0.51 against 0.86 ms)
+  if (longrow_applies<T>(d, k) && (sizeof(T) == 4 || d >= (k <= 8 ? 96 : 224))) return ASSIGN_LONGROW;
   return ASSIGN_TILED;
 }
 

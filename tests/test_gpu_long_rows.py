@@ -132,7 +132,8 @@ def test_duplicate_centroids_lowest_index_wins(hip):
 def test_which_shapes_take_it_by_default(hip):
     for n, d, k, dtype, want in [(2000, 64, 8, np.float32, "valu"), (2000, 784, 17, np.float32, "mfma_tiled"),
                                  (2000, 1028, 8, np.float32, "mfma_tiled"), (2000, 786, 8, np.float32, "mfma_tiled"),
-                                 (2000, 96, 8, np.float32, "mfma_rowstat"), (2000, 96, 8, np.float64, "mfma_tiled"), (2000, 256, 8, np.float64, "wave_row"),
+                                 (2000, 96, 8, np.float32, "mfma_rowstat"), (2000, 96, 8, np.float64, "wave_row"), (2000, 92, 8, np.float64, "mfma_tiled"),
+                                 (2000, 200, 12, np.float64, "mfma_tiled"), (2000, 256, 12, np.float64, "wave_row"),
                                  (2000, 784, 10, np.float32, "wave_row"), (2000, 256, 16, np.float32, "wave_row"),
                                  (2000, 516, 4, np.float64, "mfma_tiled"), (2000, 96, 4, np.float32, "wave_row"),
                                  (2000, 96, 5, np.float32, "mfma_rowstat"), (2000, 72, 2, np.float64, "wave_row")]:
